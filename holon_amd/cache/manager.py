@@ -1,0 +1,217 @@
+"""The cache manager: slots, paged groups with block tables, and fixed-size per-request state.
+
+A request is given a *slot* when it is admitted: its row in every block table and in every fixed-size state tensor.
+State that grows lives in pages. Runs of the model whose mixers declare equal `PagedState`s form a *group*: one page
+pool, one block table, one storage tensor `[sites, pages, page_size * elems]` — page id p means row p of every site of
+the group. Groups with different needs (all tokens, a window of them) have pools of their own; a windowed group gives
+pages back as soon as the window has passed them, a finished request gives back everything.
+
+core/holon/core/state.py:124-554 (`StateManager`: admit/reserve/release, `BlockTable`), core/holon/core/assembly.py:
+140-189 (grouping by declaration), std/holon_std/state/paged/kind.py:10-19 (pages needed).
+"""
+from __future__ import annotations
+
+import dataclasses
+
+import numpy as np
+import torch
+
+from ..parts.base import PagedState, SlotState
+from .pool import OutOfPages, PagePool
+
+
+@dataclasses.dataclass
+class PagedGroup:
+    gid: int
+    decl: PagedState                              # with name ignored: elems, window, dtype decide the group
+    sites: list[int]
+    pool: PagePool
+    storage: torch.Tensor                         # [len(sites), num_pages, page_size * elems]
+    table: np.ndarray                             # [max_seqs + 1, max_pages] int32, null page where nothing is held
+    table_dev: torch.Tensor
+    first: list[int]                              # per slot: first page index still held
+    count: list[int]                              # per slot: page indices [first, count) are held
+    dirty: set[int] = dataclasses.field(default_factory=set)
+
+
+class CacheManager:
+    """`sites`: the model's run entries (`holon_amd.model.Site`), filled here with their storage; `decls[i]`: what
+    run i keeps. `tokens`: capacity of every paged pool, in tokens."""
+
+    def __init__(self, sites: list, decls: list[list[PagedState | SlotState]], *, page_size: int, max_seqs: int,
+                 max_model_len: int, tokens: int, device: torch.device, dtype: torch.dtype) -> None:
+        self.page_size, self.max_seqs, self.max_model_len = page_size, max_seqs, max_model_len
+        self.device, self.dtype = device, dtype
+        self.max_pages = -(-max_model_len // page_size)
+        self.padding_slot = max_seqs                              # a row of null pages, for rows that compute nothing
+        self.groups: list[PagedGroup] = []
+        self.slot_states: list[tuple[int, SlotState, torch.Tensor]] = []
+        self._free_slots = list(range(max_seqs - 1, -1, -1))
+        self._live: set[int] = set()
+        self.computed = [0] * (max_seqs + 1)
+        num_pages = -(-tokens // page_size) + 1
+        if tokens < 1:
+            raise ValueError("the cache needs room for at least one token")
+        keyed: dict[tuple, list[int]] = {}
+        for site, site_decls in zip(sites, decls, strict=True):
+            for d in site_decls:
+                if isinstance(d, PagedState):
+                    if site.group is not None:
+                        raise NotImplementedError("one paged state per run")
+                    key = (d.elems, d.window, d.dtype or dtype)
+                    keyed.setdefault(key, []).append(site.run)
+                    site.group = -1
+                elif isinstance(d, SlotState):
+                    t = torch.zeros((max_seqs + 1, *d.shape), dtype=d.dtype or dtype, device=device)
+                    site.slot_state[d.name] = t
+                    self.slot_states.append((site.run, d, t))
+                else:
+                    raise TypeError(f"run {site.run}: unknown state declaration {d!r}")
+        for gid, ((elems, window, gdtype), runs) in enumerate(keyed.items()):
+            pool = PagePool(num_pages)
+            storage = torch.zeros((len(runs), num_pages, page_size * elems), dtype=gdtype, device=device)
+            table = np.full((max_seqs + 1, self.max_pages), pool.null, dtype=np.int32)
+            group = PagedGroup(gid, PagedState("", elems, window, gdtype), runs, pool, storage, table,
+                               torch.from_numpy(table.copy()).to(device), [0] * (max_seqs + 1), [0] * (max_seqs + 1))
+            self.groups.append(group)
+            for at, run in enumerate(runs):
+                sites[run].group, sites[run].pages = gid, storage[at]
+        for site in sites:                                        # runs that read another run's cache
+            if site.owner is not None:
+                owner = sites[site.owner]
+                site.group, site.pages, site.slot_state = owner.group, owner.pages, owner.slot_state
+
+    # -- slots ----------------------------------------------------------------------------------------------------
+    @property
+    def free_slots(self) -> int:
+        return len(self._free_slots)
+
+    def admit(self) -> int | None:
+        """A slot for a new request (its fixed-size state zeroed), or None when all are taken."""
+        if not self._free_slots:
+            return None
+        slot = self._free_slots.pop()
+        self._live.add(slot)
+        self.computed[slot] = 0
+        for _, _, t in self.slot_states:
+            t[slot].zero_()
+        return slot
+
+    def release(self, slot: int) -> None:
+        """Give back everything the request holds."""
+        if slot not in self._live:
+            raise RuntimeError(f"slot {slot} released twice (or never admitted)")
+        for g in self.groups:
+            for i in range(g.first[slot], g.count[slot]):
+                g.pool.decref(int(g.table[slot, i]))
+            g.table[slot, : g.count[slot]] = g.pool.null
+            g.first[slot] = g.count[slot] = 0
+            g.dirty.add(slot)
+        self._live.remove(slot)
+        self.computed[slot] = 0
+        self._free_slots.append(slot)
+
+    # -- pages ----------------------------------------------------------------------------------------------------
+    def pages_needed(self, slot: int, total: int) -> list[int]:
+        """Per group, the pages a request needs beyond what it holds to keep `total` tokens."""
+        want = -(-total // self.page_size)
+        return [max(0, want - g.count[slot]) for g in self.groups]
+
+    def reserve(self, slot: int, total: int) -> bool:
+        """Make room for the request's tokens 0 .. total-1 in every group, or take nothing and return False."""
+        if slot not in self._live:
+            raise RuntimeError(f"slot {slot} is not admitted")
+        if total > self.max_model_len:
+            raise ValueError(f"{total} tokens exceed max_model_len {self.max_model_len}")
+        need = self.pages_needed(slot, total)
+        if any(n > g.pool.free for n, g in zip(need, self.groups)):
+            return False
+        for n, g in zip(need, self.groups):
+            if n:
+                pages = g.pool.alloc(n)
+                g.table[slot, g.count[slot]: g.count[slot] + n] = pages
+                g.count[slot] += n
+                g.dirty.add(slot)
+        return True
+
+    def capacity(self, slot: int) -> int:
+        """Tokens the request's pages hold (the smallest over groups)."""
+        if not self.groups:
+            return self.max_model_len
+        return min(g.count[slot] for g in self.groups) * self.page_size
+
+    def advance(self, slot: int, computed: int) -> None:
+        """The request now has `computed` tokens in the cache: pages a window has passed are given back."""
+        self.computed[slot] = computed
+        for g in self.groups:
+            w = g.decl.window
+            if w <= 0:
+                continue
+            keep_from = max(0, computed - w + 1) // self.page_size      # the next query reads keys from computed-w+1
+            keep_from = min(keep_from, g.count[slot])
+            if keep_from > g.first[slot]:
+                for i in range(g.first[slot], keep_from):
+                    g.pool.decref(int(g.table[slot, i]))
+                g.table[slot, g.first[slot]: keep_from] = g.pool.null
+                g.first[slot] = keep_from
+                g.dirty.add(slot)
+
+    def could_fit(self, slot: int | None, total: int, victims: list[int]) -> bool:
+        """Whether releasing the requests in `victims` (slots) would let `slot` (None: a new request) keep `total`
+        tokens (core/holon/core/state.py:478-497)."""
+        want = -(-total // self.page_size)
+        for g in self.groups:
+            have = g.count[slot] if slot is not None else 0
+            freed = sum(g.count[v] - g.first[v] for v in victims)
+            if want - have > g.pool.free + freed:
+                return False
+        return True
+
+    def fits_alone(self, total: int) -> bool:
+        """Whether an empty cache holds one request of `total` tokens."""
+        return all(-(-total // self.page_size) <= g.pool.usable for g in self.groups)
+
+    # -- per-step views -------------------------------------------------------------------------------------------
+    def upload(self) -> None:
+        """Copy the block-table rows that changed to the device (core/holon/core/state.py:51-58)."""
+        for g in self.groups:
+            if g.dirty:
+                rows = sorted(g.dirty)
+                idx = torch.tensor(rows, dtype=torch.long, device=self.device)
+                g.table_dev.index_copy_(0, idx, torch.from_numpy(g.table[rows]).to(self.device))
+                g.dirty.clear()
+
+    def write_targets(self, gid: int, slots: np.ndarray, positions: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
+        """(page, offset) of each token's position in its request's pages (core/holon/core/state.py:541-554)."""
+        g = self.groups[gid]
+        return g.table[slots, positions // self.page_size].astype(np.int32), \
+            (positions % self.page_size).astype(np.int32)
+
+    # -- accounting -----------------------------------------------------------------------------------------------
+    def nbytes(self) -> int:
+        total = sum(g.storage.numel() * g.storage.element_size() for g in self.groups)
+        return total + sum(t.numel() * t.element_size() for _, _, t in self.slot_states)
+
+    def check(self) -> None:
+        """Every page is free or held exactly as often as its count says; no table points at a page it does not hold."""
+        for g in self.groups:
+            held: dict[int, int] = {}
+            for slot in range(self.max_seqs + 1):
+                row = g.table[slot]
+                inside = row[g.first[slot]: g.count[slot]]
+                outside = np.concatenate((row[: g.first[slot]], row[g.count[slot]:]))
+                if slot not in self._live and g.count[slot]:
+                    raise AssertionError(f"group {g.gid}: free slot {slot} holds pages")
+                if (outside != g.pool.null).any() or (inside == g.pool.null).any():
+                    raise AssertionError(f"group {g.gid}: slot {slot}'s table does not match what it holds")
+                for p in inside.tolist():
+                    held[p] = held.get(p, 0) + 1
+            free = set(g.pool._free)
+            if len(free) != len(g.pool._free):
+                raise AssertionError(f"group {g.gid}: a page is in the free list twice")
+            for p in range(g.pool.usable):
+                if held.get(p, 0) != g.pool.refs(p) or ((p in free) != (g.pool.refs(p) == 0)):
+                    raise AssertionError(f"group {g.gid}: page {p} held {held.get(p, 0)}x, count {g.pool.refs(p)}, "
+                                         f"free {p in free}")
+            if g.pool.free + len(held) != g.pool.usable:
+                raise AssertionError(f"group {g.gid}: {g.pool.usable - g.pool.free - len(held)} pages lost")

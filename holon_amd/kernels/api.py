@@ -1,0 +1,90 @@
+"""The kernel contract: every device operation the parts call, with shapes, dtypes and in-place rules.
+
+`holon_amd.kernels.hip.HipKernels` is the only implementation the product has (hand-written gfx950 HIP, loaded from
+the in-tree library; it fails loudly when the library is missing). A plain twin with the same methods lives under
+`tests/` and is handed to the engine only by tests. The shapes follow the reference's op contracts
+(std/holon_std/ops/kernels.py:1-45, std/holon_std/mixers/gqa/kernels.py:1-52), with this engine's cache layout.
+
+Conventions: T tokens in the step, B rows (requests in the step), Hq/Hkv heads, D head_dim, P page size. Activations
+and weights are `dtype` (bfloat16 or float32) unless stated; index tensors are int32. Norms, softmax, rotation angles
+and every sum are computed in float32 and rounded once to `dtype`.
+
+Cache layout of one page of one site, `pages[page]` = `[2, Hkv, P * D]`: keys as rows `[P, D]` (token-major),
+values as columns `[D, P]` (transposed inside the page, so that a matrix-core operand of the value product is one
+contiguous 16-byte load). Block table row `slot` lists the page of token positions `i*P .. i*P+P-1` at index i.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Protocol
+
+import torch
+
+
+@dataclasses.dataclass
+class AttnRows:
+    """The rows of a step, as attention sees them. Row b reads block table row `slots[b]`, holds `lens[b]` tokens
+    including this step's, and owns query tokens `query_start[b]:query_start[b+1]`, the last of its sequence
+    ("bottom-right causal": query i of the row sits at position lens[b] - n_query[b] + i). Rows with one query token
+    are listed in `decode_rows`, the others in `chunk_rows` (row indices, int32, device)."""
+
+    slots: torch.Tensor                  # [B] int32
+    lens: torch.Tensor                   # [B] int32
+    query_start: torch.Tensor            # [B+1] int32
+    decode_rows: torch.Tensor            # [n_decode] int32
+    chunk_rows: torch.Tensor             # [n_chunk] int32
+    n_decode: int
+    n_chunk: int
+    max_decode_len: int                  # host bounds for launch shapes
+    max_chunk_query: int
+    max_chunk_len: int
+
+
+class Kernels(Protocol):
+    name: str
+
+    def embedding(self, ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+        """ids [T] int32, table [V, H] -> [T, H] (rows of the table)."""
+
+    def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+        """x [..., dim] contiguous -> a new tensor; x is not modified."""
+
+    def add_rmsnorm(self, x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+        """residual += x in place (sum rounded to dtype), returns rmsnorm(residual) as a new tensor."""
+
+    def linear(self, x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        """x [T, K] @ weight [N, K].T -> [T, N], float32 accumulation, rounded to out_dtype (default: x's)."""
+
+    def silu_mul(self, gate_up: torch.Tensor) -> torch.Tensor:
+        """gate_up [T, 2I] (gate columns first) -> [T, I] = round(silu(gate)) * up."""
+
+    def rope(self, x: torch.Tensor, positions: torch.Tensor, table: torch.Tensor) -> None:
+        """Rotate the first table.shape[1] dims of x [T, heads, D] in place, half-split pairing; table
+        [max_positions, rotary_dim] float32 = cos of the rotary_dim/2 angles, then their sin."""
+
+    def kv_write(self, k: torch.Tensor, v: torch.Tensor, pages: torch.Tensor, write_page: torch.Tensor,
+                 write_off: torch.Tensor, page_size: int) -> None:
+        """k, v [T, Hkv, D] into the cache layout at (write_page[t], write_off[t])."""
+
+    def qk_norm_rope_write(self, qkv: torch.Tensor, heads: int, kv_heads: int, head_dim: int,
+                           q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float,
+                           table: torch.Tensor | None, positions: torch.Tensor, pages: torch.Tensor | None,
+                           write_page: torch.Tensor | None, write_off: torch.Tensor | None, page_size: int
+                           ) -> torch.Tensor:
+        """The fused form of per-head rmsnorm (if weights), rope (if table) and kv_write (if pages) on the merged
+        projection qkv [T, (Hq + 2 Hkv) D]: q and k heads are normed and rounded, rotated and rounded; k and v go to
+        the cache; returns q' [T, Hq, D], a new tensor. Same roundings as the three ops one after the other."""
+
+    def paged_attention(self, q: torch.Tensor, pages: torch.Tensor, table: torch.Tensor, rows: AttnRows,
+                        page_size: int, scale: float, window: int) -> torch.Tensor:
+        """softmax(q k^T * scale) v per row over its cached tokens, causal; with window W > 0 a query at position p
+        sees keys p-W+1 .. p. q [T, Hq, D] -> [T, Hq, D]. This step's keys are already in the cache."""
+
+    def argmax(self, logits: torch.Tensor) -> torch.Tensor:
+        """logits [R, V] float32 -> [R] int32, the first maximal index of each row."""
+
+    def sample(self, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+               min_p: torch.Tensor, seeds: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        """One token per row [R] int32. temperature/top_p/min_p float32 [R], top_k int32 [R], seeds int64 [R],
+        positions int64 [R] (the position of the token being drawn). Rows with temperature 0 take the argmax;
+        the others draw by inverse CDF in vocabulary order with the hashed uniform of (seed, position)."""

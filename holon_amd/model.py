@@ -1,0 +1,64 @@
+"""A model built from a spec: embedding, blocks in run order, final norm, head.
+core/holon/core/build.py:273-314 (`Model`, `build_model`)."""
+from __future__ import annotations
+
+import dataclasses
+
+import torch
+
+from .parts.base import Build, PagedState, Part, SlotState
+from .spec import ModelSpec
+
+
+@dataclasses.dataclass
+class Site:
+    """One entry of the run order as the cache sees it: which layer runs, which cache it uses and whether it writes
+    it. The cache manager fills `group`, `pages` and `slot_state` when it allocates."""
+
+    run: int
+    layer: int
+    writes: bool = True
+    owner: int | None = None                      # the run whose cache this one reads (None: its own)
+    group: int | None = None                      # paged group id
+    pages: torch.Tensor | None = None             # this site's page storage [num_pages, P * elems]
+    slot_state: dict[str, torch.Tensor] = dataclasses.field(default_factory=dict)   # name -> [S+1, *shape]
+
+
+class Model(Part):
+    def __init__(self, spec: ModelSpec, build: Build) -> None:
+        super().__init__(build)
+        self.spec = spec
+        self.attach("embed", build.make(spec.embed, vocab=spec.vocab, hidden=spec.hidden))
+        self.blocks: list[Part] = []
+        for i, layer in enumerate(spec.layers):
+            block = build.make(layer.block, layer=i, hidden=spec.hidden, mixer=layer.mixer, ffn=layer.ffn,
+                               norm=layer.norm)
+            self.blocks.append(self.attach(f"layers.{i}", block))
+        self.attach("norm", build.make(spec.norm, dim=spec.hidden))
+        self.attach("lm_head", build.make(spec.head, vocab=spec.vocab, hidden=spec.hidden, embed=self.embed))
+        self.sites = [Site(run=at, layer=r.layer, writes=r.reads is None, owner=r.reads)
+                      for at, r in enumerate(spec.order)]
+
+    def state_decls(self) -> list[list[PagedState | SlotState]]:
+        """Per run, what its mixer keeps between steps (empty for a run that reads another's cache)."""
+        out = []
+        for site in self.sites:
+            mixer = getattr(self.blocks[site.layer], "mixer", None)
+            out.append(list(mixer.state()) if mixer is not None and site.writes else [])
+        return out
+
+    def trunk(self, step) -> tuple[torch.Tensor, torch.Tensor | None]:
+        """The residual stream after every run, as (h, delta) with h + delta the stream [T, hidden]."""
+        h, delta = self.embed(step.token_ids), None
+        for site in self.sites:
+            h, delta = self.blocks[site.layer](h, delta, step, site)
+        return h, delta
+
+    def head(self, h: torch.Tensor, delta: torch.Tensor | None) -> torch.Tensor:
+        """Final norm and head on the given rows -> float32 logits [R, vocab]. The rows are consumed."""
+        x = self.norm(h) if delta is None else self.norm.add(delta, h)[0]
+        return self.lm_head(x)
+
+
+def build_model(spec: ModelSpec, build: Build) -> Model:
+    return Model(spec, build)

@@ -1,0 +1,117 @@
+"""What every part is: an object that declares its tensors and sub-parts, is filled by the weight loader, and is called
+with the step's context. Parts know their own sizes and constants and nothing of the model they are in.
+
+State a mixer keeps between steps is declared, not allocated: `PagedState` grows with the sequence and lives in
+pages; `SlotState` has a fixed size per request and lives in the request's slot. The cache manager allocates both
+(core/holon/api/state.py:27-53 is the reference's form of the two shapes).
+"""
+from __future__ import annotations
+
+import dataclasses
+from collections.abc import Iterator
+from typing import Any
+
+import torch
+
+from ..registry import part_class
+from ..spec import PartRef
+
+MODEL, FLOAT32, INT32 = "model", "float32", "int32"
+
+
+@dataclasses.dataclass(frozen=True)
+class ParamDecl:
+    """A tensor a part owns. `kind`: "model" is kept in the engine's dtype; "float32" is kept in 32-bit whatever the
+    engine's dtype; "int32" is an integer table."""
+
+    shape: tuple[int, ...]
+    kind: str = MODEL
+    init: str = "linear"                          # how random weights draw it: linear | norm
+
+
+@dataclasses.dataclass(frozen=True)
+class PagedState:
+    """State that grows by `elems` values per token. Sites whose declarations are equal share a page pool and a block
+    table; a window W > 0 says that tokens more than W-1 behind the newest are never read again."""
+
+    name: str
+    elems: int
+    window: int = 0
+    dtype: torch.dtype | None = None              # None: the engine's dtype
+
+
+@dataclasses.dataclass(frozen=True)
+class SlotState:
+    """State of fixed shape per request, addressed by the request's slot; zeroed when the slot is given out."""
+
+    name: str
+    shape: tuple[int, ...]
+    dtype: torch.dtype | None = None
+
+
+@dataclasses.dataclass
+class Build:
+    """What a part may know of the engine while it is built."""
+
+    kernels: Any
+    device: torch.device
+    dtype: torch.dtype
+    page_size: int = 16
+    max_model_len: int = 8192
+    max_seqs: int = 64
+    max_step_tokens: int = 4096
+
+    def make(self, ref: PartRef, **site: Any) -> "Part":
+        return part_class(ref)(self, **ref.get(), **site)
+
+
+class Part:
+    """Base of all parts. Subclasses call `declare` for tensors and `attach` for sub-parts in `__init__`."""
+
+    def __init__(self, build: Build) -> None:
+        self.build = build
+        self.kernels = build.kernels
+        self._decls: dict[str, ParamDecl] = {}
+        self._children: dict[str, Part] = {}
+
+    def declare(self, name: str, shape: tuple[int, ...], kind: str = MODEL, init: str = "linear") -> None:
+        self._decls[name] = ParamDecl(tuple(int(s) for s in shape), kind, init)
+        setattr(self, name, None)
+
+    def attach(self, name: str, part: "Part") -> "Part":
+        self._children[name] = part
+        setattr(self, name, part)
+        return part
+
+    def drop(self, name: str) -> None:
+        """Forget a sub-part (its weights were merged into another tensor)."""
+        self._children.pop(name)
+        setattr(self, name, None)
+
+    def named_params(self, prefix: str = "") -> Iterator[tuple[str, "Part", str, ParamDecl]]:
+        for name, decl in self._decls.items():
+            yield prefix + name, self, name, decl
+        for cname, child in self._children.items():
+            yield from child.named_params(f"{prefix}{cname}.")
+
+    def walk(self) -> Iterator["Part"]:
+        """Children first."""
+        for child in list(self._children.values()):
+            yield from child.walk()
+        yield self
+
+    def finalize(self) -> None:
+        """Called once after every tensor is loaded, children before parents (merge weights, build tables)."""
+
+    def state(self) -> list[PagedState | SlotState]:
+        """What this part keeps between steps (mixers)."""
+        return []
+
+    def nbytes(self) -> int:
+        total = 0
+        for part in self.walk():
+            for name in part._decls:
+                t = getattr(part, name)
+                if t is not None:
+                    total += t.numel() * t.element_size()
+        return total

@@ -1,0 +1,34 @@
+"""How a layer's parts are wired. Pre-norm residual block: std/holon_std/blocks/units.py:8-25."""
+from __future__ import annotations
+
+import torch
+
+from ..registry import register_part
+from ..spec import PartRef
+from .base import Build, Part
+
+
+@register_part("block", "prenorm")
+class PreNorm(Part):
+    """a = mixer(input_norm(h)); h += a; x = post_norm(h); h += ffn(x). Every add is fused into the norm that reads
+    its sum (the block's last add into the next reader's norm: `delta` is a term not yet added to `h`); all adds are
+    in the activation dtype."""
+
+    def __init__(self, build: Build, *, layer: int, hidden: int, mixer: PartRef, ffn: PartRef, norm: PartRef) -> None:
+        super().__init__(build)
+        self.attach("input_norm", build.make(norm, dim=hidden))
+        self.attach("mixer", build.make(mixer, layer=layer, hidden=hidden))
+        self.attach("post_norm", build.make(norm, dim=hidden))
+        self.attach("ffn", build.make(ffn, layer=layer, hidden=hidden))
+
+    def forward(self, h: torch.Tensor, delta: torch.Tensor | None, step, site
+                ) -> tuple[torch.Tensor, torch.Tensor | None]:
+        """The residual stream is `h + delta` on entry and on return; `h` is updated in place."""
+        if delta is None:
+            a = self.input_norm(h)
+        else:
+            a, h = self.input_norm.add(delta, h)
+        x, h = self.post_norm.add(self.mixer(a, step, site), h)
+        return h, self.ffn(x, step)
+
+    __call__ = forward

@@ -1,0 +1,32 @@
+"""Feed-forward parts. SwiGLU: std/holon_std/ffn/units.py:12-50, activation std/holon_std/ffn/reference.py:7-12."""
+from __future__ import annotations
+
+import torch
+
+from ..registry import register_part
+from .base import Build, Part
+from .linear import Linear
+
+
+@register_part("ffn", "swiglu")
+class SwiGLU(Part):
+    """down(silu(gate(x)) * up(x)); gate and up are merged into one product after loading (gate rows first)."""
+
+    def __init__(self, build: Build, *, inter: int, hidden: int, layer: int) -> None:
+        super().__init__(build)
+        self.inter, self.hidden = inter, hidden
+        self.attach("gate_proj", Linear(build, inp=hidden, out=inter))
+        self.attach("up_proj", Linear(build, inp=hidden, out=inter))
+        self.attach("down_proj", Linear(build, inp=inter, out=hidden))
+        self.gate_up: Linear | None = None
+
+    def finalize(self) -> None:
+        self.gate_up = Linear.merge(self.build, self.gate_proj, self.up_proj)
+        self.drop("gate_proj")
+        self.drop("up_proj")
+        self._children["gate_up"] = self.gate_up
+
+    def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
+        return self.down_proj(self.kernels.silu_mul(self.gate_up(x)))
+
+    __call__ = forward

@@ -1,0 +1,28 @@
+"""Dense projection without bias, and the merge of several into one product.
+std/holon_std/ops/units.py:189-277 (`Linear`, `merge`)."""
+from __future__ import annotations
+
+import torch
+
+from .base import Build, Part
+
+
+class Linear(Part):
+    def __init__(self, build: Build, *, inp: int, out: int) -> None:
+        super().__init__(build)
+        self.inp, self.out = inp, out
+        self.declare("weight", (out, inp))
+
+    def forward(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        return self.kernels.linear(x, self.weight, out_dtype)
+
+    __call__ = forward
+
+    @staticmethod
+    def merge(build: Build, *parts: "Linear") -> "Linear":
+        """One projection whose rows are the parts' rows in order; the parts give up their tensors."""
+        merged = Linear(build, inp=parts[0].inp, out=sum(p.out for p in parts))
+        merged.weight = torch.cat([p.weight for p in parts], dim=0)
+        for p in parts:
+            p.weight = None
+        return merged

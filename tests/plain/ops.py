@@ -1,0 +1,133 @@
+"""Plain twins of the device kernels: one slow torch function per operation of `holon_amd.kernels.api.Kernels`, with
+the same arguments and the same cache layout. Two uses: the yardstick each HIP kernel is compared with, alone, on the
+GPU; and a stand-in that lets the engine's logic (cache, step function, scheduler) run on the CPU in tests. The product
+never falls back to it.
+
+Formulas: std/holon_std/ops/reference.py:7-30 (norms, rope), std/holon_std/ffn/reference.py:7-12 (silu_mul),
+std/holon_std/mixers/gqa/reference.py:26-60 (paged attention), :91-101 (kv write),
+std/holon_std/sampling/sampler.py:24-61 (uniform, inverse CDF).
+"""
+from __future__ import annotations
+
+import torch
+
+
+def _rmsnorm(x, w, eps):
+    x32 = x.float()
+    return (x32 * torch.rsqrt(x32.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(x.dtype)
+
+
+def _rope(x, positions, table):
+    rd = table.shape[1]
+    cs = table[positions.long()]
+    cos, sin = cs[:, None, : rd // 2], cs[:, None, rd // 2:]
+    a, b = x[..., : rd // 2].float(), x[..., rd // 2: rd].float()
+    return torch.cat(((a * cos - b * sin).to(x.dtype), (b * cos + a * sin).to(x.dtype), x[..., rd:]), dim=-1)
+
+
+def _mix32(x):
+    m = 0xFFFFFFFF
+    x = x ^ (x >> 16)
+    x = (x * 0x7FEB352D) & m
+    x = x ^ (x >> 15)
+    x = (x * 0x846CA68B) & m
+    return x ^ (x >> 16)
+
+
+class TorchKernels:
+    name = "torch-plain"
+
+    def embedding(self, ids, table):
+        return table[ids.long()]
+
+    def rmsnorm(self, x, weight, eps):
+        return _rmsnorm(x, weight, eps)
+
+    def add_rmsnorm(self, x, residual, weight, eps):
+        residual.add_(x)
+        return _rmsnorm(residual, weight, eps)
+
+    def linear(self, x, weight, out_dtype=None):
+        return (x.float() @ weight.float().T).to(out_dtype or x.dtype)
+
+    def silu_mul(self, gate_up):
+        gate, up = gate_up.chunk(2, dim=-1)
+        return torch.nn.functional.silu(gate.float()).to(gate.dtype) * up
+
+    def rope(self, x, positions, table):
+        x.copy_(_rope(x, positions, table))
+
+    def kv_write(self, k, v, pages, write_page, write_off, page_size):
+        t, hkv, d = k.shape
+        kp = pages[:, 0].view(-1, hkv, page_size, d)
+        vp = pages[:, 1].view(-1, hkv, d, page_size)
+        kp[write_page.long(), :, write_off.long()] = k
+        vp[write_page.long(), :, :, write_off.long()] = v
+
+    def qk_norm_rope_write(self, qkv, heads, kv_heads, head_dim, q_weight, k_weight, eps, table, positions, pages,
+                           write_page, write_off, page_size):
+        t = qkv.shape[0]
+        q = qkv[:, : heads * head_dim].reshape(t, heads, head_dim)
+        k = qkv[:, heads * head_dim: (heads + kv_heads) * head_dim].reshape(t, kv_heads, head_dim)
+        v = qkv[:, (heads + kv_heads) * head_dim:].reshape(t, kv_heads, head_dim)
+        if q_weight is not None:
+            q, k = _rmsnorm(q, q_weight, eps), _rmsnorm(k, k_weight, eps)
+        if table is not None:
+            q, k = _rope(q, positions, table), _rope(k, positions, table)
+        if pages is not None:
+            self.kv_write(k, v, pages, write_page, write_off, page_size)
+        return q.contiguous()
+
+    def paged_attention(self, q, pages, table, rows, page_size, scale, window):
+        t, hq, d = q.shape
+        hkv = pages.shape[2]
+        kp = pages[:, 0].view(-1, hkv, page_size, d)
+        vp = pages[:, 1].view(-1, hkv, d, page_size)
+        out = torch.zeros_like(q)
+        qs = rows.query_start.tolist()
+        for b, (slot, n) in enumerate(zip(rows.slots.tolist(), rows.lens.tolist())):
+            s, e = qs[b], qs[b + 1]
+            if n == 0 or s == e:
+                continue
+            units = table[slot, : -(-n // page_size)].long()
+            k = kp[units].transpose(1, 2).reshape(-1, hkv, d)[:n].float().repeat_interleave(hq // hkv, dim=1)
+            v = vp[units].permute(0, 3, 1, 2).reshape(-1, hkv, d)[:n].float().repeat_interleave(hq // hkv, dim=1)
+            scores = torch.einsum("qhd,khd->hqk", q[s:e].float(), k) * scale
+            pos = torch.arange(n - (e - s), n, device=q.device)[:, None]
+            key = torch.arange(n, device=q.device)[None, :]
+            hidden = key > pos
+            if window:
+                hidden = hidden | (pos - key >= window)
+            probs = scores.masked_fill(hidden, float("-inf")).softmax(-1)
+            out[s:e] = torch.einsum("hqk,khd->qhd", probs, v).to(q.dtype)
+        return out
+
+    def argmax(self, logits):
+        return logits.argmax(-1).to(torch.int32)
+
+    def sample(self, logits, temperature, top_k, top_p, min_p, seeds, positions):
+        m = 0xFFFFFFFF
+        h = _mix32(seeds & m) ^ ((seeds >> 32) & m) ^ _mix32(positions & m)
+        h = _mix32(h)
+        u = (((h >> 8).float() + 0.5) * 2.0 ** -24).clamp(max=1 - 2.0 ** -24)
+        out = logits.argmax(-1)
+        for r in range(logits.shape[0]):
+            temp = float(temperature[r])
+            if temp == 0:
+                continue
+            x = logits[r].float() / temp
+            keep = torch.ones_like(x, dtype=torch.bool)
+            order = x.argsort(descending=True, stable=True)
+            if int(top_k[r]) > 0:
+                keep[order[int(top_k[r]):]] = False
+            q = torch.where(keep, x, float("-inf")).softmax(-1)
+            if float(top_p[r]) < 1:
+                sq = q[order]
+                keep[order[sq.cumsum(-1) - sq > float(top_p[r])]] = False
+            if float(min_p[r]) > 0:
+                keep &= q >= float(min_p[r]) * q.max()
+            q = torch.where(keep, q, 0.0)
+            c = q.cumsum(-1)
+            idx = torch.searchsorted(c, (u[r] * c[-1]).reshape(1), right=True)[0]
+            out[r] = idx.clamp(max=x.numel() - 1)
+        return out.to(torch.int32)

@@ -1,0 +1,71 @@
+"""Plain sampling: the distribution a row is drawn from (float64) and the counter-based uniform, in Python integers.
+
+Shares no code with `holon_amd.sampling`.
+"""
+from __future__ import annotations
+
+import torch
+
+M32 = 0xFFFFFFFF
+
+
+def mix32(x: int) -> int:
+    """lowbias32. std/holon_std/sampling/sampler.py:24-30."""
+    x &= M32
+    x ^= x >> 16
+    x = (x * 0x7FEB352D) & M32
+    x ^= x >> 15
+    x = (x * 0x846CA68B) & M32
+    x ^= x >> 16
+    return x
+
+
+def uniform(seed: int, position: int) -> float:
+    """One uniform in (0, 1) from (seed, position), 24 bits, as a float32 value.
+    std/holon_std/sampling/sampler.py:33-40."""
+    h = mix32(seed & M32) ^ ((seed >> 32) & M32) ^ mix32(position & M32)
+    h = mix32(h)
+    u = torch.tensor(float(h >> 8), dtype=torch.float32)
+    u = (u + 0.5) * torch.tensor(2.0 ** -24, dtype=torch.float32)
+    return float(torch.clamp(u, max=1 - 2.0 ** -24))
+
+
+def sequence_seed(seed: int, index: int) -> int:
+    """core/holon/api/batch.py:64-77."""
+    base = seed & (2 ** 63 - 1)
+    if index == 0:
+        return base
+    x = (base + index + 0x9E3779B97F4A7C15) & 0xFFFFFFFFFFFFFFFF
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9 & 0xFFFFFFFFFFFFFFFF
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EB & 0xFFFFFFFFFFFFFFFF
+    return (x ^ (x >> 31)) & (2 ** 63 - 1)
+
+
+def probs(logits: torch.Tensor, temperature: float, top_k: int = 0, top_p: float = 1.0, min_p: float = 0.0
+          ) -> torch.Tensor:
+    """The law of one row [V] in float64: temperature, then top-k, then top-p over the renormalised rest (the most
+    likely token always stays), then min-p against the largest probability after top-k; temperature 0 is one-hot at
+    the first maximum. std/holon_std/sampling/reference.py:13-30."""
+    x = logits.double()
+    if temperature == 0:
+        return torch.nn.functional.one_hot(x.argmax(), x.numel()).double()
+    x = x / temperature
+    keep = torch.ones_like(x, dtype=torch.bool)
+    order = x.argsort(descending=True, stable=True)
+    if top_k > 0:
+        keep[order[top_k:]] = False
+    q = torch.where(keep, x, float("-inf")).softmax(-1)
+    if top_p < 1:
+        sorted_q = q[order]
+        keep[order[sorted_q.cumsum(-1) - sorted_q > top_p]] = False
+    if min_p > 0:
+        keep &= q >= min_p * q.max()
+    return torch.where(keep, x, float("-inf")).softmax(-1)
+
+
+def draw(q: torch.Tensor, u: float) -> int:
+    """Inverse CDF in vocabulary order: the first index whose cumulative mass exceeds u * total.
+    std/holon_std/sampling/sampler.py:57-61."""
+    c = q.double().cumsum(-1)
+    idx = int(torch.searchsorted(c, torch.tensor(u, dtype=torch.float64) * c[-1], right=True))
+    return min(idx, q.numel() - 1)
