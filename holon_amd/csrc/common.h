@@ -1,0 +1,63 @@
+// Shared device helpers for the gfx950 kernels: element types, rounding, wave and block reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define WAVE 64
+
+typedef uint16_t bf16_t;   // bfloat16 kept as its bit pattern; all arithmetic is float32
+
+__device__ __forceinline__ float bf16_to_float(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+
+// Round to nearest, ties to even (what torch's .bfloat16() does); NaN stays NaN.
+__device__ __forceinline__ bf16_t float_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+  static constexpr int kVec = 4;   // elements in 16 bytes
+  static __device__ __forceinline__ float load(float v) { return v; }
+  static __device__ __forceinline__ float store(float v) { return v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+template <> struct Elem<bf16_t> {
+  static constexpr int kVec = 8;
+  static __device__ __forceinline__ float load(bf16_t v) { return bf16_to_float(v); }
+  static __device__ __forceinline__ bf16_t store(float v) { return float_to_bf16(v); }
+  static __device__ __forceinline__ float round(float v) { return bf16_to_float(float_to_bf16(v)); }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+
+// Host side: every entry point returns 0 or a negative code and leaves a message for holon_last_error().
+void holon_set_error(const char* fmt, ...);
+#define HOLON_CHECK(cond, ...)        \
+  do {                                \
+    if (!(cond)) {                    \
+      holon_set_error(__VA_ARGS__);   \
+      return -1;                      \
+    }                                 \
+  } while (0)
+#define HOLON_LAUNCH_OK()                                                        \
+  do {                                                                           \
+    hipError_t e_ = hipGetLastError();                                           \
+    if (e_ != hipSuccess) {                                                      \
+      holon_set_error("%s: launch failed: %s", __func__, hipGetErrorString(e_)); \
+      return -2;                                                                 \
+    }                                                                            \
+  } while (0)
+
+enum { HOLON_F32 = 0, HOLON_BF16 = 1 };

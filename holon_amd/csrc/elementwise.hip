@@ -1,0 +1,238 @@
+// Per-token operations: embedding gather, RMSNorm (plain and with the residual add), SiLU*mul, and the fused
+// per-head norm + rotary embedding + cache write. Everything is computed in float32 and rounded once per result.
+#include "common.h"
+#include "holon_hip.h"
+
+// ---------------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void embedding_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table, T* __restrict__ out,
+                                 int hidden) {
+  const int64_t t = blockIdx.x;
+  const T* src = table + (int64_t)ids[t] * hidden;
+  T* dst = out + t * hidden;
+  constexpr int V = Elem<T>::kVec;
+  if (hidden % V == 0) {
+    const uint4* s4 = reinterpret_cast<const uint4*>(src);
+    uint4* d4 = reinterpret_cast<uint4*>(dst);
+    for (int i = threadIdx.x; i < hidden / V; i += blockDim.x) d4[i] = s4[i];
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+  }
+}
+
+extern "C" int holon_embedding(const int32_t* ids, const void* table, void* out, int tokens, int hidden, int vocab,
+                               int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && hidden > 0 && vocab > 0, "embedding: bad sizes tokens=%d hidden=%d", tokens, hidden);
+  if (tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HOLON_F32)
+    embedding_kernel<float><<<tokens, 256, 0, s>>>(ids, (const float*)table, (float*)out, hidden);
+  else
+    embedding_kernel<bf16_t><<<tokens, 256, 0, s>>>(ids, (const bf16_t*)table, (bf16_t*)out, hidden);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// One wave per row. Pass 1: (residual += x, rounded) and the sum of squares; pass 2: scale and weight.
+template <typename T, bool ADD>
+__global__ void rmsnorm_kernel(const T* __restrict__ x, T* __restrict__ residual, const T* __restrict__ weight,
+                               T* __restrict__ y, int64_t rows, int dim, float eps) {
+  const int lane = threadIdx.x % WAVE;
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  if (row >= rows) return;
+  const T* xr = x + row * dim;
+  T* rr = ADD ? residual + row * dim : nullptr;
+  float ss = 0.f;
+  for (int i = lane; i < dim; i += WAVE) {
+    float v = Elem<T>::load(xr[i]);
+    if (ADD) {
+      v = Elem<T>::round(Elem<T>::load(rr[i]) + v);
+      rr[i] = Elem<T>::store(v);
+    }
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+  T* yr = y + row * dim;
+  for (int i = lane; i < dim; i += WAVE) {
+    const float v = ADD ? Elem<T>::load(rr[i]) : Elem<T>::load(xr[i]);
+    yr[i] = Elem<T>::store((v * inv) * Elem<T>::load(weight[i]));
+  }
+}
+
+extern "C" int holon_rmsnorm(const void* x, void* residual, const void* weight, void* y, int64_t rows, int dim,
+                             float eps, int dtype, void* stream) {
+  HOLON_CHECK(rows >= 0 && dim > 0, "rmsnorm: bad sizes rows=%lld dim=%d", (long long)rows, dim);
+  if (rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int waves = 4;
+  const unsigned grid = (unsigned)((rows + waves - 1) / waves);
+#define RMS_LAUNCH(T, ADD) \
+  rmsnorm_kernel<T, ADD><<<grid, waves * WAVE, 0, s>>>((const T*)x, (T*)residual, (const T*)weight, (T*)y, rows, dim, eps)
+  if (dtype == HOLON_F32) {
+    if (residual) RMS_LAUNCH(float, true); else RMS_LAUNCH(float, false);
+  } else {
+    if (residual) RMS_LAUNCH(bf16_t, true); else RMS_LAUNCH(bf16_t, false);
+  }
+#undef RMS_LAUNCH
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int64_t tokens, int inter) {
+  const int64_t n = tokens * inter;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = i / inter;
+    const int c = (int)(i - t * inter);
+    const float g = Elem<T>::load(gu[t * 2 * inter + c]);
+    const float u = Elem<T>::load(gu[t * 2 * inter + inter + c]);
+    const float s = Elem<T>::round(g / (1.0f + expf(-g)));
+    out[i] = Elem<T>::store(s * u);
+  }
+}
+
+extern "C" int holon_silu_mul(const void* gate_up, void* out, int64_t tokens, int inter, int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && inter > 0, "silu_mul: bad sizes");
+  if (tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t n = tokens * inter;
+  const unsigned grid = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+  if (dtype == HOLON_F32)
+    silu_mul_kernel<float><<<grid, 256, 0, s>>>((const float*)gate_up, (float*)out, tokens, inter);
+  else
+    silu_mul_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)gate_up, (bf16_t*)out, tokens, inter);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// One wave per (token, head) of the merged projection. Head index h: [0, Hq) queries, [Hq, Hq+Hkv) keys, the rest
+// values. The head is staged in LDS as float32 so that a lane can read its rotation partner.
+#define MAX_HEAD_DIM 512
+template <typename T>
+__global__ void qk_norm_rope_write_kernel(const T* qkv, int64_t qkv_stride, T* q_out,
+                                          int heads, int kv_heads, int head_dim, const T* __restrict__ q_weight,
+                                          const T* __restrict__ k_weight, float eps, const float* __restrict__ table,
+                                          int rotary_dim, const int32_t* __restrict__ positions,
+                                          T* __restrict__ pages, const int32_t* __restrict__ write_page,
+                                          const int32_t* __restrict__ write_off, int page_size, int total_heads) {
+  __shared__ float stage[4][MAX_HEAD_DIM];
+  const int w = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int t = blockIdx.x;
+  const int h = blockIdx.y * 4 + w;
+  const bool active = h < total_heads;   // no early return: every wave reaches the barrier below
+  const T* src = qkv + (int64_t)t * qkv_stride + (int64_t)h * head_dim;
+  const bool is_q = active && h < heads, is_k = active && !is_q && h < heads + kv_heads;
+  float* buf = stage[w];
+  if (is_q || is_k) {
+    const T* weight = is_q ? q_weight : k_weight;
+    float ss = 0.f;
+    for (int d = lane; d < head_dim; d += WAVE) {
+      const float v = Elem<T>::load(src[d]);
+      buf[d] = v;
+      ss += v * v;
+    }
+    if (weight != nullptr) {
+      ss = wave_sum(ss);
+      const float inv = 1.0f / sqrtf(ss / (float)head_dim + eps);
+      for (int d = lane; d < head_dim; d += WAVE) buf[d] = Elem<T>::round((buf[d] * inv) * Elem<T>::load(weight[d]));
+    }
+  }
+  __syncthreads();   // rotation partners were staged by other lanes
+  if (is_q || is_k) {
+    T* dst;
+    int64_t dstride = 1;
+    if (is_q) {
+      dst = q_out + ((int64_t)t * heads + h) * head_dim;
+    } else {
+      const int hk = h - heads;
+      dst = pages + (((int64_t)write_page[t] * 2 + 0) * kv_heads + hk) * (int64_t)page_size * head_dim +
+            (int64_t)write_off[t] * head_dim;
+    }
+    const int half = rotary_dim / 2;
+    const float* cs = table != nullptr ? table + (int64_t)positions[t] * rotary_dim : nullptr;
+    for (int d = lane; d < head_dim; d += WAVE) {
+      float o;
+      if (cs != nullptr && d < half) {
+        o = buf[d] * cs[d] - buf[d + half] * cs[half + d];
+      } else if (cs != nullptr && d < rotary_dim) {
+        const int i = d - half;
+        o = buf[d] * cs[i] + buf[i] * cs[half + i];
+      } else {
+        o = buf[d];
+      }
+      dst[d * dstride] = Elem<T>::store(o);
+    }
+  } else if (active) {
+    const int hk = h - heads - kv_heads;
+    T* dst = pages + (((int64_t)write_page[t] * 2 + 1) * kv_heads + hk) * (int64_t)page_size * head_dim +
+             write_off[t];
+    for (int d = lane; d < head_dim; d += WAVE) dst[(int64_t)d * page_size] = src[d];
+  }
+}
+
+extern "C" int holon_qk_norm_rope_write(const void* qkv, int64_t qkv_stride, void* q_out, int tokens, int heads,
+                                        int kv_heads, int head_dim, const void* q_weight, const void* k_weight,
+                                        float eps, const float* table, int rotary_dim, int max_positions,
+                                        const int32_t* positions, void* pages, const int32_t* write_page,
+                                        const int32_t* write_off, int page_size, int num_pages, int dtype,
+                                        void* stream) {
+  HOLON_CHECK(tokens >= 0 && heads > 0 && kv_heads >= 0 && head_dim > 0, "qk_norm_rope_write: bad sizes");
+  HOLON_CHECK(head_dim <= MAX_HEAD_DIM, "qk_norm_rope_write: head_dim %d exceeds %d", head_dim, MAX_HEAD_DIM);
+  HOLON_CHECK((q_weight == nullptr) == (k_weight == nullptr) || kv_heads == 0 || pages == nullptr,
+              "qk_norm_rope_write: q and k norm weights must both be given or both be absent");
+  HOLON_CHECK(table == nullptr || (rotary_dim > 0 && rotary_dim % 2 == 0 && rotary_dim <= head_dim && positions),
+              "qk_norm_rope_write: rotary_dim %d must be even and within head_dim %d", rotary_dim, head_dim);
+  HOLON_CHECK(pages == nullptr || (write_page && write_off && page_size > 0 && num_pages > 0),
+              "qk_norm_rope_write: a cache needs write targets and a page size");
+  if (tokens == 0) return 0;
+  const int total_heads = pages != nullptr ? heads + 2 * kv_heads : heads;
+  dim3 grid(tokens, (total_heads + 3) / 4);
+  hipStream_t s = (hipStream_t)stream;
+#define QK_LAUNCH(T)                                                                                              \
+  qk_norm_rope_write_kernel<T><<<grid, 4 * WAVE, 0, s>>>((const T*)qkv, qkv_stride, (T*)q_out, heads, kv_heads,    \
+                                                        head_dim, (const T*)q_weight, (const T*)k_weight, eps,    \
+                                                        table, rotary_dim, positions, (T*)pages, write_page,      \
+                                                        write_off, page_size, total_heads)
+  if (dtype == HOLON_F32) QK_LAUNCH(float); else QK_LAUNCH(bf16_t);
+#undef QK_LAUNCH
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v, T* __restrict__ pages,
+                                const int32_t* __restrict__ write_page, const int32_t* __restrict__ write_off,
+                                int kv_heads, int head_dim, int page_size) {
+  const int t = blockIdx.x, hk = blockIdx.y;
+  const int64_t plane = (int64_t)page_size * head_dim;
+  const T* ks = k + ((int64_t)t * kv_heads + hk) * head_dim;
+  const T* vs = v + ((int64_t)t * kv_heads + hk) * head_dim;
+  T* kd = pages + (((int64_t)write_page[t] * 2 + 0) * kv_heads + hk) * plane + (int64_t)write_off[t] * head_dim;
+  T* vd = pages + (((int64_t)write_page[t] * 2 + 1) * kv_heads + hk) * plane + write_off[t];
+  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+    kd[d] = ks[d];
+    vd[(int64_t)d * page_size] = vs[d];
+  }
+}
+
+extern "C" int holon_kv_write(const void* k, const void* v, void* pages, const int32_t* write_page,
+                              const int32_t* write_off, int tokens, int kv_heads, int head_dim, int page_size,
+                              int num_pages, int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && kv_heads > 0 && head_dim > 0 && page_size > 0 && num_pages > 0, "kv_write: bad sizes");
+  if (tokens == 0) return 0;
+  dim3 grid(tokens, kv_heads);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HOLON_F32)
+    kv_write_kernel<float><<<grid, WAVE, 0, s>>>((const float*)k, (const float*)v, (float*)pages, write_page,
+                                                 write_off, kv_heads, head_dim, page_size);
+  else
+    kv_write_kernel<bf16_t><<<grid, WAVE, 0, s>>>((const bf16_t*)k, (const bf16_t*)v, (bf16_t*)pages, write_page,
+                                                  write_off, kv_heads, head_dim, page_size);
+  HOLON_LAUNCH_OK();
+  return 0;
+}

@@ -1,0 +1,225 @@
+"""The HIP kernels behind the `Kernels` contract: ctypes bindings to libholon_hip.so (hand-written gfx950 kernels in
+`holon_amd/csrc`). Dense matrix products go to the vendor library through torch where the reference uses its vendor
+library for them (std/holon_std/ops/units.py:229); everything else is this package's own code. There is no fallback:
+a missing library is built, and if that fails, loading raises."""
+from __future__ import annotations
+
+import ctypes
+import sys
+
+import torch
+
+from . import build as _build
+from .api import AttnRows
+
+_P, _I, _L, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+class HipKernels:
+    name = "hip-gfx950"
+    _instance: "HipKernels | None" = None
+
+    @classmethod
+    def load(cls, build_if_missing: bool = True) -> "HipKernels":
+        if cls._instance is None:
+            path = _build.find_library()
+            if path is None:
+                if not build_if_missing:
+                    raise KernelError("libholon_hip.so is not built (run `python -m holon_amd.kernels.build`)")
+                path = _build.build()
+            else:
+                stamp = path.parent / (path.name + ".hash")
+                if stamp.is_file() and stamp.read_text().strip() != _build.source_hash():
+                    print(f"holon_amd: warning: {path} was built from other sources than holon_amd/csrc holds; "
+                          "rebuild with `python -m holon_amd.kernels.build`", file=sys.stderr)
+            cls._instance = cls(str(path))
+        return cls._instance
+
+    def __init__(self, path: str) -> None:
+        try:
+            self.lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError(f"cannot load {path}: {e}") from e
+        self.path = path
+        lib = self.lib
+        lib.holon_last_error.restype = ctypes.c_char_p
+        sig = {
+            "holon_embedding": [_P, _P, _P, _I, _I, _I, _I, _P],
+            "holon_rmsnorm": [_P, _P, _P, _P, _L, _I, _F, _I, _P],
+            "holon_silu_mul": [_P, _P, _L, _I, _I, _P],
+            "holon_qk_norm_rope_write": [_P, _L, _P, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _P, _P, _P, _P, _I, _I,
+                                         _I, _P],
+            "holon_kv_write": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+            "holon_attention_generic": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+            "holon_argmax": [_P, _P, _I, _I, _P],
+            "holon_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
+        }
+        for name, args in sig.items():
+            fn = getattr(lib, name)
+            fn.argtypes, fn.restype = args, _I
+
+    # -- plumbing -------------------------------------------------------------------------------------------------
+    def _call(self, fn, *args) -> None:
+        if fn(*args) != 0:
+            raise KernelError(self.lib.holon_last_error().decode())
+
+    @staticmethod
+    def _stream() -> int:
+        return torch.cuda.current_stream().cuda_stream
+
+    @staticmethod
+    def _check(t: torch.Tensor, what: str, dtype: torch.dtype | None = None) -> None:
+        if not t.is_cuda:
+            raise KernelError(f"{what}: the HIP kernels need a GPU tensor, got one on {t.device}")
+        if not t.is_contiguous():
+            raise KernelError(f"{what}: tensor must be contiguous")
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError(f"{what}: expected {dtype}, got {t.dtype}")
+
+    @staticmethod
+    def _dt(t: torch.Tensor, what: str) -> int:
+        if t.dtype not in _DT:
+            raise KernelError(f"{what}: dtype {t.dtype} is not served (float32 and bfloat16 are)")
+        return _DT[t.dtype]
+
+    # -- ops ------------------------------------------------------------------------------------------------------
+    def embedding(self, ids, table):
+        self._check(ids, "embedding ids", torch.int32)
+        self._check(table, "embedding table")
+        out = torch.empty((ids.shape[0], table.shape[1]), dtype=table.dtype, device=table.device)
+        self._call(self.lib.holon_embedding, ids.data_ptr(), table.data_ptr(), out.data_ptr(), ids.shape[0],
+                   table.shape[1], table.shape[0], self._dt(table, "embedding"), self._stream())
+        return out
+
+    def rmsnorm(self, x, weight, eps):
+        self._check(x, "rmsnorm x")
+        self._check(weight, "rmsnorm weight", x.dtype)
+        dim = x.shape[-1]
+        if weight.shape != (dim,):
+            raise KernelError(f"rmsnorm: weight {tuple(weight.shape)} does not fit rows of {dim}")
+        y = torch.empty_like(x)
+        self._call(self.lib.holon_rmsnorm, x.data_ptr(), None, weight.data_ptr(), y.data_ptr(), x.numel() // dim, dim,
+                   float(eps), self._dt(x, "rmsnorm"), self._stream())
+        return y
+
+    def add_rmsnorm(self, x, residual, weight, eps):
+        self._check(x, "add_rmsnorm x")
+        self._check(residual, "add_rmsnorm residual", x.dtype)
+        self._check(weight, "add_rmsnorm weight", x.dtype)
+        dim = x.shape[-1]
+        if residual.shape != x.shape or weight.shape != (dim,):
+            raise KernelError(f"add_rmsnorm: shapes {tuple(x.shape)}, {tuple(residual.shape)}, {tuple(weight.shape)}")
+        y = torch.empty_like(x)
+        self._call(self.lib.holon_rmsnorm, x.data_ptr(), residual.data_ptr(), weight.data_ptr(), y.data_ptr(),
+                   x.numel() // dim, dim, float(eps), self._dt(x, "add_rmsnorm"), self._stream())
+        return y
+
+    def linear(self, x, weight, out_dtype=None):
+        # the vendor library's product, float32 accumulation (no reduced-precision mode for float32 operands)
+        y = torch.matmul(x, weight.t())
+        return y if out_dtype in (None, y.dtype) else y.to(out_dtype)
+
+    def silu_mul(self, gate_up):
+        self._check(gate_up, "silu_mul")
+        t, two_i = gate_up.shape
+        if two_i % 2:
+            raise KernelError(f"silu_mul: width {two_i} is odd")
+        out = torch.empty((t, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+        self._call(self.lib.holon_silu_mul, gate_up.data_ptr(), out.data_ptr(), t, two_i // 2,
+                   self._dt(gate_up, "silu_mul"), self._stream())
+        return out
+
+    def rope(self, x, positions, table):
+        self._check(x, "rope x")
+        self._check(positions, "rope positions", torch.int32)
+        self._check(table, "rope table", torch.float32)
+        t, heads, d = x.shape
+        self._call(self.lib.holon_qk_norm_rope_write, x.data_ptr(), heads * d, x.data_ptr(), t, heads, 0, d, None,
+                   None, 0.0, table.data_ptr(), table.shape[1], table.shape[0], positions.data_ptr(), None, None,
+                   None, 1, 1, self._dt(x, "rope"), self._stream())
+
+    def kv_write(self, k, v, pages, write_page, write_off, page_size):
+        for t, what in ((k, "k"), (v, "v"), (pages, "pages")):
+            self._check(t, f"kv_write {what}", k.dtype)
+        self._check(write_page, "kv_write page", torch.int32)
+        self._check(write_off, "kv_write offset", torch.int32)
+        t, hkv, d = k.shape
+        if pages.shape[1:] != (2, hkv, page_size * d) or v.shape != k.shape:
+            raise KernelError(f"kv_write: pages {tuple(pages.shape)} do not fit {hkv} heads of {d} in pages of {page_size}")
+        self._call(self.lib.holon_kv_write, k.data_ptr(), v.data_ptr(), pages.data_ptr(), write_page.data_ptr(),
+                   write_off.data_ptr(), t, hkv, d, page_size, pages.shape[0], self._dt(k, "kv_write"), self._stream())
+
+    def qk_norm_rope_write(self, qkv, heads, kv_heads, head_dim, q_weight, k_weight, eps, table, positions, pages,
+                           write_page, write_off, page_size):
+        self._check(qkv, "qkv")
+        t, width = qkv.shape
+        if width != (heads + 2 * kv_heads) * head_dim:
+            raise KernelError(f"qkv width {width} is not ({heads} + 2*{kv_heads}) * {head_dim}")
+        for w in (q_weight, k_weight):
+            if w is not None:
+                self._check(w, "q/k norm weight", qkv.dtype)
+                if w.shape != (head_dim,):
+                    raise KernelError(f"q/k norm weight {tuple(w.shape)} does not fit head_dim {head_dim}")
+        if table is not None:
+            self._check(table, "rope table", torch.float32)
+            self._check(positions, "positions", torch.int32)
+        if pages is not None:
+            self._check(pages, "pages", qkv.dtype)
+            self._check(write_page, "write_page", torch.int32)
+            self._check(write_off, "write_off", torch.int32)
+            if pages.shape[1:] != (2, kv_heads, page_size * head_dim):
+                raise KernelError(f"pages {tuple(pages.shape)} do not fit {kv_heads} heads of {head_dim}, page {page_size}")
+        q = torch.empty((t, heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+        self._call(self.lib.holon_qk_norm_rope_write, qkv.data_ptr(), width, q.data_ptr(), t, heads, kv_heads,
+                   head_dim, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(table),
+                   table.shape[1] if table is not None else 0, table.shape[0] if table is not None else 0,
+                   _ptr(positions), _ptr(pages), _ptr(write_page), _ptr(write_off), page_size,
+                   pages.shape[0] if pages is not None else 0, self._dt(qkv, "qkv"), self._stream())
+        return q
+
+    def paged_attention(self, q, pages, table, rows: AttnRows, page_size, scale, window):
+        self._check(q, "attention q")
+        self._check(pages, "attention pages", q.dtype)
+        self._check(table, "block table", torch.int32)
+        t, hq, d = q.shape
+        hkv = pages.shape[2]
+        if pages.shape[1] != 2 or pages.shape[3] != page_size * d:
+            raise KernelError(f"attention: pages {tuple(pages.shape)} do not fit head_dim {d}, page {page_size}")
+        out = torch.empty_like(q)
+        b = rows.slots.shape[0]
+        self._call(self.lib.holon_attention_generic, q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(),
+                   table.shape[1], rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr(), b, t, hq,
+                   hkv, d, page_size, pages.shape[0], float(scale), int(window), self._dt(q, "attention"),
+                   self._stream())
+        return out
+
+    def argmax(self, logits):
+        self._check(logits, "argmax logits", torch.float32)
+        out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+        self._call(self.lib.holon_argmax, logits.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1],
+                   self._stream())
+        return out
+
+    def sample(self, logits, temperature, top_k, top_p, min_p, seeds, positions):
+        self._check(logits, "sample logits", torch.float32)
+        r = logits.shape[0]
+        for t, dt, what in ((temperature, torch.float32, "temperature"), (top_k, torch.int32, "top_k"),
+                            (top_p, torch.float32, "top_p"), (min_p, torch.float32, "min_p"),
+                            (seeds, torch.int64, "seeds"), (positions, torch.int64, "positions")):
+            self._check(t, f"sample {what}", dt)
+            if t.shape != (r,):
+                raise KernelError(f"sample {what}: shape {tuple(t.shape)} for {r} rows")
+        out = torch.empty((r,), dtype=torch.int32, device=logits.device)
+        self._call(self.lib.holon_sample, logits.data_ptr(), out.data_ptr(), r, logits.shape[1],
+                   temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), min_p.data_ptr(), seeds.data_ptr(),
+                   positions.data_ptr(), self._stream())
+        return out

@@ -1,0 +1,275 @@
+"""Each HIP kernel alone against its plain twin (tests/plain/ops.py) on the same inputs, at sizes other than the tiny
+models': the reference's own test shapes (plugins/tests/test_op_kernels.py:28-72, test_attention_kernels.py:20-66)
+and awkward ones (widths that are no power of two, head sizes in steps of 16, page sizes from 1 up)."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from holon_amd.kernels.api import AttnRows
+from tests import helpers as H
+from tests.plain.ops import TorchKernels
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+PLAIN = TorchKernels()
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from holon_amd.kernels import load_hip
+    return load_hip()
+
+
+def _randn(*shape, dtype, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(37, 4096), (37, 8, 128), (5, 100), (3, 7, 48), (1, 12288), (130, 16)])
+def test_rmsnorm_and_add(hip, dtype, shape):
+    x, r = _randn(*shape, dtype=dtype, seed=1), _randn(*shape, dtype=dtype, seed=2)
+    w = (1 + 0.1 * torch.randn(shape[-1], generator=torch.Generator().manual_seed(3))).to(dtype).cuda()
+    x0 = x.clone()
+    for eps in (1e-6, 1e-2):
+        got, want = hip.rmsnorm(x, w, eps), PLAIN.rmsnorm(x.float(), w.float(), eps)
+        assert torch.equal(x, x0), "rmsnorm wrote its input"
+        assert H.op_budget_usage(got, want, dtype, shape[-1]) <= 1
+    x2, r_hip, r_ref = x.reshape(-1, shape[-1]), r.reshape(-1, shape[-1]).clone(), r.reshape(-1, shape[-1]).clone()
+    got = hip.add_rmsnorm(x2, r_hip, w, 1e-6)
+    want = PLAIN.add_rmsnorm(x2, r_ref, w, 1e-6)
+    assert torch.equal(r_hip, r_ref), "the residual sum is one rounding of x + r"
+    assert H.op_budget_usage(got, want.float(), dtype, shape[-1]) <= 1
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding_and_silu_mul(hip, dtype):
+    table = _randn(1000, 120, dtype=dtype, seed=4)
+    ids = torch.tensor([0, 999, 5, 5, 123], dtype=torch.int32).cuda()
+    assert torch.equal(hip.embedding(ids, table), table[ids.long()])
+    table = _randn(333, 4096, dtype=dtype, seed=5)
+    assert torch.equal(hip.embedding(ids[2:], table), table[ids[2:].long()])
+    for t, inter in ((17, 12288), (3, 100), (1, 7)):
+        gu = _randn(t, 2 * inter, dtype=dtype, seed=6, scale=3.0)
+        got, want = hip.silu_mul(gu), PLAIN.silu_mul(gu.float())
+        assert H.op_budget_usage(got, want, dtype, 1) <= 1
+    gu = torch.zeros(2, 8, dtype=dtype).cuda()
+    gu[:, 4:] = 1
+    assert torch.equal(hip.silu_mul(gu), torch.zeros(2, 4, dtype=dtype).cuda())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize(("head_dim", "rotary_dim", "theta"), [(128, 128, 1e6), (256, 64, 1e7), (48, 48, 1e4), (16, 8, 1e4)])
+def test_rope(hip, dtype, head_dim, rotary_dim, theta):
+    from holon_amd.parts.positions import rope_table
+    table = rope_table(8192, rotary_dim, theta).cuda()
+    pos = torch.tensor([0, 1, 2, 15, 16, 1000, 4095, 8191] + list(range(100, 121)), dtype=torch.int32).cuda()
+    q = _randn(29, 24, head_dim, dtype=dtype, seed=7)
+    want = q.clone()
+    PLAIN.rope(want, pos, table)
+    got = q.clone()
+    hip.rope(got, pos, table)
+    assert H.op_budget_usage(got, want, dtype, 2) <= 1
+    assert torch.equal(got[..., rotary_dim:], q[..., rotary_dim:])          # the rest passes through untouched
+    assert torch.equal(got[0], q[0])                                         # position 0: identity
+    # against the formula itself, in float64, half-split pairing
+    inv = theta ** (-torch.arange(0, rotary_dim, 2, dtype=torch.float64) / rotary_dim)
+    ang = pos.double().cpu()[:, None] * inv
+    a, b = q[..., : rotary_dim // 2].double().cpu(), q[..., rotary_dim // 2: rotary_dim].double().cpu()
+    ref = torch.cat((a * ang.cos()[:, None] - b * ang.sin()[:, None], b * ang.cos()[:, None] + a * ang.sin()[:, None]), -1)
+    assert (got[..., :rotary_dim].double().cpu() - ref).abs().max() < (4e-3 if dtype == torch.float32 else 4e-2)
+
+
+def _paged_case(rows, heads, kv_heads, head_dim, page, dtype, seed=0, max_seqs=8, scale_q=1.0):
+    """rows: (tokens before this step, tokens this step). A shuffled block table with spare pages."""
+    g = torch.Generator().manual_seed(seed)
+    rng = np.random.default_rng(seed)
+    slots = rng.permutation(max_seqs)[: len(rows)].astype(np.int32)
+    max_pages = -(-max(s + n for s, n in rows) // page)
+    units = max_seqs * max_pages + 7
+    table = torch.from_numpy(rng.permutation(units)[: max_seqs * max_pages].reshape(max_seqs, max_pages).astype(np.int32))
+    pages = torch.randn(units, 2, kv_heads, page * head_dim, generator=g).to(dtype).cuda()
+    counts = np.array([n for _, n in rows])
+    lens = np.array([s + n for s, n in rows])
+    qstart = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    q = (torch.randn(int(counts.sum()), heads, head_dim, generator=g) * scale_q).to(dtype).cuda()
+    dec, chk = np.flatnonzero(counts == 1), np.flatnonzero(counts > 1)
+    i32 = lambda a: torch.as_tensor(np.asarray(a, dtype=np.int32)).cuda()
+    attn = AttnRows(slots=i32(slots), lens=i32(lens), query_start=i32(qstart), decode_rows=i32(dec), chunk_rows=i32(chk),
+                    n_decode=len(dec), n_chunk=len(chk), max_decode_len=int(lens[dec].max()) if len(dec) else 0,
+                    max_chunk_query=int(counts[chk].max()) if len(chk) else 0,
+                    max_chunk_len=int(lens[chk].max()) if len(chk) else 0)
+    return q, pages, table.cuda(), attn
+
+
+GEOMETRIES = [(32, 8, 128), (16, 4, 256), (16, 8, 64), (6, 3, 32), (4, 1, 16), (5, 5, 48), (12, 2, 80)]
+ROWSETS = [[(0, 1), (0, 17), (5, 16), (31, 33), (0, 64), (100, 7), (16, 16)],
+           [(0, 1), (15, 1), (16, 1), (99, 1), (999, 1), (4096, 1)],
+           [(63, 1), (200, 2), (17, 1), (0, 130), (1, 1)]]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page", [16, 8, 64, 1, 5])
+@pytest.mark.parametrize("geometry", GEOMETRIES)
+def test_paged_attention(hip, dtype, page, geometry):
+    heads, kv_heads, head_dim = geometry
+    if page in (1, 5) and head_dim > 64:
+        pytest.skip("the odd page sizes are covered at the small head sizes")
+    for seed, rows in enumerate(ROWSETS):
+        if page < 8:
+            rows = [(min(s, 300), n) for s, n in rows]
+        q, pages, table, attn = _paged_case(rows, heads, kv_heads, head_dim, page, dtype, seed)
+        scale = head_dim ** -0.5
+        want = PLAIN.paged_attention(q.float(), pages.float(), table, attn, page, scale, 0)
+        got = hip.paged_attention(q, pages, table, attn, page, scale, 0)
+        again = hip.paged_attention(q, pages, table, attn, page, scale, 0)
+        assert torch.equal(got, again), "two runs differ"
+        assert H.op_budget_usage(got, want, dtype, head_dim) <= 1, (geometry, page, rows)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 7, 16, 100])
+def test_paged_attention_window(hip, dtype, window):
+    for geometry, page in (((16, 8, 64), 16), ((6, 3, 32), 8), ((32, 8, 128), 16)):
+        heads, kv_heads, head_dim = geometry
+        q, pages, table, attn = _paged_case(ROWSETS[0] + [(300, 1), (98, 1)], heads, kv_heads, head_dim, page, dtype, 3)
+        want = PLAIN.paged_attention(q.float(), pages.float(), table, attn, page, head_dim ** -0.5, window)
+        got = hip.paged_attention(q, pages, table, attn, page, head_dim ** -0.5, window)
+        assert H.op_budget_usage(got, want, dtype, head_dim) <= 1, (geometry, window)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_a_far_key(hip, dtype):
+    """One key among thousands carries the weight: its query is aligned with it and scaled up. A kernel that skips or
+    misplaces a page, a tile edge or the last key shows here."""
+    heads, kv_heads, head_dim, page = 8, 2, 64, 16
+    for n, target in ((4097, 0), (4097, 4096), (1000, 511), (1000, 512), (2049, 1023), (130, 64), (130, 63)):
+        q, pages, table, attn = _paged_case([(n - 1, 1)], heads, kv_heads, head_dim, page, dtype, seed=n + target)
+        slot = int(attn.slots[0])
+        unit, off = int(table[slot, target // page]), target % page
+        kp = pages[:, 0].view(-1, kv_heads, page, head_dim)
+        for h in range(heads):
+            q[0, h] = kp[unit, h // (heads // kv_heads), off].float().mul(4.0).to(dtype)
+        want = PLAIN.paged_attention(q.float(), pages.float(), table, attn, page, head_dim ** -0.5, 0)
+        vp = pages[:, 1].view(-1, kv_heads, head_dim, page)
+        assert (want[0, 0] - vp[unit, 0, :, off].float()).abs().max() < 0.05       # the test itself singles the key out
+        got = hip.paged_attention(q, pages, table, attn, page, head_dim ** -0.5, 0)
+        assert H.op_budget_usage(got, want, dtype, head_dim) <= 1, (n, target)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geometry", [(32, 8, 128, 16), (6, 3, 32, 8), (4, 1, 16, 16), (5, 5, 48, 4), (16, 4, 256, 32)])
+def test_fused_norm_rope_write_is_the_three_ops(hip, dtype, geometry):
+    from holon_amd.parts.positions import rope_table
+    heads, kv_heads, head_dim, page = geometry
+    t, units = 45, 40
+    qkv = _randn(t, (heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=8)
+    qw, kw = _randn(head_dim, dtype=dtype, seed=9), _randn(head_dim, dtype=dtype, seed=10)
+    table = rope_table(4096, head_dim, 1e6).cuda()
+    rng = np.random.default_rng(0)
+    where = rng.permutation(units * page)[:t]
+    pos = torch.as_tensor(rng.integers(0, 4096, t).astype(np.int32)).cuda()
+    wp, wo = (torch.as_tensor((where // page).astype(np.int32)).cuda(), torch.as_tensor((where % page).astype(np.int32)).cuda())
+    for use_norm, use_rope in ((True, True), (False, True), (True, False), (False, False)):
+        pages_h = torch.zeros(units, 2, kv_heads, page * head_dim, dtype=dtype).cuda()
+        pages_p = pages_h.clone()
+        args = (heads, kv_heads, head_dim, qw if use_norm else None, kw if use_norm else None, 1e-6,
+                table if use_rope else None, pos)
+        got = hip.qk_norm_rope_write(qkv, *args, pages_h, wp, wo, page)
+        want = PLAIN.qk_norm_rope_write(qkv, *args, pages_p, wp, wo, page)
+        assert H.op_budget_usage(got, want, dtype, head_dim) <= 1
+        assert H.op_budget_usage(pages_h, pages_p, dtype, head_dim) <= 1
+        assert torch.equal(pages_h == 0, pages_p == 0), "a cache entry outside the written ones changed"
+        assert torch.equal(pages_h[:, 1], pages_p[:, 1]), "values are copied bit for bit"
+    # queries only (a run that reads another run's cache)
+    got = hip.qk_norm_rope_write(qkv, heads, kv_heads, head_dim, qw, kw, 1e-6, table, pos, None, None, None, page)
+    want = PLAIN.qk_norm_rope_write(qkv, heads, kv_heads, head_dim, qw, kw, 1e-6, table, pos, None, None, None, page)
+    assert H.op_budget_usage(got, want, dtype, head_dim) <= 1
+    # the unfused write
+    k, v = _randn(t, kv_heads, head_dim, dtype=dtype, seed=11), _randn(t, kv_heads, head_dim, dtype=dtype, seed=12)
+    pages_h, pages_p = torch.zeros_like(pages_h), torch.zeros_like(pages_p)
+    hip.kv_write(k, v, pages_h, wp, wo, page)
+    PLAIN.kv_write(k, v, pages_p, wp, wo, page)
+    assert torch.equal(pages_h, pages_p)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_linear(hip, dtype):
+    for t, k, n in ((1, 4096, 6144), (8, 4096, 1000), (17, 100, 333), (64, 12288, 4096), (300, 120, 1000), (2, 96, 384)):
+        x, w = _randn(t, k, dtype=dtype, seed=13), _randn(n, k, dtype=dtype, seed=14, scale=0.05)
+        want = x.double() @ w.double().T
+        got = hip.linear(x, w)
+        assert got.dtype == dtype and H.op_budget_usage(got, want, dtype, k) <= 1, (t, k, n)
+        got32 = hip.linear(x, w, torch.float32)
+        assert got32.dtype == torch.float32 and H.op_budget_usage(got32, want, dtype, k) <= 1
+    # exact arithmetic: activations in {-1, 0, 1} and weights in {-1, 0, 1} / 8 make every partial sum exact, so any
+    # order of summation gives the same bits (plugins/tests/test_attention_kv_quant.py:244-261)
+    g = torch.Generator().manual_seed(15)
+    x = torch.randint(-1, 2, (5, 512), generator=g).to(dtype).cuda()
+    w = (torch.randint(-1, 2, (200, 512), generator=g).float() / 8).to(dtype).cuda()
+    assert torch.equal(hip.linear(x, w).float(), x.float() @ w.float().T)
+    # a row's result does not depend on the rows beside it, beyond rounding
+    x = _randn(64, 4096, dtype=dtype, seed=16)
+    w = _randn(512, 4096, dtype=dtype, seed=17, scale=0.02)
+    assert H.op_budget_usage(hip.linear(x[:1].contiguous(), w), hip.linear(x, w)[:1].float(), dtype, 4096) <= 1
+
+
+def test_argmax_and_sampling(hip):
+    from tests.plain import sampling as S
+    g = torch.Generator().manual_seed(20)
+    logits = (torch.randn(9, 151_936, generator=g) * 3).cuda()
+    logits[3, 777] = logits[3, 90_000] = 50.0                     # a tie: the first index wins
+    assert hip.argmax(logits).tolist() == logits.argmax(-1).tolist()
+    assert int(hip.argmax(logits)[3]) == 777
+    # the law, by counting: one row of 40 logits drawn 100,000 times at consecutive positions
+    v, n = 40, 100_000
+    row = torch.randn(v, generator=torch.Generator().manual_seed(0)) * 2
+    row[7] = row[11]                                              # equal logits straddling a top-k edge
+    cases = [(0.7, 0, 1.0, 0.0), (1.0, 5, 1.0, 0.0), (1.0, 0, 0.8, 0.0), (1.3, 0, 1.0, 0.1), (0.9, 12, 0.9, 0.02),
+             (1.0, 1, 1.0, 0.0), (1.0, 0, 1e-6, 0.0)]
+    for temp, top_k, top_p, min_p in cases:
+        f = lambda x, dt: torch.full((n,), x, dtype=dt).cuda()
+        tokens = hip.sample(row.expand(n, v).contiguous().cuda(), f(temp, torch.float32), f(top_k, torch.int32),
+                            f(top_p, torch.float32), f(min_p, torch.float32), f(1234, torch.int64),
+                            torch.arange(n, dtype=torch.int64).cuda())
+        freq = torch.bincount(tokens.long().cpu(), minlength=v).double() / n
+        p = S.probs(row, temp, top_k, top_p, min_p)
+        assert (freq[p == 0] == 0).all(), (temp, top_k, top_p, min_p, "a filtered token was drawn")
+        assert 0.5 * (freq - p).abs().sum() < 0.02, (temp, top_k, top_p, min_p)
+    # a draw depends on (seed, position) only: not on the row's place in the batch or on the other rows
+    logits = torch.randn(6, v, generator=torch.Generator().manual_seed(1)).cuda()
+    one = lambda x, dt, r: torch.full((r,), x, dtype=dt).cuda()
+    seeds = torch.tensor([100, 101, 102, 103, 100, 101], dtype=torch.int64).cuda()
+    pos = torch.tensor([5, 5, 5, 5, 9, 9], dtype=torch.int64).cuda()
+    together = hip.sample(logits, one(1.0, torch.float32, 6), one(0, torch.int32, 6), one(1.0, torch.float32, 6),
+                          one(0.0, torch.float32, 6), seeds, pos)
+    alone = hip.sample(logits[[1, 5]].contiguous(), one(1.0, torch.float32, 2), one(0, torch.int32, 2),
+                       one(1.0, torch.float32, 2), one(0.0, torch.float32, 2), seeds[[1, 5]].contiguous(),
+                       pos[[1, 5]].contiguous())
+    assert together[[1, 5]].tolist() == alone.tolist()
+    # the draw is the inverse CDF at the hashed uniform, in vocabulary order, at the full vocabulary
+    big = (torch.randn(4, 151_936, generator=g) * 3).cuda()
+    toks = hip.sample(big, one(1.0, torch.float32, 4), one(0, torch.int32, 4), one(1.0, torch.float32, 4),
+                      one(0.0, torch.float32, 4), one(77, torch.int64, 4), torch.arange(4, dtype=torch.int64).cuda())
+    for r in range(4):
+        cdf = big[r].double().softmax(-1).cumsum(0).cpu()
+        u, t = S.uniform(77, r), int(toks[r])
+        assert (cdf[t - 1] if t else 0.0) - 1e-5 <= u < cdf[t] + 1e-5
+    # temperature 0 rows take the argmax beside sampled rows
+    mixed_t = torch.tensor([0.0, 1.0, 0.0, 1.0], dtype=torch.float32).cuda()
+    toks = hip.sample(big, mixed_t, one(0, torch.int32, 4), one(1.0, torch.float32, 4), one(0.0, torch.float32, 4),
+                      one(5, torch.int64, 4), torch.arange(4, dtype=torch.int64).cuda())
+    assert toks[[0, 2]].tolist() == big[[0, 2]].argmax(-1).tolist()
+
+
+def test_kernels_refuse_what_they_do_not_serve(hip):
+    from holon_amd.kernels.hip import KernelError
+    with pytest.raises(KernelError):
+        hip.rmsnorm(torch.zeros(4, 8), torch.ones(8), 1e-6)                         # a CPU tensor: no fallback
+    with pytest.raises(KernelError):
+        hip.rmsnorm(torch.zeros(4, 8, dtype=torch.float16).cuda(), torch.ones(8, dtype=torch.float16).cuda(), 1e-6)
+    q, pages, table, attn = _paged_case([(0, 4)], 2, 1, 12, 16, torch.float32)     # head_dim 12: not a multiple of 8
+    with pytest.raises(KernelError, match="head_dim"):
+        hip.paged_attention(q, pages, table, attn, 16, 1.0, 0)

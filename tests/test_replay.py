@@ -1,0 +1,144 @@
+"""The engine against the plain model, through the step function: the same requests whole, with the last tokens one by
+one, in portions of changing size, and mixed with other requests in a pool so small that pages are used again; in
+float32 and in bfloat16. On the CPU the plain kernel twins stand in for the HIP kernels (this checks the cache, the
+batch layout and the step function); the `gpu` cases run the HIP kernels."""
+from __future__ import annotations
+
+import functools
+
+import pytest
+import torch
+
+from tests import helpers as H
+from tests.plain.ops import TorchKernels
+from tests.plain.qwen3 import PlainQwen3
+
+DEVICES = [pytest.param("cpu", id="cpu-twin"), pytest.param("cuda", marks=pytest.mark.gpu, id="hip")]
+DTYPES = ["float32", "bfloat16"]
+MODELS = {"A": (H.CONFIG_A, 0, 1.0, 16), "B": (H.CONFIG_B, 1, 1.0, 8), "C": (H.CONFIG_C, 2, 1.0, 16),
+          "A-sharp": (H.CONFIG_A, 3, 3.0, 16), "B-sharp": (H.CONFIG_B, 4, 2.5, 8), "C-sharp": (H.CONFIG_C, 5, 3.0, 32)}
+LENGTHS = (40, 70, 33, 90, 50, 64, 21)
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("models")
+    return {name: H.make_folder(root / name, cfg, seed, gain) for name, (cfg, seed, gain, _) in MODELS.items()}
+
+
+@functools.lru_cache(maxsize=None)
+def _plain(folder: str, dtype: str) -> PlainQwen3:
+    return PlainQwen3(folder, getattr(torch, dtype))
+
+
+@functools.lru_cache(maxsize=None)
+def _plain_logits(folder: str, dtype: str, ids: tuple[int, ...]) -> torch.Tensor:
+    return _plain(folder, dtype).logits(list(ids))
+
+
+def _requests(name: str, lengths=LENGTHS) -> dict[str, list[int]]:
+    vocab = MODELS[name][0]["vocab_size"]
+    return {f"r{i}": H.random_ids(n, vocab, 100 + i) for i, n in enumerate(lengths)}
+
+
+def _replayer(folder, name, device, dtype, cache_tokens, max_seqs=4, max_model_len=512):
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    loaded = load_model(folder, device=device, dtype=dtype, kernels=TorchKernels() if device == "cpu" else None,
+                        page_size=MODELS[name][3], max_seqs=max_seqs, max_model_len=max_model_len,
+                        max_step_tokens=max_model_len, cache_tokens=cache_tokens)
+    return Replayer(loaded)
+
+
+def _check(folder, dtype, requests, got, what):
+    want = {r: _plain_logits(str(folder), "float32", tuple(ids)) for r, ids in requests.items()}
+    g, w = H.gather(want, got)
+    if dtype == "float32":
+        H.assert_fp32_close(g, w, what)
+    else:
+        floor = {r: _plain_logits(str(folder), "bfloat16", tuple(ids)) for r, ids in requests.items()}
+        _, f = H.gather(floor, got)
+        H.assert_bf16_close(g, w, f, what)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(MODELS))
+def test_every_way_of_cutting(folders, name, dtype, device):
+    folder, requests = folders[name], _requests(name)
+    page = MODELS[name][3]
+    # whole, one request at a time, in a pool that holds only the longest: pages are used again by each request
+    rep = _replayer(folder, name, device, dtype, cache_tokens=-(-max(LENGTHS) // page) * page)
+    got = H.run_trace(rep, H.trace_whole(requests))
+    assert len(got) == sum(LENGTHS)
+    _check(folder, dtype, requests, got, f"{name} {dtype} whole")
+    rep.cache.check()
+    # most of it in one step, the last 32 tokens one by one
+    for rid in ("r1", "r3"):
+        got = H.run_trace(rep, H.trace_decode_tail(rid, requests[rid], 32))
+        _check(folder, dtype, requests, got, f"{name} {dtype} decode tail {rid}")
+    # portions of changing size, down to two tokens, off the page edges
+    for rid, sizes in (("r3", [7, 2, 13, 3, 2, 30, 5]), ("r1", [2, 2, 17, 16, 1 + page, 2])):
+        got = H.run_trace(rep, H.trace_chunks(rid, requests[rid], sizes))
+        assert len(got) == len(requests[rid])
+        _check(folder, dtype, requests, got, f"{name} {dtype} portions {rid}")
+    rep.cache.check()
+    assert all(g.pool.free == g.pool.usable for g in rep.cache.groups)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C-sharp", "B-sharp"])
+def test_mixed_batches_in_a_tight_pool(folders, name, dtype, device):
+    folder, requests = folders[name], _requests(name)
+    for seed in (0, 1):
+        trace = H.trace_mixed(requests, seed)
+        tokens = H.peak_live_tokens(trace, 64)
+        rep = _replayer(folder, name, device, dtype, cache_tokens=tokens)
+        got = H.run_trace(rep, trace)
+        assert len(got) == sum(LENGTHS)
+        _check(folder, dtype, requests, got, f"{name} {dtype} mixed seed {seed}")
+        rep.cache.check()
+        assert all(g.pool.free == g.pool.usable for g in rep.cache.groups)
+        assert rep.cache.free_slots == rep.cache.max_seqs
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B-sharp"])
+def test_long_decoding_and_first_tokens(folders, name, dtype, device):
+    folder = folders[name]
+    vocab = MODELS[name][0]["vocab_size"]
+    requests = {"long": H.random_ids(300, vocab, 7), "one": H.random_ids(1, vocab, 8), "two": H.random_ids(2, vocab, 9),
+                "three": H.random_ids(3, vocab, 10)}
+    rep = _replayer(folder, name, device, dtype, cache_tokens=320)
+    trace = H.Trace()
+    trace.add([("long", 0, requests["long"][:4], [0, 1, 2, 3])])
+    for p in range(4, 300):                        # 296 single-token steps across many page edges
+        trace.add([("long", p, [requests["long"][p]], [0])], end=["long"] if p == 299 else [])
+    got = H.run_trace(rep, trace)
+    _check(folder, dtype, {"long": requests["long"]}, got, f"{name} {dtype} long decoding")
+    trace = H.Trace()                              # the first tokens of sequences: whole, and one by one from nothing
+    trace.add([("one", 0, requests["one"], [0]), ("two", 0, requests["two"], [0, 1]),
+               ("three", 0, requests["three"][:1], [0])], end=["one", "two"])
+    trace.add([("three", 1, requests["three"][1:2], [0])])
+    trace.add([("three", 2, requests["three"][2:3], [0])], end=["three"])
+    got = H.run_trace(rep, trace)
+    _check(folder, dtype, {k: requests[k] for k in ("one", "two", "three")}, got, f"{name} {dtype} first tokens")
+    rep.cache.check()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_logits_do_not_depend_on_the_cut_in_float32(folders, device):
+    """Beyond the comparison with the plain model: the same position computed whole, in portions and one by one
+    agrees within the same float32 budget as the comparison with the plain model."""
+    folder, name = folders["B-sharp"], "B-sharp"
+    ids = _requests(name)["r3"]
+    rep = _replayer(folder, name, device, "float32", cache_tokens=128)
+    whole = H.run_trace(rep, H.trace_whole({"r3": ids}))
+    parts = H.run_trace(rep, H.trace_chunks("r3", ids, [5, 2, 9, 24, 3]))
+    tail = H.run_trace(rep, H.trace_decode_tail("r3", ids, 40))
+    a = torch.stack([whole[k] for k in sorted(whole)])
+    for other in (parts, tail):
+        b = torch.stack([other[k] for k in sorted(whole)])
+        H.assert_fp32_close(b, a, "cut independence")
