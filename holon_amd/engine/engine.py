@@ -1,0 +1,191 @@
+"""The engine: requests in, tokens out. core/holon/core/engine.py:143-282 (start), :332-376 (`add`), :474-524
+(`generate`, `step`), :603-709 (commit and finishing).
+
+    engine = Engine(EngineConfig(model=folder))
+    rid = engine.add(token_ids, SamplingParams(temperature=0, max_tokens=16))
+    while engine.has_work():
+        for delta in engine.step(): ...
+    engine.generate([ids, ids], params) -> [[token, ...], [token, ...]]
+
+Token ids in, token ids out. One step: the scheduler picks rows, the step function runs them as one batch, the
+sampler draws a token for every row that ended its prompt or decoded, the commit appends tokens and finishes requests.
+"""
+from __future__ import annotations
+
+import itertools
+import secrets
+import sys
+
+import numpy as np
+import torch
+
+from ..cache.pool import OutOfPages
+from ..config.engine import EngineConfig, SamplingParams
+from ..sampling.sampler import Sampler, sequence_seed
+from .batch import StepRow
+from .loading import Loaded, attach_cache, build_from_spec, default_kernels, torch_dtype
+from .request import Seq, Status, TokenDelta
+from .scheduler import Scheduler
+
+
+def activation_bytes(spec, max_step_tokens: int, max_seqs: int, itemsize: int) -> int:
+    """An upper estimate of what one step allocates beside weights and cache: a few copies of the widest activation
+    per token, and float32 logits for the rows that sample."""
+    width = spec.hidden
+    for layer in spec.layers:
+        m, f = layer.mixer.get(), layer.ffn.get()
+        width = max(width, 2 * f.get("inter", 0), (m.get("heads", 0) + 2 * m.get("kv_heads", 0)) * m.get("head_dim", 0))
+    return max_step_tokens * (3 * width + 6 * spec.hidden) * itemsize + 3 * max_seqs * spec.vocab * 4 + (256 << 20)
+
+
+class Engine:
+    def __init__(self, cfg: EngineConfig, kernels=None) -> None:
+        from ..config.model import read_config_json
+        from ..registry import resolve
+        from ..weights.loader import load_weights
+        self.cfg = cfg
+        device, dtype = torch.device(cfg.device), torch_dtype(cfg.dtype)
+        self.device, self.dtype = device, dtype
+        self.kernels = kernels if kernels is not None else default_kernels(device)
+        config_json, generation = read_config_json(cfg.model)
+        self.model_config, self.spec = resolve(config_json, generation)
+        self.eos = set(self.spec.eos_token_ids)
+        shape = dict(page_size=cfg.page_size, max_seqs=cfg.max_seqs, max_model_len=cfg.max_model_len,
+                     max_step_tokens=cfg.max_step_tokens)
+        self.model, _ = build_from_spec(self.spec, device=device, dtype=dtype, kernels=self.kernels, **shape)
+        load_weights(self.model, self.spec, cfg.model, device, dtype)
+        tokens = self._cache_tokens()
+        self.cache, self.runner = attach_cache(self.model, device=device, dtype=dtype, kernels=self.kernels,
+                                               cache_tokens=tokens, **shape)
+        if not self.cache.fits_alone(cfg.max_model_len):
+            raise OutOfPages(f"the cache holds {tokens} tokens, fewer than one request of max_model_len "
+                             f"{cfg.max_model_len}; lower max_model_len or give the cache more memory")
+        self.sampler = Sampler(self.kernels, cfg.max_seqs, device)
+        self.sched = Scheduler(self.cache, cfg.max_step_tokens, cfg.max_model_len, cfg.chunk_with_decode,
+                               on_admit=lambda seq: self.sampler.admit(seq.slot, seq.params))
+        self._ids = itertools.count()
+        self._live: dict[str, Seq] = {}
+        self.steps = 0
+
+    # -- memory accounting ----------------------------------------------------------------------------------------
+    def token_bytes(self) -> int:
+        """Bytes of paged state one token takes over all runs of the model."""
+        item = torch.empty((), dtype=self.dtype).element_size()
+        return sum((d.dtype or self.dtype).itemsize if d.dtype else item * 1 for decls in [[]] for d in decls) + sum(
+            d.elems * (torch.empty((), dtype=d.dtype).element_size() if d.dtype else item)
+            for decls in self.model.state_decls() for d in decls if hasattr(d, "elems"))
+
+    def _cache_tokens(self) -> int:
+        cfg = self.cfg
+        if cfg.cache_tokens is not None:
+            return cfg.cache_tokens
+        per_token = max(1, self.token_bytes())
+        if cfg.state_memory is not None:
+            budget = cfg.state_memory
+        elif self.device.type == "cuda":
+            free, _ = torch.cuda.mem_get_info(self.device)
+            item = torch.empty((), dtype=self.dtype).element_size()
+            budget = int(free * cfg.memory_fraction) - activation_bytes(self.spec, cfg.max_step_tokens, cfg.max_seqs, item)
+            print(f"holon_amd: weights {self.model.nbytes() / 2**30:.2f} GiB, {free / 2**30:.1f} GiB free, "
+                  f"{max(budget, 0) / 2**30:.1f} GiB for the cache ({per_token} B a token)", file=sys.stderr)
+        else:
+            budget = cfg.max_seqs * cfg.max_model_len * per_token
+        tokens = min(budget // per_token, cfg.max_seqs * cfg.max_model_len)
+        return max(int(tokens), 0) // cfg.page_size * cfg.page_size or cfg.page_size
+
+    # -- requests -------------------------------------------------------------------------------------------------
+    def add(self, token_ids: list[int], params: SamplingParams | None = None, rid: str | None = None) -> str:
+        p = params or SamplingParams()
+        p.check()
+        if not token_ids:
+            raise ValueError("empty prompt")
+        if len(token_ids) >= self.cfg.max_model_len:
+            raise ValueError(f"prompt of {len(token_ids)} tokens leaves no room under max_model_len "
+                             f"{self.cfg.max_model_len}")
+        if min(token_ids) < 0 or max(token_ids) >= self.spec.vocab:
+            raise ValueError(f"token ids must lie in [0, {self.spec.vocab})")
+        rid = rid if rid is not None else str(next(self._ids))
+        if rid in self._live:
+            raise ValueError(f"request id {rid!r} is already in flight")
+        seed = p.seed if p.seed is not None else secrets.randbits(63)
+        import dataclasses
+        seq = Seq(rid=rid, tokens=list(token_ids), params=dataclasses.replace(p, seed=sequence_seed(seed, 0)))
+        self._live[rid] = seq
+        self.sched.add(seq)
+        return rid
+
+    def has_work(self) -> bool:
+        return bool(self.sched.waiting or self.sched.running)
+
+    def abort(self, rid: str, reason: str = "abort") -> list[TokenDelta]:
+        seq = self._live.pop(rid, None)
+        if seq is None or seq.status is Status.FINISHED:
+            return []
+        self.sched.finish(seq, reason)
+        return [TokenDelta(rid, [], reason)]
+
+    def stats(self) -> dict[str, int]:
+        return {"waiting": len(self.sched.waiting), "running": len(self.sched.running),
+                "preemptions": self.sched.preemptions, "mixed_steps": self.sched.mixed_steps, "steps": self.steps,
+                "free_pages": min((g.pool.free for g in self.cache.groups), default=0),
+                "graphs": len(getattr(self.runner, "graphs", {}))}
+
+    def close(self) -> None:
+        self._live.clear()
+
+    def generate(self, prompts: list[list[int]], params: SamplingParams | None = None) -> list[list[int]]:
+        """Token ids generated for each prompt."""
+        rids = [self.add(p, params) for p in prompts]
+        out: dict[str, list[int]] = {r: [] for r in rids}
+        pending = set(rids)
+        while pending:
+            for d in self.step():
+                if d.rid in out:
+                    out[d.rid].extend(d.token_ids)
+                    if d.finish_reason:
+                        pending.discard(d.rid)
+        return [out[r] for r in rids]
+
+    # -- one step -------------------------------------------------------------------------------------------------
+    @torch.no_grad()
+    def step(self) -> list[TokenDelta]:
+        rows = self.sched.schedule()
+        if rows is None:
+            if self.has_work():
+                raise RuntimeError("the scheduler made no progress with requests pending")
+            return []
+        step_rows = [StepRow(seq.slot, seq.num_computed, seq.tokens[seq.num_computed: seq.num_computed + n],
+                             [n - 1] if m else []) for seq, n, m in rows]
+        logits = self.runner.run(step_rows)
+        self.steps += 1
+        sampled = [(seq, n) for seq, n, m in rows if m]
+        tokens: list[int] = []
+        if sampled:
+            slots = np.array([seq.slot for seq, _ in sampled], dtype=np.int64)
+            positions = np.array([seq.num_computed + n for seq, n in sampled], dtype=np.int64)
+            tokens = self.sampler.sample(logits, slots, positions).tolist()
+        deltas, at = [], 0
+        for seq, n, m in rows:
+            seq.num_computed += n
+            if not m:
+                continue
+            token = tokens[at]
+            at += 1
+            if seq.status is not Status.RUNNING:
+                self.sched.finished_prefill(seq)
+            seq.tokens.append(token)
+            reason = self._finish_reason(seq, token)
+            if reason:
+                self.sched.finish(seq, reason)
+                self._live.pop(seq.rid, None)
+            deltas.append(TokenDelta(seq.rid, [token], reason))
+        return deltas
+
+    def _finish_reason(self, seq: Seq, token: int) -> str | None:
+        p = seq.params
+        if (token in self.eos and not p.ignore_eos) or token in p.stop_token_ids:
+            return "stop"
+        generated = len(seq.tokens) - seq.prompt_len
+        if (p.max_tokens is not None and generated >= p.max_tokens) or len(seq.tokens) >= self.cfg.max_model_len:
+            return "length"
+        return None

@@ -1,0 +1,40 @@
+"""Requests as the engine tracks them, and what it streams back.
+core/holon/api/batch.py:80-104 (`Seq`), core/holon/api/frontend.py:26-52 (`TokenDelta`)."""
+from __future__ import annotations
+
+import dataclasses
+import enum
+
+from ..config.engine import SamplingParams
+
+
+class Status(enum.Enum):
+    WAITING = "waiting"
+    RUNNING = "running"
+    PREEMPTED = "preempted"
+    FINISHED = "finished"
+
+
+@dataclasses.dataclass(eq=False)
+class Seq:
+    rid: str
+    tokens: list[int]                    # prompt and generated tokens
+    params: SamplingParams
+    prompt_len: int = 0
+    slot: int = -1                       # its row in the cache's tables while admitted
+    num_computed: int = 0                # tokens whose state is in the cache
+    status: Status = Status.WAITING
+    finish_reason: str | None = None
+
+    def __post_init__(self) -> None:
+        if not self.prompt_len:
+            self.prompt_len = len(self.tokens)
+
+
+@dataclasses.dataclass
+class TokenDelta:
+    """New tokens of one request; `finish_reason` ("stop" | "length" | "abort") on its last delta."""
+
+    rid: str
+    token_ids: list[int]
+    finish_reason: str | None = None

@@ -1,0 +1,149 @@
+"""Generation through the entry point (`Engine`), against the plain model: greedy and seeded temperature sampling,
+chunked prompts, mixed steps, preemption, rejections. CPU cases run the plain kernel twins; `gpu` cases the HIP kernels.
+Workloads: the two tiny configurations' own (BASELINE.json configs 0 and 1) and the reference's engine tests
+(plugins/tests/test_engine.py:25-106)."""
+from __future__ import annotations
+
+import pytest
+import torch
+
+from holon_amd.cache import OutOfPages
+from holon_amd.config import EngineConfig, SamplingParams
+from tests import helpers as H
+from tests.plain import sampling as S
+from tests.plain.ops import TorchKernels
+from tests.plain.qwen3 import PlainQwen3
+
+DEVICES = [pytest.param("cpu", id="cpu-twin"), pytest.param("cuda", marks=pytest.mark.gpu, id="hip")]
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("engine-models")
+    return {"A": H.make_folder(root / "A", H.CONFIG_A, 0), "B": H.make_folder(root / "B", H.CONFIG_B, 1, qk_gain=2.0),
+            "Bu": H.make_folder(root / "Bu", H.CONFIG_B, 6, scale=3.0)}
+
+
+def _engine(folder, device, **kw):
+    from holon_amd.engine.engine import Engine
+    kw.setdefault("dtype", "float32")
+    return Engine(EngineConfig(model=str(folder), device=device, **kw),
+                  kernels=TorchKernels() if device == "cpu" else None)
+
+
+def _released(engine):
+    engine.cache.check()
+    return all(g.pool.free == g.pool.usable for g in engine.cache.groups) and \
+        engine.cache.free_slots == engine.cache.max_seqs
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation_is_the_plain_model(folders, device):
+    """Tiny A's workload: 3 requests of 5/17/33 tokens, 16 greedy tokens each, pages of 16."""
+    plain = PlainQwen3(folders["Bu"])
+    prompts = [H.random_ids(n, 384, 40 + n) for n in (5, 17, 33)]
+    engine = _engine(folders["Bu"], device, page_size=16, max_seqs=3, max_model_len=64, max_step_tokens=64)
+    out = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16, ignore_eos=True))
+    assert out == [plain.greedy(p, 16) for p in prompts]
+    assert len({tuple(o) for o in out}) == 3 and all(len(set(o)) > 2 for o in out)   # not a degenerate model
+    assert _released(engine)
+    # the reference's shape: short pages, few slots, a step budget that cuts prompts, requests that wait
+    prompts = [H.random_ids(n, 384, 50 + n) for n in (3, 17, 8, 25)]
+    engine = _engine(folders["Bu"], device, page_size=4, max_seqs=3, max_step_tokens=10, max_model_len=40)
+    out = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    assert out == [plain.greedy(p, 12) for p in prompts]
+    assert _released(engine)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_tied_tiny_model_greedy(folders, device):
+    plain = PlainQwen3(folders["A"])
+    prompts = [H.random_ids(n, 256, n) for n in (5, 17, 33)]
+    engine = _engine(folders["A"], device, page_size=16, max_seqs=4, max_model_len=128)
+    out = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16, ignore_eos=True))
+    assert out == [plain.greedy(p, 16) for p in prompts]
+
+
+def _plain_sampled(plain, prompt, n, seed, temperature, **filters):
+    ids, out = list(prompt), []
+    for _ in range(n):
+        q = S.probs(plain.logits(ids)[-1], temperature, **filters)
+        token = S.draw(q, S.uniform(seed, len(ids)))
+        out.append(token)
+        ids.append(token)
+    return out
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_seeded_sampling_mixed_with_chunked_prompts(folders, device):
+    """Tiny B's workload: prompts of 1/8/31/64 tokens, portions of 16 beside decode tokens, 24 tokens at temperature
+    0.8 with a fixed seed, pages of 8. Every draw is the plain model's law at the plain uniform of (seed, position)."""
+    plain = PlainQwen3(folders["B"])
+    prompts = [H.random_ids(n, 384, 60 + n) for n in (1, 8, 31, 64)]
+    engine = _engine(folders["B"], device, page_size=8, max_seqs=4, max_model_len=96, max_step_tokens=32,
+                     chunk_with_decode=16)
+    params = SamplingParams(temperature=0.8, max_tokens=24, ignore_eos=True, seed=1234)
+    out = engine.generate(prompts, params)
+    assert out == [_plain_sampled(plain, p, 24, 1234, 0.8) for p in prompts]
+    assert engine.stats()["mixed_steps"] > 0
+    assert _released(engine)
+    filtered = SamplingParams(temperature=0.9, top_k=12, top_p=0.9, min_p=0.02, max_tokens=10, ignore_eos=True, seed=7)
+    out = engine.generate(prompts[:2], filtered)
+    assert out == [_plain_sampled(plain, p, 10, 7, 0.9, top_k=12, top_p=0.9, min_p=0.02) for p in prompts[:2]]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_preemption_changes_nothing(folders, device):
+    prompts = [H.random_ids(n, 384, 70 + n) for n in (3, 17, 8, 25)]
+    params = SamplingParams(temperature=1.0, top_k=50, seed=7, max_tokens=12, ignore_eos=True)
+    shape = dict(page_size=4, max_seqs=3, max_step_tokens=10, max_model_len=40)
+    roomy = _engine(folders["Bu"], device, **shape)
+    want = roomy.generate(prompts, params)
+    tight = _engine(folders["Bu"], device, cache_tokens=48, **shape)          # 12 pages
+    assert tight.generate(prompts, params) == want
+    assert tight.stats()["preemptions"] > 0 and roomy.stats()["preemptions"] == 0
+    assert _released(tight)
+    greedy = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
+    assert tight.generate(prompts, greedy) == roomy.generate(prompts, greedy)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_rejections_and_limits(folders, device):
+    engine = _engine(folders["Bu"], device, page_size=4, max_seqs=3, max_step_tokens=10, max_model_len=40)
+    with pytest.raises(ValueError):
+        engine.add([])
+    with pytest.raises(ValueError):
+        engine.add(list(range(40)))
+    with pytest.raises(ValueError):
+        engine.add([1, 2, 384])
+    with pytest.raises(NotImplementedError):
+        engine.add([1, 2], SamplingParams(repetition_penalty=1.1))
+    with pytest.raises(OutOfPages):
+        _engine(folders["Bu"], device, page_size=4, max_seqs=3, max_model_len=40, cache_tokens=36)
+    out = engine.generate([H.random_ids(30, 384, 1)], SamplingParams(temperature=0.0, ignore_eos=True))
+    assert len(out[0]) == 10                                                  # stops at max_model_len
+    # stop tokens and abort
+    first = engine.generate([[5, 6, 7]], SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True))[0]
+    out = engine.generate([[5, 6, 7]], SamplingParams(temperature=0.0, max_tokens=5, stop_token_ids=(first[1],)))
+    assert out[0] == first[: first.index(first[1]) + 1]
+    rid = engine.add([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=50))
+    engine.step()
+    assert [d.finish_reason for d in engine.abort(rid)] == ["abort"]
+    assert not engine.has_work() and _released(engine)
+
+
+@pytest.mark.gpu
+def test_bfloat16_generation_stays_with_the_plain_model(folders):
+    """In bfloat16 a near-tie may flip a token; every token the engine picks must be within the rounding floor of the
+    plain model's best at that place, and the first token of a clear-cut prompt is the plain one."""
+    plain32, plain16 = PlainQwen3(folders["Bu"]), PlainQwen3(folders["Bu"], torch.bfloat16)
+    prompts = [H.random_ids(n, 384, 40 + n) for n in (5, 17, 33)]
+    engine = _engine(folders["Bu"], "cuda", dtype="bfloat16", page_size=16, max_seqs=3, max_model_len=64)
+    out = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16, ignore_eos=True))
+    for prompt, tokens in zip(prompts, out):
+        ids = list(prompt)
+        for t in tokens:
+            want, floor = plain32.logits(ids)[-1], plain16.logits(ids)[-1]
+            margin = 2 * (floor - want).abs().max().item() + 1e-3
+            assert want[t] >= want.max() - 2 * margin
+            ids.append(t)

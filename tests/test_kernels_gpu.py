@@ -34,7 +34,7 @@ def test_rmsnorm_and_add(hip, dtype, shape):
     w = (1 + 0.1 * torch.randn(shape[-1], generator=torch.Generator().manual_seed(3))).to(dtype).cuda()
     x0 = x.clone()
     for eps in (1e-6, 1e-2):
-        got, want = hip.rmsnorm(x, w, eps), PLAIN.rmsnorm(x.float(), w.float(), eps)
+        got, want = hip.rmsnorm(x, w, eps), PLAIN.rmsnorm(x.double(), w.double(), eps)
         assert torch.equal(x, x0), "rmsnorm wrote its input"
         assert H.op_budget_usage(got, want, dtype, shape[-1]) <= 1
     x2, r_hip, r_ref = x.reshape(-1, shape[-1]), r.reshape(-1, shape[-1]).clone(), r.reshape(-1, shape[-1]).clone()
@@ -53,7 +53,7 @@ def test_embedding_and_silu_mul(hip, dtype):
     assert torch.equal(hip.embedding(ids[2:], table), table[ids[2:].long()])
     for t, inter in ((17, 12288), (3, 100), (1, 7)):
         gu = _randn(t, 2 * inter, dtype=dtype, seed=6, scale=3.0)
-        got, want = hip.silu_mul(gu), PLAIN.silu_mul(gu.float())
+        got, want = hip.silu_mul(gu), PLAIN.silu_mul(gu.double())
         assert H.op_budget_usage(got, want, dtype, 1) <= 1
     gu = torch.zeros(2, 8, dtype=dtype).cuda()
     gu[:, 4:] = 1
@@ -122,11 +122,12 @@ def test_paged_attention(hip, dtype, page, geometry):
             rows = [(min(s, 300), n) for s, n in rows]
         q, pages, table, attn = _paged_case(rows, heads, kv_heads, head_dim, page, dtype, seed)
         scale = head_dim ** -0.5
-        want = PLAIN.paged_attention(q.float(), pages.float(), table, attn, page, scale, 0)
+        want = PLAIN.paged_attention(q.double(), pages.double(), table, attn, page, scale, 0)
         got = hip.paged_attention(q, pages, table, attn, page, scale, 0)
         again = hip.paged_attention(q, pages, table, attn, page, scale, 0)
         assert torch.equal(got, again), "two runs differ"
-        assert H.op_budget_usage(got, want, dtype, head_dim) <= 1, (geometry, page, rows)
+        # sums over head_dim (scores) and over the keys (softmax, values)
+        assert H.op_budget_usage(got, want, dtype, head_dim + max(s + n for s, n in rows)) <= 1, (geometry, page, rows)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -135,9 +136,9 @@ def test_paged_attention_window(hip, dtype, window):
     for geometry, page in (((16, 8, 64), 16), ((6, 3, 32), 8), ((32, 8, 128), 16)):
         heads, kv_heads, head_dim = geometry
         q, pages, table, attn = _paged_case(ROWSETS[0] + [(300, 1), (98, 1)], heads, kv_heads, head_dim, page, dtype, 3)
-        want = PLAIN.paged_attention(q.float(), pages.float(), table, attn, page, head_dim ** -0.5, window)
+        want = PLAIN.paged_attention(q.double(), pages.double(), table, attn, page, head_dim ** -0.5, window)
         got = hip.paged_attention(q, pages, table, attn, page, head_dim ** -0.5, window)
-        assert H.op_budget_usage(got, want, dtype, head_dim) <= 1, (geometry, window)
+        assert H.op_budget_usage(got, want, dtype, head_dim + window) <= 1, (geometry, window)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -152,11 +153,11 @@ def test_attention_finds_a_far_key(hip, dtype):
         kp = pages[:, 0].view(-1, kv_heads, page, head_dim)
         for h in range(heads):
             q[0, h] = kp[unit, h // (heads // kv_heads), off].float().mul(4.0).to(dtype)
-        want = PLAIN.paged_attention(q.float(), pages.float(), table, attn, page, head_dim ** -0.5, 0)
+        want = PLAIN.paged_attention(q.double(), pages.double(), table, attn, page, head_dim ** -0.5, 0)
         vp = pages[:, 1].view(-1, kv_heads, head_dim, page)
-        assert (want[0, 0] - vp[unit, 0, :, off].float()).abs().max() < 0.05       # the test itself singles the key out
+        assert (want[0, 0] - vp[unit, 0, :, off].double()).abs().max() < 0.05       # the test itself singles the key out
         got = hip.paged_attention(q, pages, table, attn, page, head_dim ** -0.5, 0)
-        assert H.op_budget_usage(got, want, dtype, head_dim) <= 1, (n, target)
+        assert H.op_budget_usage(got, want, dtype, head_dim + n) <= 1, (n, target)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
