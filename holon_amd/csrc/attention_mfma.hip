@@ -1,0 +1,371 @@
+// Paged causal attention on the matrix cores, bfloat16, for head_dim in {64, 128, 256} and page sizes that are
+// multiples of 16. Two kernels share one tile loop:
+//   * prompt portions: one wave owns NT tiles of 16 (query, head) rows and walks the keys 0 .. its last position;
+//   * decode rows: the keys of a row are split over waves, each writes an unnormalised partial (max, sum, values) and a
+//     second kernel merges the partials in a fixed order.
+//
+// A tile's 16 rows are the G query heads of one kv head at 16/G consecutive positions (grouped-query attention: the
+// heads of a group read the same keys, so each key is loaded once per group, not once per head).
+//
+// Operand layouts (v_mfma_f32_16x16x32_bf16: A is 16x32, B is 32x16, lane l holds 8 consecutive k of row/column l%16
+// starting at 8*(l/16); the 16x16 result has rows 4*(l/16)+r, r<4, of column l%16 in lane l):
+//   S^T = K Q^T: A = 16 keys x 32 dims straight from a key page (keys are rows there), B = Q^T from registers.
+//     Two products cover 32 keys; their rows are permuted (row i of the first is key 8*(i/4) + i%4 of the block, of the
+//     second 4 more) so that lane group g ends up with the scores of keys 8g .. 8g+7 of one query:
+//     exactly the B operand of the next product, with no data movement.
+//   O^T = V^T P^T: A = 16 dims x 32 keys straight from a value page (values are stored transposed inside a page, so the
+//     8 keys a lane needs are one 16-byte load), B = P^T from the registers above, rounded to bfloat16.
+// Softmax is online, float32, in base 2 with log2(e) folded into the scale.
+#include "common.h"
+#include "holon_hip.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x8_t load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8_t*>(p); }
+
+struct AttnArgs {
+  const bf16_t* q;         // [T, Hq, D]
+  bf16_t* out;             // [T, Hq, D]
+  const bf16_t* pages;     // [num_pages, 2, Hkv, P*D]
+  const int32_t* table;    // [slots, table_stride]
+  int table_stride;
+  const int32_t* slots;    // [B]
+  const int32_t* lens;     // [B]
+  const int32_t* qstart;   // [B+1]
+  const int32_t* row_ids;  // rows this launch serves
+  int heads, kv_heads, page_size;
+  float scale_log2;        // scale * log2(e)
+  int window;
+  // decode only
+  float* part_o;           // [n_rows, Hq, splits, D]
+  float* part_ml;          // [n_rows, Hq, splits, 2]
+  int splits, keys_per_split;
+};
+
+// How the 16 rows of a tile map to (position, head) for a group of G heads.
+struct TileMap {
+  int rows_per_pos;   // min(G, 16)
+  int pos_per_tile;   // 16 / rows_per_pos
+  int head_blocks;    // ceil(G / 16)
+};
+__host__ __device__ inline TileMap tile_map(int group) {
+  TileMap m;
+  m.rows_per_pos = group < 16 ? group : 16;
+  m.pos_per_tile = 16 / m.rows_per_pos;
+  m.head_blocks = (group + 15) / 16;
+  return m;
+}
+
+// One wave: NT tiles against keys [key_lo, key_hi] (inclusive, as bounded per row by causality and the window).
+// On return o[t][dsub] holds the unnormalised O^T, m[t] the running max (base-2 scaled), l[t] this lane's share of
+// the sum (to be added over the four lane groups).
+template <int D, int NT>
+__device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __restrict__ trow, int hk,
+                                           const bf16x8_t (&qf)[NT][D / 32], const int (&qpos)[NT],
+                                           const int (&tile_last)[NT], int key_lo, int key_hi,
+                                           f32x4_t (&o)[NT][D / 16], float (&m)[NT], float (&l)[NT]) {
+  const int lane = threadIdx.x % WAVE;
+  const int g = lane / 16, c = lane % 16;
+  const int P = a.page_size;
+  const int64_t plane = (int64_t)P * D;
+  const int64_t page_stride = 2 * (int64_t)a.kv_heads * plane;
+  const bf16_t* kbase = a.pages + (int64_t)hk * plane;
+  const bf16_t* vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
+  const int krow = 8 * (c / 4) + (c % 4);   // this lane's key (row of A) within the 32-key block, first product
+  const int khalf = krow / 16, kin = krow % 16;
+  const int max_page = a.table_stride - 1;
+
+  for (int kb = (key_lo / 32) * 32; kb <= key_hi; kb += 32) {
+    // the two pages this block touches (a block of 32 keys is two groups of 16; a group never straddles a page)
+    const int pi0 = min(kb / P, max_page), pi1 = min((kb + 16) / P, max_page);
+    const int64_t pg0 = (int64_t)trow[pi0] * page_stride, pg1 = (int64_t)trow[pi1] * page_stride;
+    const int off0 = kb % P, off1 = (kb + 16) % P;
+    const bf16_t* krowp = kbase + (khalf ? pg1 : pg0) + (int64_t)((khalf ? off1 : off0) + kin) * D + 8 * g;
+    bf16x8_t kf0[D / 32], kf1[D / 32];
+#pragma unroll
+    for (int ks = 0; ks < D / 32; ++ks) {
+      kf0[ks] = load8(krowp + ks * 32);
+      kf1[ks] = load8(krowp + 4 * D + ks * 32);   // the key 4 further on
+    }
+    // values: lane group g needs keys 8g .. 8g+7 of the block, for dims dsub*16 + c
+    const bf16_t* vrowp = vbase + (g >= 2 ? pg1 : pg0) + (int64_t)c * P + (g >= 2 ? off1 : off0) + 8 * (g % 2);
+    bf16x8_t pb[NT];
+    bool any = false;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if (kb > tile_last[t]) continue;   // every key of the block lies after every query of the tile
+      any = true;
+      f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < D / 32; ++ks) {
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf0[ks], qf[t][ks], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf1[ks], qf[t][ks], s1, 0, 0, 0);
+      }
+      // lane (g, c): s0[r] is key kb+8g+r against query column c, s1[r] key kb+8g+4+r
+      const int qp = qpos[t];
+      const int first = a.window > 0 ? qp - a.window + 1 : 0;
+      float sv[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const int key = kb + 8 * g + r;
+        const float v = (r < 4 ? s0[r] : s1[r - 4]) * a.scale_log2;
+        sv[r] = (key <= qp && key >= first && key >= key_lo && key <= key_hi) ? v : -INFINITY;
+        mx = fmaxf(mx, sv[r]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+      const float m_new = fmaxf(m[t], mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;   // nothing visible yet: keep everything at zero
+      const float alpha = exp2f(m[t] - m_use);
+      m[t] = m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const float p = exp2f(sv[r] - m_use);
+        psum += p;
+        pb[t][r] = (__bf16)p;
+      }
+      l[t] = l[t] * alpha + psum;
+#pragma unroll
+      for (int ds = 0; ds < D / 16; ++ds) o[t][ds] *= alpha;
+    }
+    if (!any) continue;
+#pragma unroll
+    for (int ds = 0; ds < D / 16; ++ds) {
+      const bf16x8_t vf = load8(vrowp + (int64_t)ds * 16 * P);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        if (kb > tile_last[t]) continue;
+        o[t][ds] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[t], o[t][ds], 0, 0, 0);
+      }
+    }
+  }
+}
+
+// Column c of tile (first position index `p0`): which query token, head and position it is, or invalid.
+struct RowRef {
+  bool valid;
+  int token, head, qpos;
+};
+__device__ __forceinline__ RowRef row_ref(const TileMap& tm, int c, int p0, int hb, int hk, int group, int qs, int nq,
+                                          int n) {
+  RowRef r;
+  const int pi = c / tm.rows_per_pos, hi = hb * 16 + c % tm.rows_per_pos;
+  const int qi = p0 + pi;
+  r.valid = pi < tm.pos_per_tile && qi < nq && hi < group;
+  r.token = qs + qi;
+  r.head = hk * group + hi;
+  r.qpos = n - nq + qi;
+  return r;
+}
+
+template <int D, int NT>
+__global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int g = lane / 16, c = lane % 16;
+  const int b = a.row_ids[blockIdx.z];
+  const int group = a.heads / a.kv_heads;
+  const TileMap tm = tile_map(group);
+  const int hk = blockIdx.y / tm.head_blocks, hb = blockIdx.y % tm.head_blocks;
+  const int qs = a.qstart[b], nq = a.qstart[b + 1] - qs, n = a.lens[b];
+  const int p_first = (blockIdx.x * 4 + wave) * NT * tm.pos_per_tile;   // first position index of this wave
+  if (p_first >= nq || n <= 0) return;
+  const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
+
+  bf16x8_t qf[NT][D / 32];
+  int qpos[NT], tile_last[NT];
+  RowRef rr[NT];
+  int key_hi = 0, key_lo = 0x7fffffff;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int p0 = p_first + t * tm.pos_per_tile;
+    rr[t] = row_ref(tm, c, p0, hb, hk, group, qs, nq, n);
+    qpos[t] = rr[t].valid ? rr[t].qpos : -1;   // an unused row sees no key
+    const int last_qi = min(nq, p0 + tm.pos_per_tile) - 1;
+    tile_last[t] = p0 < nq ? n - nq + last_qi : -1;
+    key_hi = max(key_hi, tile_last[t]);
+    if (p0 < nq) key_lo = min(key_lo, a.window > 0 ? max(0, n - nq + p0 - a.window + 1) : 0);
+    const bf16_t* qp = a.q + ((int64_t)rr[t].token * a.heads + rr[t].head) * D + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < D / 32; ++ks) {
+      if (rr[t].valid) {
+        qf[t][ks] = load8(qp + ks * 32);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) qf[t][ks][i] = (__bf16)0.f;
+      }
+    }
+  }
+  f32x4_t o[NT][D / 16];
+  float m[NT], l[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    m[t] = -INFINITY;
+    l[t] = 0.f;
+#pragma unroll
+    for (int ds = 0; ds < D / 16; ++ds) o[t][ds] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  attn_tiles<D, NT>(a, trow, hk, qf, qpos, tile_last, key_lo, key_hi, o, m, l);
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    float lt = l[t];
+    lt += __shfl_xor(lt, 16, WAVE);
+    lt += __shfl_xor(lt, 32, WAVE);
+    if (!rr[t].valid) continue;
+    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    bf16_t* op = a.out + ((int64_t)rr[t].token * a.heads + rr[t].head) * D + 4 * g;
+#pragma unroll
+    for (int ds = 0; ds < D / 16; ++ds) {
+      ushort4 w;
+      w.x = float_to_bf16(o[t][ds][0] * inv);
+      w.y = float_to_bf16(o[t][ds][1] * inv);
+      w.z = float_to_bf16(o[t][ds][2] * inv);
+      w.w = float_to_bf16(o[t][ds][3] * inv);
+      *reinterpret_cast<ushort4*>(op + ds * 16) = w;
+    }
+  }
+}
+
+// Decode rows: block (split, kv head x head block, row), one wave. Partials go to part_o / part_ml.
+template <int D>
+__global__ void __launch_bounds__(64) attn_decode_kernel(AttnArgs a) {
+  const int lane = threadIdx.x % WAVE;
+  const int g = lane / 16, c = lane % 16;
+  const int ri = blockIdx.z;
+  const int b = a.row_ids[ri];
+  const int group = a.heads / a.kv_heads;
+  const TileMap tm = tile_map(group);
+  const int hk = blockIdx.y / tm.head_blocks, hb = blockIdx.y % tm.head_blocks;
+  const int split = blockIdx.x;
+  const int qs = a.qstart[b], nq = a.qstart[b + 1] - qs, n = a.lens[b];
+  const RowRef rr = row_ref(tm, c, 0, hb, hk, group, qs, nq > 0 ? 1 : 0, n);
+  // the keys this row can see, cut into `splits` ranges of keys_per_split
+  const int qp_row = n - 1;
+  const int first = a.window > 0 ? max(0, qp_row - a.window + 1) : 0;
+  const int key_lo = (first / 32) * 32 + split * a.keys_per_split;
+  const int key_hi = min(qp_row, key_lo + a.keys_per_split - 1);
+  float* po = a.part_o + (((int64_t)ri * a.heads + rr.head) * a.splits + split) * D + 4 * g;
+  float* pml = a.part_ml + (((int64_t)ri * a.heads + rr.head) * a.splits + split) * 2;
+  if (n <= 0 || key_lo > key_hi) {   // an empty range: a partial that weighs nothing
+    if (rr.valid && g == 0) { pml[0] = -INFINITY; pml[1] = 0.f; }
+    return;
+  }
+  const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
+  bf16x8_t qf[1][D / 32];
+  const bf16_t* qptr = a.q + ((int64_t)rr.token * a.heads + rr.head) * D + 8 * g;
+#pragma unroll
+  for (int ks = 0; ks < D / 32; ++ks) {
+    if (rr.valid) {
+      qf[0][ks] = load8(qptr + ks * 32);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[0][ks][i] = (__bf16)0.f;
+    }
+  }
+  int qpos[1] = {rr.valid ? qp_row : -1}, tile_last[1] = {qp_row};
+  f32x4_t o[1][D / 16];
+  float m[1] = {-INFINITY}, l[1] = {0.f};
+#pragma unroll
+  for (int ds = 0; ds < D / 16; ++ds) o[0][ds] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  attn_tiles<D, 1>(a, trow, hk, qf, qpos, tile_last, max(key_lo, first), key_hi, o, m, l);
+  float lt = l[0];
+  lt += __shfl_xor(lt, 16, WAVE);
+  lt += __shfl_xor(lt, 32, WAVE);
+  if (!rr.valid) return;
+#pragma unroll
+  for (int ds = 0; ds < D / 16; ++ds) *reinterpret_cast<f32x4_t*>(po + ds * 16) = o[0][ds];
+  if (g == 0) { pml[0] = m[0]; pml[1] = lt; }
+}
+
+// out[row, head, :] = sum_i 2^(m_i - M) o_i / sum_i 2^(m_i - M) l_i, splits in index order.
+__global__ void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                  bf16_t* __restrict__ out, const int32_t* __restrict__ row_ids,
+                                  const int32_t* __restrict__ qstart, int heads, int splits, int head_dim) {
+  const int ri = blockIdx.x, h = blockIdx.y;
+  const int token = qstart[row_ids[ri]];
+  const float* ml = part_ml + ((int64_t)ri * heads + h) * splits * 2;
+  const float* po = part_o + ((int64_t)ri * heads + h) * splits * head_dim;
+  float big = -INFINITY;
+  for (int s = 0; s < splits; ++s) big = fmaxf(big, ml[2 * s]);
+  float denom = 0.f;
+  for (int s = 0; s < splits; ++s) denom += ml[2 * s + 1] > 0.f ? exp2f(ml[2 * s] - big) * ml[2 * s + 1] : 0.f;
+  const float inv = denom > 0.f ? 1.0f / denom : 0.f;
+  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < splits; ++s)
+      if (ml[2 * s + 1] > 0.f) acc += exp2f(ml[2 * s] - big) * po[(int64_t)s * head_dim + d];
+    out[((int64_t)token * heads + h) * head_dim + d] = float_to_bf16(acc * inv);
+  }
+}
+
+static bool mfma_serves(int head_dim, int page_size) {
+  return (head_dim == 64 || head_dim == 128 || head_dim == 256) && page_size % 16 == 0;
+}
+
+extern "C" int holon_attention_mfma_supported(int head_dim, int page_size, int dtype) {
+  return dtype == HOLON_BF16 && mfma_serves(head_dim, page_size);
+}
+
+extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                            int table_stride, const int32_t* slots, const int32_t* lens,
+                                            const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                            int max_query, int heads, int kv_heads, int head_dim, int page_size,
+                                            float scale, int window, void* stream) {
+  HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
+              page_size);
+  HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
+              "attention: bad sizes");
+  if (n_rows <= 0 || max_query <= 0) return 0;
+  AttnArgs a{};
+  a.q = (const bf16_t*)q; a.out = (bf16_t*)out; a.pages = (const bf16_t*)pages; a.table = table;
+  a.table_stride = table_stride; a.slots = slots; a.lens = lens; a.qstart = query_start; a.row_ids = row_ids;
+  a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size;
+  a.scale_log2 = scale * 1.4426950408889634f; a.window = window;
+  const TileMap tm = tile_map(heads / kv_heads);
+  const int nt = head_dim == 256 ? 1 : 2;
+  const int pos_per_block = 4 * nt * tm.pos_per_tile;
+  dim3 grid((max_query + pos_per_block - 1) / pos_per_block, kv_heads * tm.head_blocks, n_rows);
+  hipStream_t s = (hipStream_t)stream;
+  if (head_dim == 64) attn_prefill_kernel<64, 2><<<grid, 256, 0, s>>>(a);
+  else if (head_dim == 128) attn_prefill_kernel<128, 2><<<grid, 256, 0, s>>>(a);
+  else attn_prefill_kernel<256, 1><<<grid, 256, 0, s>>>(a);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_attention_decode_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                           int table_stride, const int32_t* slots, const int32_t* lens,
+                                           const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
+                                           int heads, int kv_heads, int head_dim, int page_size, float scale,
+                                           int window, float* part_o, float* part_ml, int splits, int keys_per_split,
+                                           void* stream) {
+  HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
+              page_size);
+  HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
+              "attention: bad sizes");
+  HOLON_CHECK(splits > 0 && keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml,
+              "attention decode: splits %d of %d keys (a multiple of 32) need a workspace", splits, keys_per_split);
+  const int span = window > 0 ? (window < max_len ? window + 31 : max_len) : max_len;
+  HOLON_CHECK((int64_t)splits * keys_per_split >= span, "attention decode: %d splits of %d keys do not cover %d keys",
+              splits, keys_per_split, span);
+  if (n_rows <= 0) return 0;
+  AttnArgs a{};
+  a.q = (const bf16_t*)q; a.out = (bf16_t*)out; a.pages = (const bf16_t*)pages; a.table = table;
+  a.table_stride = table_stride; a.slots = slots; a.lens = lens; a.qstart = query_start; a.row_ids = row_ids;
+  a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size;
+  a.scale_log2 = scale * 1.4426950408889634f; a.window = window;
+  a.part_o = part_o; a.part_ml = part_ml; a.splits = splits; a.keys_per_split = keys_per_split;
+  const TileMap tm = tile_map(heads / kv_heads);
+  dim3 grid(splits, kv_heads * tm.head_blocks, n_rows);
+  hipStream_t s = (hipStream_t)stream;
+  if (head_dim == 64) attn_decode_kernel<64><<<grid, 64, 0, s>>>(a);
+  else if (head_dim == 128) attn_decode_kernel<128><<<grid, 64, 0, s>>>(a);
+  else attn_decode_kernel<256><<<grid, 64, 0, s>>>(a);
+  HOLON_LAUNCH_OK();
+  dim3 mgrid(n_rows, heads);
+  attn_merge_kernel<<<mgrid, 64, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits, head_dim);
+  HOLON_LAUNCH_OK();
+  return 0;
+}

@@ -30,6 +30,23 @@ int holon_attention_generic(const void* q, void* out, const void* pages, const i
                             const int32_t* slots, const int32_t* lens, const int32_t* query_start, int rows,
                             int tokens, int heads, int kv_heads, int head_dim, int page_size, int num_pages,
                             float scale, int window, int dtype, void* stream);
+// Matrix-core attention (bfloat16, head_dim 64/128/256, page_size % 16 == 0). `row_ids` lists the rows served.
+int holon_attention_mfma_supported(int head_dim, int page_size, int dtype);
+int holon_attention_prefill_bf16(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
+                                 const int32_t* slots, const int32_t* lens, const int32_t* query_start,
+                                 const int32_t* row_ids, int n_rows, int max_query, int heads, int kv_heads,
+                                 int head_dim, int page_size, float scale, int window, void* stream);
+// One query token per row; the keys are split over `splits` waves of `keys_per_split` keys (a multiple of 32) whose
+// partial results (part_o [n_rows, heads, splits, head_dim], part_ml [n_rows, heads, splits, 2], float32) are merged
+// in split order.
+int holon_attention_decode_bf16(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
+                                const int32_t* slots, const int32_t* lens, const int32_t* query_start,
+                                const int32_t* row_ids, int n_rows, int max_len, int heads, int kv_heads, int head_dim,
+                                int page_size, float scale, int window, float* part_o, float* part_ml, int splits,
+                                int keys_per_split, void* stream);
+// y[M, N] = x[M, K] w[N, K]^T for M <= 64 rows, bfloat16 in, float32 accumulation; out_f32 picks the output type.
+int holon_gemm_skinny_supported(int M, int N, int K);
+int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_f32, void* stream);
 int holon_argmax(const float* logits, int32_t* out, int rows, int vocab, void* stream);
 int holon_sample(const float* logits, int32_t* out, int rows, int vocab, const float* temperature,
                  const int32_t* top_k, const float* top_p, const float* min_p, const int64_t* seeds,

@@ -60,6 +60,12 @@ class HipKernels:
                                          _I, _P],
             "holon_kv_write": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
             "holon_attention_generic": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+            "holon_attention_mfma_supported": [_I, _I, _I],
+            "holon_attention_prefill_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+            "holon_attention_decode_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P,
+                                            _I, _I, _P],
+            "holon_gemm_skinny_supported": [_I, _I, _I],
+            "holon_gemm_skinny_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
             "holon_argmax": [_P, _P, _I, _I, _P],
             "holon_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
         }
@@ -123,7 +129,20 @@ class HipKernels:
                    x.numel() // dim, dim, float(eps), self._dt(x, "add_rmsnorm"), self._stream())
         return y
 
+    skinny_rows = 16          # up to this many rows the hand-written weight-streaming product runs
+
     def linear(self, x, weight, out_dtype=None):
+        m, k = x.shape
+        n = weight.shape[0]
+        if weight.shape[1] != k:
+            raise KernelError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(weight.shape)}")
+        if (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows and k >= 256
+                and x.is_contiguous() and weight.is_contiguous() and self.lib.holon_gemm_skinny_supported(m, n, k)):
+            to_f32 = out_dtype == torch.float32
+            y = torch.empty((m, n), dtype=torch.float32 if to_f32 else torch.bfloat16, device=x.device)
+            self._call(self.lib.holon_gemm_skinny_bf16, x.data_ptr(), weight.data_ptr(), y.data_ptr(), m, n, k,
+                       int(to_f32), self._stream())
+            return y
         # the vendor library's product, float32 accumulation (no reduced-precision mode for float32 operands)
         y = torch.matmul(x, weight.t())
         return y if out_dtype in (None, y.dtype) else y.to(out_dtype)
@@ -196,11 +215,35 @@ class HipKernels:
             raise KernelError(f"attention: pages {tuple(pages.shape)} do not fit head_dim {d}, page {page_size}")
         out = torch.empty_like(q)
         b = rows.slots.shape[0]
+        if self.lib.holon_attention_mfma_supported(d, page_size, self._dt(q, "attention")):
+            common = (q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(), table.shape[1],
+                      rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr())
+            if rows.n_chunk:
+                self._call(self.lib.holon_attention_prefill_bf16, *common, rows.chunk_rows.data_ptr(), rows.n_chunk,
+                           rows.max_chunk_query, hq, hkv, d, page_size, float(scale), int(window), self._stream())
+            if rows.n_decode:
+                span = rows.max_decode_len if not window else min(rows.max_decode_len, window + 31)
+                splits, per = self.decode_splits(rows.n_decode * hkv * ((hq // hkv + 15) // 16), span)
+                part_o = torch.empty((rows.n_decode * hq * splits * d,), dtype=torch.float32, device=q.device)
+                part_ml = torch.empty((rows.n_decode * hq * splits * 2,), dtype=torch.float32, device=q.device)
+                self._call(self.lib.holon_attention_decode_bf16, *common, rows.decode_rows.data_ptr(), rows.n_decode,
+                           rows.max_decode_len, hq, hkv, d, page_size, float(scale), int(window), part_o.data_ptr(),
+                           part_ml.data_ptr(), splits, per, self._stream())
+            return out
         self._call(self.lib.holon_attention_generic, q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(),
                    table.shape[1], rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr(), b, t, hq,
                    hkv, d, page_size, pages.shape[0], float(scale), int(window), self._dt(q, "attention"),
                    self._stream())
         return out
+
+    @staticmethod
+    def decode_splits(waves_per_split: int, span: int, target_waves: int = 2048, min_keys: int = 64) -> tuple[int, int]:
+        """How a decode row's keys are cut over waves: (splits, keys per split, a multiple of 32), enough waves to
+        fill the GPU but at least `min_keys` keys each."""
+        want = max(1, min(64, target_waves // max(1, waves_per_split)))
+        per = max(min_keys, -(-span // want))
+        per = -(-per // 32) * 32
+        return max(1, -(-span // per)), per
 
     def argmax(self, logits):
         self._check(logits, "argmax logits", torch.float32)

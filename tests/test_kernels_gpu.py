@@ -86,6 +86,7 @@ def _paged_case(rows, heads, kv_heads, head_dim, page, dtype, seed=0, max_seqs=8
     """rows: (tokens before this step, tokens this step). A shuffled block table with spare pages."""
     g = torch.Generator().manual_seed(seed)
     rng = np.random.default_rng(seed)
+    assert len(rows) <= max_seqs
     slots = rng.permutation(max_seqs)[: len(rows)].astype(np.int32)
     max_pages = -(-max(s + n for s, n in rows) // page)
     units = max_seqs * max_pages + 7
@@ -135,7 +136,8 @@ def test_paged_attention(hip, dtype, page, geometry):
 def test_paged_attention_window(hip, dtype, window):
     for geometry, page in (((16, 8, 64), 16), ((6, 3, 32), 8), ((32, 8, 128), 16)):
         heads, kv_heads, head_dim = geometry
-        q, pages, table, attn = _paged_case(ROWSETS[0] + [(300, 1), (98, 1)], heads, kv_heads, head_dim, page, dtype, 3)
+        q, pages, table, attn = _paged_case(ROWSETS[0] + [(300, 1), (98, 1)], heads, kv_heads, head_dim, page, dtype, 3,
+                                            max_seqs=12)
         want = PLAIN.paged_attention(q.double(), pages.double(), table, attn, page, head_dim ** -0.5, window)
         got = hip.paged_attention(q, pages, table, attn, page, head_dim ** -0.5, window)
         assert H.op_budget_usage(got, want, dtype, head_dim + window) <= 1, (geometry, window)
@@ -197,8 +199,11 @@ def test_fused_norm_rope_write_is_the_three_ops(hip, dtype, geometry):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_linear(hip, dtype):
-    for t, k, n in ((1, 4096, 6144), (8, 4096, 1000), (17, 100, 333), (64, 12288, 4096), (300, 120, 1000), (2, 96, 384)):
+def test_linear(hip, dtype, monkeypatch):
+    monkeypatch.setattr(hip, "skinny_rows", 64)       # the few-row kernel at every row count it is built for
+    for t, k, n in ((1, 4096, 6144), (8, 4096, 1000), (17, 100, 333), (64, 12288, 4096), (300, 120, 1000), (2, 96, 384),
+                    (1, 4096, 4096), (16, 12288, 4096), (3, 4096, 24576), (9, 512, 208), (33, 1024, 4096),
+                    (48, 4096, 512), (5, 12288, 151936 // 8), (65, 4096, 512)):
         x, w = _randn(t, k, dtype=dtype, seed=13), _randn(n, k, dtype=dtype, seed=14, scale=0.05)
         want = x.double() @ w.double().T
         got = hip.linear(x, w)
@@ -209,8 +214,9 @@ def test_linear(hip, dtype):
     # order of summation gives the same bits (plugins/tests/test_attention_kv_quant.py:244-261)
     g = torch.Generator().manual_seed(15)
     x = torch.randint(-1, 2, (5, 512), generator=g).to(dtype).cuda()
-    w = (torch.randint(-1, 2, (200, 512), generator=g).float() / 8).to(dtype).cuda()
-    assert torch.equal(hip.linear(x, w).float(), x.float() @ w.float().T)
+    for n in (200, 208, 4096):
+        w = (torch.randint(-1, 2, (n, 512), generator=g).float() / 8).to(dtype).cuda()
+        assert torch.equal(hip.linear(x, w).float(), x.float() @ w.float().T)
     # a row's result does not depend on the rows beside it, beyond rounding
     x = _randn(64, 4096, dtype=dtype, seed=16)
     w = _randn(512, 4096, dtype=dtype, seed=17, scale=0.02)
