@@ -39,21 +39,25 @@ def activation_bytes(spec, max_step_tokens: int, max_seqs: int, itemsize: int) -
 
 
 class Engine:
-    def __init__(self, cfg: EngineConfig, kernels=None) -> None:
+    def __init__(self, cfg: EngineConfig, kernels=None, *, random_config: dict | None = None, seed: int = 0) -> None:
         from ..config.model import read_config_json
         from ..registry import resolve
         from ..weights.loader import load_weights
+        from ..weights.random_init import fill_random
         self.cfg = cfg
         device, dtype = torch.device(cfg.device), torch_dtype(cfg.dtype)
         self.device, self.dtype = device, dtype
         self.kernels = kernels if kernels is not None else default_kernels(device)
-        config_json, generation = read_config_json(cfg.model)
+        config_json, generation = (random_config, None) if random_config is not None else read_config_json(cfg.model)
         self.model_config, self.spec = resolve(config_json, generation)
         self.eos = set(self.spec.eos_token_ids)
         shape = dict(page_size=cfg.page_size, max_seqs=cfg.max_seqs, max_model_len=cfg.max_model_len,
                      max_step_tokens=cfg.max_step_tokens)
         self.model, _ = build_from_spec(self.spec, device=device, dtype=dtype, kernels=self.kernels, **shape)
-        load_weights(self.model, self.spec, cfg.model, device, dtype)
+        if random_config is not None:
+            fill_random(self.model, self.spec, seed, device, dtype)
+        else:
+            load_weights(self.model, self.spec, cfg.model, device, dtype)
         tokens = self._cache_tokens()
         self.cache, self.runner = attach_cache(self.model, device=device, dtype=dtype, kernels=self.kernels,
                                                cache_tokens=tokens, **shape)
@@ -67,13 +71,17 @@ class Engine:
         self._live: dict[str, Seq] = {}
         self.steps = 0
 
+    @classmethod
+    def from_random(cls, config_json: dict, seed: int, cfg: EngineConfig, kernels=None) -> "Engine":
+        """An engine over random weights drawn on the device from a config.json dict (no folder is read)."""
+        return cls(cfg, kernels, random_config=config_json, seed=seed)
+
     # -- memory accounting ----------------------------------------------------------------------------------------
     def token_bytes(self) -> int:
         """Bytes of paged state one token takes over all runs of the model."""
         item = torch.empty((), dtype=self.dtype).element_size()
-        return sum((d.dtype or self.dtype).itemsize if d.dtype else item * 1 for decls in [[]] for d in decls) + sum(
-            d.elems * (torch.empty((), dtype=d.dtype).element_size() if d.dtype else item)
-            for decls in self.model.state_decls() for d in decls if hasattr(d, "elems"))
+        return sum(d.elems * (torch.empty((), dtype=d.dtype).element_size() if d.dtype else item)
+                   for decls in self.model.state_decls() for d in decls if hasattr(d, "elems"))
 
     def _cache_tokens(self) -> int:
         cfg = self.cfg
