@@ -60,7 +60,7 @@ class Engine:
             load_weights(self.model, self.spec, cfg.model, device, dtype)
         tokens = self._cache_tokens()
         self.cache, self.runner = attach_cache(self.model, device=device, dtype=dtype, kernels=self.kernels,
-                                               cache_tokens=tokens, **shape)
+                                               cache_tokens=tokens, graphs=cfg.graphs, **shape)
         if not self.cache.fits_alone(cfg.max_model_len):
             raise OutOfPages(f"the cache holds {tokens} tokens, fewer than one request of max_model_len "
                              f"{cfg.max_model_len}; lower max_model_len or give the cache more memory")

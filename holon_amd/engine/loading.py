@@ -58,16 +58,18 @@ def build_from_spec(spec: ModelSpec, *, device: torch.device, dtype: torch.dtype
 
 
 def attach_cache(model: Model, *, device: torch.device, dtype: torch.dtype, kernels, page_size: int, max_seqs: int,
-                 max_model_len: int, max_step_tokens: int, cache_tokens: int) -> tuple[CacheManager, StepRunner]:
+                 max_model_len: int, max_step_tokens: int, cache_tokens: int, graphs: bool = False
+                 ) -> tuple[CacheManager, StepRunner]:
     cache = CacheManager(model.sites, model.state_decls(), page_size=page_size, max_seqs=max_seqs,
                          max_model_len=max_model_len, tokens=cache_tokens, device=device, dtype=dtype)
-    runner = StepRunner(model, cache, kernels, device, max_step_tokens=max_step_tokens, max_seqs=max_seqs)
+    runner = StepRunner(model, cache, kernels, device, max_step_tokens=max_step_tokens, max_seqs=max_seqs,
+                        graphs=graphs)
     return cache, runner
 
 
 def load_model(folder: str | pathlib.Path, *, device: str | torch.device = "cuda", dtype: str | torch.dtype = "bfloat16",
                kernels=None, page_size: int = 16, max_seqs: int = 64, max_model_len: int = 8192,
-               max_step_tokens: int = 4096, cache_tokens: int | None = None) -> Loaded:
+               max_step_tokens: int = 4096, cache_tokens: int | None = None, graphs: bool = False) -> Loaded:
     """Read config.json, pick the model by its architecture name, load the weights, allocate the cache."""
     device, dtype = torch.device(device), torch_dtype(dtype)
     kernels = kernels if kernels is not None else default_kernels(device)
@@ -79,5 +81,5 @@ def load_model(folder: str | pathlib.Path, *, device: str | torch.device = "cuda
     tokens = cache_tokens if cache_tokens is not None else max_model_len
     cache, runner = attach_cache(model, device=device, dtype=dtype, kernels=kernels, page_size=page_size,
                                  max_seqs=max_seqs, max_model_len=max_model_len, max_step_tokens=max_step_tokens,
-                                 cache_tokens=tokens)
+                                 cache_tokens=tokens, graphs=graphs)
     return Loaded(cfg, spec, model, cache, runner, kernels, device, dtype)

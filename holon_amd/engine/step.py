@@ -2,9 +2,16 @@
 
 It runs only the tokens it is given, as one flat batch, against the cache that earlier steps left: portions of
 prompts beside single decoded tokens, cut anywhere. core/holon/core/executor.py:357-430 (`Executor.launch`), :497-564
-(host half of the inputs), :460-470 (logits only where wanted).
+(host half of the inputs), :460-470 (logits only where wanted), :316-354 (graphs for decode steps).
+
+Decode-only steps (one token a row, every row sampled) may be replayed from a HIP graph: rows are padded to a
+batch-size bucket with rows on the padding slot (whose block-table row is all null pages, so they read and write only
+the null page), inputs are copied into buffers of fixed address, and the captured launch sequence is replayed. The
+first step of a bucket runs eagerly on those buffers, the second captures, later ones replay.
 """
 from __future__ import annotations
+
+import dataclasses
 
 import numpy as np
 import torch
@@ -14,34 +21,83 @@ from ..kernels.api import AttnRows
 from ..model import Model
 from .batch import PagedView, Step, StepRow
 
+BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256)    # core/holon/core/executor.py:28
+LEN_BUCKET_MIN = 1024
+
+
+@dataclasses.dataclass
+class _Graph:
+    arena: torch.Tensor                           # int32 inputs at a fixed address
+    step: Step
+    logits: torch.Tensor | None = None
+    graph: torch.cuda.CUDAGraph | None = None
+    runs: int = 0
+
 
 class StepRunner:
     def __init__(self, model: Model, cache: CacheManager, kernels, device: torch.device, *, max_step_tokens: int,
-                 max_seqs: int) -> None:
+                 max_seqs: int, graphs: bool = False) -> None:
         self.model, self.cache, self.kernels, self.device = model, cache, kernels, device
         self.max_step_tokens, self.max_seqs = max_step_tokens, max_seqs
         self.vocab = model.spec.vocab
         self.steps = 0
         self.pinned = device.type == "cuda"
+        self.use_graphs = graphs and device.type == "cuda"
+        self.graphs: dict[tuple[int, int], _Graph] = {}
+        self.graph_replays = 0
 
     # -- inputs ---------------------------------------------------------------------------------------------------
-    def _upload(self, arrays: list[np.ndarray]) -> list[torch.Tensor]:
-        """Several int32 arrays to the device in one copy."""
+    def _arrays(self, slots: np.ndarray, starts: np.ndarray, counts: np.ndarray, tokens: np.ndarray
+                ) -> tuple[list[np.ndarray], dict]:
+        """The int32 arrays of a step, in a fixed order, and the host-side facts about them."""
+        cache = self.cache
+        total = int(counts.sum())
+        qstart = np.concatenate(([0], np.cumsum(counts)))
+        token_row = np.repeat(np.arange(len(slots)), counts)
+        positions = np.repeat(starts, counts) + (np.arange(total) - np.repeat(qstart[:-1], counts))
+        lens = starts + counts
+        decode = np.flatnonzero(counts == 1)
+        chunk = np.flatnonzero(counts > 1)
+        arrays = [tokens, positions, token_row, slots, starts, lens, qstart, decode, chunk]
+        for g in cache.groups:
+            page, off = cache.write_targets(g.gid, slots[token_row], positions)
+            arrays += [page, off]
+        facts = dict(total=total, n_rows=len(slots), n_decode=len(decode), n_chunk=len(chunk),
+                     max_decode_len=int(lens[decode].max()) if len(decode) else 0,
+                     max_chunk_query=int(counts[chunk].max()) if len(chunk) else 0,
+                     max_chunk_len=int(lens[chunk].max()) if len(chunk) else 0)
+        return arrays, facts
+
+    def _to_device(self, arrays: list[np.ndarray], arena: torch.Tensor | None = None) -> list[torch.Tensor]:
+        """Several int32 arrays to the device in one copy (into `arena`, a buffer of fixed address, when given)."""
         sizes = [a.size for a in arrays]
-        flat = np.concatenate([a.astype(np.int32, copy=False).ravel() for a in arrays]) if arrays else np.zeros(0, np.int32)
+        flat = np.concatenate([a.astype(np.int32, copy=False).ravel() for a in arrays])
         host = torch.from_numpy(flat)
         if self.pinned:
             host = host.pin_memory()
-        dev = host.to(self.device, non_blocking=True)
+        if arena is None:
+            dev = host.to(self.device, non_blocking=True)
+        else:
+            dev = arena[: flat.size]
+            dev.copy_(host, non_blocking=True)
         out, at = [], 0
         for n in sizes:
             out.append(dev[at: at + n])
             at += n
         return out
 
-    def prepare(self, rows: list[StepRow]) -> tuple[Step, np.ndarray]:
-        """Device inputs of a step, and the flat indices of the tokens whose logits are wanted (in row order, then in
-        the order of each row's `want`)."""
+    def _step(self, dev: list[torch.Tensor], facts: dict, slots, starts, counts) -> Step:
+        cache = self.cache
+        paged = {g.gid: PagedView(cache.page_size, g.table_dev, dev[9 + 2 * i], dev[10 + 2 * i])
+                 for i, g in enumerate(cache.groups)}
+        attn = AttnRows(slots=dev[3], lens=dev[5], query_start=dev[6], decode_rows=dev[7], chunk_rows=dev[8],
+                        n_decode=facts["n_decode"], n_chunk=facts["n_chunk"], max_decode_len=facts["max_decode_len"],
+                        max_chunk_query=facts["max_chunk_query"], max_chunk_len=facts["max_chunk_len"])
+        return Step(kernels=self.kernels, n_tokens=facts["total"], n_rows=facts["n_rows"], token_ids=dev[0],
+                    positions=dev[1], token_row=dev[2], slots=dev[3], starts=dev[4], rows=attn, paged=paged,
+                    h_slots=slots, h_starts=starts, h_counts=counts)
+
+    def _check(self, rows: list[StepRow]) -> tuple[np.ndarray, np.ndarray, np.ndarray, np.ndarray, np.ndarray]:
         if not rows:
             raise ValueError("a step needs at least one row")
         cache = self.cache
@@ -60,56 +116,85 @@ class StepRunner:
                 raise ValueError(f"slot {r.slot}: the row starts at {r.start}, the cache holds {cache.computed[r.slot]}")
             if r.start + n > cache.capacity(r.slot):
                 raise RuntimeError(f"slot {r.slot}: no pages reserved for tokens up to {r.start + n}")
-        qstart = np.concatenate(([0], np.cumsum(counts)))
-        token_row = np.repeat(np.arange(len(rows)), counts)
-        positions = np.repeat(starts, counts) + (np.arange(total) - np.repeat(qstart[:-1], counts))
         tokens = np.concatenate([np.asarray(r.tokens, dtype=np.int64) for r in rows])
         if tokens.min() < 0 or tokens.max() >= self.vocab:
             raise ValueError(f"token ids must lie in [0, {self.vocab})")
-        lens = starts + counts
-        decode = np.flatnonzero(counts == 1)
-        chunk = np.flatnonzero(counts > 1)
+        qstart = np.concatenate(([0], np.cumsum(counts)))
         wanted = []
         for b, r in enumerate(rows):
             for w in r.want:
                 if not 0 <= w < counts[b]:
                     raise ValueError(f"row {b}: wanted place {w} is not among its {counts[b]} tokens")
                 wanted.append(qstart[b] + w)
-        cache.upload()
-        arrays = [tokens, positions, token_row, slots, starts, lens, qstart, decode, chunk]
-        for g in cache.groups:
-            page, off = cache.write_targets(g.gid, slots[token_row], positions)
-            arrays += [page, off]
-        dev = self._upload(arrays)
-        paged = {g.gid: PagedView(cache.page_size, g.table_dev, dev[9 + 2 * i], dev[10 + 2 * i])
-                 for i, g in enumerate(cache.groups)}
-        attn = AttnRows(slots=dev[3], lens=dev[5], query_start=dev[6], decode_rows=dev[7], chunk_rows=dev[8],
-                        n_decode=len(decode), n_chunk=len(chunk),
-                        max_decode_len=int(lens[decode].max()) if len(decode) else 0,
-                        max_chunk_query=int(counts[chunk].max()) if len(chunk) else 0,
-                        max_chunk_len=int(lens[chunk].max()) if len(chunk) else 0)
-        step = Step(kernels=self.kernels, n_tokens=total, n_rows=len(rows), token_ids=dev[0], positions=dev[1],
-                    token_row=dev[2], slots=dev[3], starts=dev[4], rows=attn, paged=paged,
-                    h_slots=slots, h_starts=starts, h_counts=counts)
-        return step, np.asarray(wanted, dtype=np.int64)
+        return slots, starts, counts, tokens, np.asarray(wanted, dtype=np.int64)
+
+    def prepare(self, rows: list[StepRow]) -> tuple[Step, np.ndarray]:
+        """Device inputs of a step, and the flat indices of the tokens whose logits are wanted (in row order, then in
+        the order of each row's `want`)."""
+        slots, starts, counts, tokens, wanted = self._check(rows)
+        self.cache.upload()
+        arrays, facts = self._arrays(slots, starts, counts, tokens)
+        return self._step(self._to_device(arrays), facts, slots, starts, counts), wanted
 
     # -- the step -------------------------------------------------------------------------------------------------
+    def _forward(self, step: Step, wanted: np.ndarray | None) -> torch.Tensor | None:
+        """The model on a step; `wanted` None: logits of every token."""
+        h, delta = self.model.trunk(step)
+        if wanted is not None and not len(wanted):
+            return None
+        if wanted is None or (len(wanted) == step.n_tokens and (wanted == np.arange(step.n_tokens)).all()):
+            return self.model.head(h, delta)
+        idx = torch.from_numpy(wanted).to(self.device)
+        return self.model.head(h.index_select(0, idx), delta.index_select(0, idx) if delta is not None else None)
+
     @torch.no_grad()
     def run(self, rows: list[StepRow]) -> torch.Tensor | None:
         """Run the rows' tokens through the model; returns float32 logits [wanted, vocab] (None when nothing is
         wanted: then the head does not run). Afterwards the cache holds the rows' tokens."""
-        step, wanted = self.prepare(rows)
-        h, delta = self.model.trunk(step)
-        logits = None
-        if len(wanted):
-            if len(wanted) == step.n_tokens and (wanted == np.arange(step.n_tokens)).all():
-                rows_h, rows_d = h, delta
-            else:
-                idx = torch.from_numpy(wanted).to(self.device)
-                rows_h = h.index_select(0, idx)
-                rows_d = delta.index_select(0, idx) if delta is not None else None
-            logits = self.model.head(rows_h, rows_d)
-        for r, n in zip(rows, step.h_counts):
-            self.cache.advance(r.slot, r.start + int(n))
+        if self.use_graphs and len(rows) <= BUCKETS[-1] and all(len(r.tokens) == 1 and r.want == [0] for r in rows):
+            logits = self._run_graphed(rows)
+        else:
+            step, wanted = self.prepare(rows)
+            logits = self._forward(step, wanted)
+        for r in rows:
+            self.cache.advance(r.slot, r.start + len(r.tokens))
         self.steps += 1
         return logits
+
+    # -- graphs ---------------------------------------------------------------------------------------------------
+    def _run_graphed(self, rows: list[StepRow]) -> torch.Tensor:
+        slots, starts, counts, tokens, _ = self._check(rows)
+        n = len(rows)
+        bucket = next(b for b in BUCKETS if b >= n)
+        longest = int((starts + counts).max())
+        len_bucket = max(LEN_BUCKET_MIN, 1 << (longest - 1).bit_length())
+        pad = bucket - n
+        if pad:                                    # rows on the padding slot: one token at position 0 of the null page
+            slots = np.concatenate((slots, np.full(pad, self.cache.padding_slot, dtype=np.int64)))
+            starts = np.concatenate((starts, np.zeros(pad, dtype=np.int64)))
+            counts = np.concatenate((counts, np.ones(pad, dtype=np.int64)))
+            tokens = np.concatenate((tokens, np.zeros(pad, dtype=np.int64)))
+        self.cache.upload()
+        arrays, facts = self._arrays(slots, starts, counts, tokens)
+        facts["max_decode_len"] = len_bucket       # launch shapes are the bucket's, whatever the rows' lengths
+        key = (bucket, len_bucket)
+        g = self.graphs.get(key)
+        if g is None:
+            size = sum(a.size for a in arrays)
+            arena = torch.zeros(size, dtype=torch.int32, device=self.device)
+            g = _Graph(arena=arena, step=self._step(self._to_device(arrays, arena), facts, slots, starts, counts))
+            self.graphs[key] = g
+        else:
+            self._to_device(arrays, g.arena)
+        g.runs += 1
+        if g.graph is None and g.runs == 1:        # the first step of a bucket: eagerly, on the fixed buffers
+            return self._forward(g.step, None)[:n]
+        if g.graph is None:
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                g.logits = self._forward(g.step, None)
+            g.graph = graph
+        g.graph.replay()
+        self.graph_replays += 1
+        return g.logits[:n]

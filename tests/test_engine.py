@@ -147,3 +147,27 @@ def test_bfloat16_generation_stays_with_the_plain_model(folders):
             margin = 2 * (floor - want).abs().max().item() + 1e-3
             assert want[t] >= want.max() - 2 * margin
             ids.append(t)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(folders, dtype):
+    """Decode steps replayed from HIP graphs give the tokens of eager steps, over many replays with the program's own
+    eager work (prompt steps, sampling, host synchronisation) between them, while the batch shrinks through the
+    buckets and pages are taken and given back."""
+    prompts = [H.random_ids(n, 384, 80 + n) for n in (3, 17, 8, 25, 40, 1)]
+    shape = dict(dtype=dtype, page_size=8, max_seqs=6, max_model_len=128, max_step_tokens=64)
+    outs = {}
+    for graphs in (False, True):
+        engine = _engine(folders["Bu"], "cuda", graphs=graphs, **shape)
+        rids = [engine.add(p, SamplingParams(temperature=0.0 if i % 2 else 0.7, seed=5, max_tokens=20 + 7 * i,
+                                             ignore_eos=True)) for i, p in enumerate(prompts)]
+        got = {r: [] for r in rids}
+        while engine.has_work():
+            for d in engine.step():
+                got[d.rid].extend(d.token_ids)
+        outs[graphs] = [got[r] for r in rids]
+        assert _released(engine)
+        if graphs:
+            assert engine.runner.graph_replays > 20 and len(engine.runner.graphs) >= 3
+    assert outs[True] == outs[False]
