@@ -1,0 +1,148 @@
+"""The scheduler's decisions, on the real cache manager without a model (no GPU): what a step holds, the token
+budget, first come first served, what happens when pages run out. core/tests/test_sched.py:13-197 is the model."""
+from __future__ import annotations
+
+import random
+
+import pytest
+import torch
+
+from holon_amd.cache import CacheManager
+from holon_amd.config import SamplingParams
+from holon_amd.engine.request import Seq, Status
+from holon_amd.engine.scheduler import Scheduler
+from holon_amd.model import Site
+from holon_amd.parts.base import PagedState
+
+
+def _sched(tokens=64, page=4, max_seqs=4, max_model_len=32, max_step_tokens=16, chunk_with_decode=0):
+    cache = CacheManager([Site(run=0, layer=0)], [[PagedState("kv", 2)]], page_size=page, max_seqs=max_seqs,
+                         max_model_len=max_model_len, tokens=tokens, device=torch.device("cpu"), dtype=torch.float32)
+    return Scheduler(cache, max_step_tokens, max_model_len, chunk_with_decode), cache
+
+
+def _seq(rid, n, max_tokens=8):
+    return Seq(rid=str(rid), tokens=list(range(n)), params=SamplingParams(temperature=0.0, max_tokens=max_tokens))
+
+
+def _commit(sched, cache, rows):
+    """What the engine does after a step: tokens are in the cache, sampled rows get a token, finished ones leave."""
+    for seq, n, m in rows:
+        cache.advance(seq.slot, seq.num_computed + n)
+        seq.num_computed += n
+        if m:
+            if seq.status is not Status.RUNNING:
+                sched.finished_prefill(seq)
+            seq.tokens.append(0)
+            if sched.at_limit(seq):
+                sched.finish(seq, "length")
+
+
+def test_prompts_are_cut_under_the_token_budget_in_arrival_order():
+    sched, cache = _sched(max_step_tokens=16)
+    a, b, c = _seq("a", 10), _seq("b", 20), _seq("c", 3)
+    for s in (a, b, c):
+        sched.add(s)
+    rows = sched.schedule()
+    assert [(s.rid, n, m) for s, n, m in rows] == [("a", 10, 1), ("b", 6, 0)]           # b is cut where the budget ends
+    _commit(sched, cache, rows)
+    rows = sched.schedule()                                                             # waiting requests go first
+    assert [(s.rid, n, m) for s, n, m in rows] == [("b", 14, 1), ("c", 2, 0)]
+    _commit(sched, cache, rows)
+    rows = sched.schedule()
+    assert [(s.rid, n, m) for s, n, m in rows] == [("c", 1, 1)]
+    _commit(sched, cache, rows)
+    rows = sched.schedule()                                                             # nothing waits: decode everyone
+    assert [(s.rid, n, m) for s, n, m in rows] == [("a", 1, 1), ("b", 1, 1), ("c", 1, 1)]
+    assert all(s.status is Status.RUNNING for s in (a, b, c))
+
+
+def test_mixed_steps_put_decode_rows_first_and_cap_the_portions():
+    sched, cache = _sched(max_step_tokens=16, chunk_with_decode=6, max_seqs=4)
+    a, b = _seq("a", 5), _seq("b", 20)
+    sched.add(a)
+    _commit(sched, cache, sched.schedule())
+    sched.add(b)
+    rows = sched.schedule()
+    assert [(s.rid, n, m) for s, n, m in rows] == [("a", 1, 1), ("b", 6, 0)]
+    assert sched.mixed_steps == 1
+    _commit(sched, cache, rows)
+    assert [(s.rid, n) for s, n, _ in sched.schedule()] == [("a", 1), ("b", 6)]
+
+
+def test_no_slot_no_admission_and_nobody_skips_ahead():
+    sched, cache = _sched(max_seqs=2, tokens=64)
+    for s in (_seq("a", 4), _seq("b", 4), _seq("c", 4)):
+        sched.add(s)
+    rows = sched.schedule()
+    assert [s.rid for s, _, _ in rows] == ["a", "b"]                                    # c has no slot yet
+    _commit(sched, cache, rows)
+    assert [s.rid for s, _, _ in sched.schedule()] == ["a", "b"]                        # c still waits: they decode
+
+
+def test_when_pages_run_out_the_lowest_ranked_is_preempted_and_recomputed():
+    sched, cache = _sched(tokens=24, page=4, max_model_len=24, max_step_tokens=32)      # 6 pages
+    a, b = _seq("a", 11, max_tokens=12), _seq("b", 11, max_tokens=12)
+    sched.add(a), sched.add(b)
+    rows = sched.schedule()
+    assert [(s.rid, n) for s, n, _ in rows] == [("a", 11), ("b", 11)]                   # 3 pages each: the pool is full
+    _commit(sched, cache, rows)
+    rows = sched.schedule()                                                             # token 12 fits the pages held
+    assert len(rows) == 2
+    _commit(sched, cache, rows)
+    rows = sched.schedule()                                                             # token 13 needs a page: b gives way
+    assert [(s.rid, n) for s, n, _ in rows] == [("a", 1)] and sched.preemptions == 1
+    assert b.status is Status.PREEMPTED and b.slot == -1 and b.num_computed == 0 and sched.waiting[0] is b
+    cache.check()
+    _commit(sched, cache, rows)
+    while a.status is not Status.FINISHED:                                              # b cannot come back while a grows
+        rows = sched.schedule()
+        assert all(s is a for s, _, _ in rows) or a.status is Status.FINISHED
+        _commit(sched, cache, rows)
+    rows = sched.schedule()                                                             # b runs its prompt and its 2 tokens again
+    assert [(s.rid, n, m) for s, n, m in rows] == [("b", 13, 1)]
+
+
+def test_a_request_alone_that_cannot_grow_preempts_itself_and_the_engine_would_refuse_that_setup():
+    sched, cache = _sched(tokens=8, page=4, max_model_len=32)
+    assert not cache.fits_alone(32)                 # the engine checks this at start and refuses (OutOfPages)
+    a = _seq("a", 8, max_tokens=8)
+    sched.add(a)
+    _commit(sched, cache, sched.schedule())
+    assert sched.schedule() is None or a.status is Status.PREEMPTED
+
+
+@pytest.mark.parametrize("mode", [0, 5])
+@pytest.mark.parametrize("seed", range(12))
+def test_every_request_finishes_under_random_traffic(seed, mode):
+    rng = random.Random(seed)
+    max_len = 32
+    sched, cache = _sched(tokens=rng.choice([32, 40, 64, 96]), page=rng.choice([1, 4, 8]), max_seqs=rng.choice([2, 4]),
+                          max_model_len=max_len, max_step_tokens=rng.choice([12, 16, 40]) if not mode else 16,
+                          chunk_with_decode=mode)
+    assert cache.fits_alone(max_len)
+    seqs = [_seq(i, rng.randint(1, 24), max_tokens=rng.randint(1, 12)) for i in range(14)]
+    pending = list(seqs)
+    for step in range(2000):
+        while pending and rng.random() < 0.4:
+            sched.add(pending.pop(0))
+        rows = sched.schedule()
+        if rows is None:
+            if not pending and not sched.waiting and not sched.running:
+                break
+            assert pending, "no progress with requests pending"
+            continue
+        n_decode = sum(1 for s, n, m in rows if s.status is Status.RUNNING)
+        assert all(s.status is Status.RUNNING for s, _, _ in rows[:n_decode])            # decode rows first, then portions
+        assert all(s.status is not Status.RUNNING for s, _, _ in rows[n_decode:])
+        assert sum(n for _, n, _ in rows) <= sched.max_step_tokens
+        if mode and n_decode:
+            assert sum(n for _, n, _ in rows[n_decode:]) <= mode
+        for s, n, m in rows:
+            assert n >= 1 and s.slot >= 0 and s.num_computed + n <= cache.capacity(s.slot)
+            assert m == int(s.num_computed + n == len(s.tokens))
+        _commit(sched, cache, rows)
+        cache.check()
+    assert all(s.status is Status.FINISHED for s in seqs)
+    assert all(len(s.tokens) - s.prompt_len == min(s.params.max_tokens, max_len - s.prompt_len) for s in seqs)
+    assert all(g.pool.free == g.pool.usable for g in cache.groups) and cache.free_slots == cache.max_seqs
