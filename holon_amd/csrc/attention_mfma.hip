@@ -279,24 +279,42 @@ __global__ void __launch_bounds__(64) attn_decode_kernel(AttnArgs a) {
   if (g == 0) { pml[0] = m[0]; pml[1] = lt; }
 }
 
-// out[row, head, :] = sum_i 2^(m_i - M) o_i / sum_i 2^(m_i - M) l_i, splits in index order.
-__global__ void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                  bf16_t* __restrict__ out, const int32_t* __restrict__ row_ids,
-                                  const int32_t* __restrict__ qstart, int heads, int splits, int head_dim) {
-  const int ri = blockIdx.x, h = blockIdx.y;
+// out[row, head, :] = sum_i 2^(m_i - M) o_i / sum_i 2^(m_i - M) l_i, splits in index order. One wave per (row, head):
+// lane s holds split s's weight (at most 64 splits), every lane a few dims of the output.
+__global__ void __launch_bounds__(64) attn_merge_kernel(const float* __restrict__ part_o,
+                                                        const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+                                                        const int32_t* __restrict__ row_ids,
+                                                        const int32_t* __restrict__ qstart, int heads, int splits,
+                                                        int head_dim) {
+  const int ri = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int token = qstart[row_ids[ri]];
   const float* ml = part_ml + ((int64_t)ri * heads + h) * splits * 2;
   const float* po = part_o + ((int64_t)ri * heads + h) * splits * head_dim;
-  float big = -INFINITY;
-  for (int s = 0; s < splits; ++s) big = fmaxf(big, ml[2 * s]);
+  float m_s = -INFINITY, l_s = 0.f;
+  if (lane < splits) {
+    const float2 v = *reinterpret_cast<const float2*>(ml + 2 * lane);
+    m_s = v.x;
+    l_s = v.y;
+  }
+  if (!(l_s > 0.f)) m_s = -INFINITY;
+  const float big = wave_max(m_s);
+  const float w_s = l_s > 0.f ? exp2f(m_s - big) : 0.f;
+  // the denominator in split order
   float denom = 0.f;
-  for (int s = 0; s < splits; ++s) denom += ml[2 * s + 1] > 0.f ? exp2f(ml[2 * s] - big) * ml[2 * s + 1] : 0.f;
+  for (int s = 0; s < splits; ++s) denom += __shfl(w_s * l_s, s, WAVE);
   const float inv = denom > 0.f ? 1.0f / denom : 0.f;
-  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-    float acc = 0.f;
-    for (int s = 0; s < splits; ++s)
-      if (ml[2 * s + 1] > 0.f) acc += exp2f(ml[2 * s] - big) * po[(int64_t)s * head_dim + d];
-    out[((int64_t)token * heads + h) * head_dim + d] = float_to_bf16(acc * inv);
+  for (int d0 = 4 * lane; d0 < head_dim; d0 += 4 * WAVE) {
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+    for (int s = 0; s < splits; ++s) {
+      const float w = __shfl(w_s, s, WAVE);
+      const f32x4_t v = *reinterpret_cast<const f32x4_t*>(po + (int64_t)s * head_dim + d0);
+      if (w > 0.f) acc += w * v;
+    }
+    ushort4 o;
+    o.x = float_to_bf16(acc[0] * inv); o.y = float_to_bf16(acc[1] * inv);
+    o.z = float_to_bf16(acc[2] * inv); o.w = float_to_bf16(acc[3] * inv);
+    *reinterpret_cast<ushort4*>(out + ((int64_t)token * heads + h) * head_dim + d0) = o;
   }
 }
 
@@ -345,7 +363,7 @@ extern "C" int holon_attention_decode_bf16(const void* q, void* out, const void*
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
               "attention: bad sizes");
-  HOLON_CHECK(splits > 0 && keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml,
+  HOLON_CHECK(splits > 0 && splits <= 64 && keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml,
               "attention decode: splits %d of %d keys (a multiple of 32) need a workspace", splits, keys_per_split);
   const int span = window > 0 ? (window < max_len ? window + 31 : max_len) : max_len;
   HOLON_CHECK((int64_t)splits * keys_per_split >= span, "attention decode: %d splits of %d keys do not cover %d keys",

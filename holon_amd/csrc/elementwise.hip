@@ -61,12 +61,101 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, T* __restrict__ residual
   }
 }
 
+// One block of 256 threads per row, for rows that fit the registers: 16-byte loads, the row is read once. VPT = vectors
+// of 16 bytes per thread. The sum of squares is reduced inside waves, then over the four waves in wave order.
+template <typename T, bool ADD, int VPT>
+__global__ void __launch_bounds__(256) rmsnorm_row_kernel(const T* __restrict__ x, T* __restrict__ residual,
+                                                          const T* __restrict__ weight, T* __restrict__ y, int dim,
+                                                          float eps) {
+  constexpr int V = Elem<T>::kVec;
+  __shared__ float part[4];
+  const int64_t row = blockIdx.x;
+  const int nvec = dim / V;
+  const uint4* xr = reinterpret_cast<const uint4*>(x + row * dim);
+  uint4* rr = ADD ? reinterpret_cast<uint4*>(residual + row * dim) : nullptr;
+  float vals[VPT][V];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int v = threadIdx.x + i * 256;
+    if (v < nvec) {
+      uint4 raw = xr[v];
+      const T* e = reinterpret_cast<const T*>(&raw);
+      if (ADD) {
+        uint4 rraw = rr[v];
+        T* re = reinterpret_cast<T*>(&rraw);
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          vals[i][j] = Elem<T>::round(Elem<T>::load(re[j]) + Elem<T>::load(e[j]));
+          re[j] = Elem<T>::store(vals[i][j]);
+        }
+        rr[v] = rraw;
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) vals[i][j] = Elem<T>::load(e[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < V; ++j) ss += vals[i][j] * vals[i][j];
+    }
+  }
+  ss = wave_sum(ss);
+  if (threadIdx.x % WAVE == 0) part[threadIdx.x / WAVE] = ss;
+  __syncthreads();
+  ss = ((part[0] + part[1]) + part[2]) + part[3];
+  const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+  const uint4* wr = reinterpret_cast<const uint4*>(weight);
+  uint4* yr = reinterpret_cast<uint4*>(y + row * dim);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int v = threadIdx.x + i * 256;
+    if (v < nvec) {
+      const uint4 wraw = wr[v];
+      const T* we = reinterpret_cast<const T*>(&wraw);
+      uint4 out;
+      T* oe = reinterpret_cast<T*>(&out);
+#pragma unroll
+      for (int j = 0; j < V; ++j) oe[j] = Elem<T>::store((vals[i][j] * inv) * Elem<T>::load(we[j]));
+      yr[v] = out;
+    }
+  }
+}
+
+template <typename T, bool ADD>
+static bool launch_rmsnorm_rows(const void* x, void* residual, const void* weight, void* y, int64_t rows, int dim,
+                                float eps, hipStream_t s) {
+  constexpr int V = Elem<T>::kVec;
+  if (dim % V != 0 || dim < 1024 || rows > 0x7fffffff) return false;
+  if ((((uintptr_t)x | (uintptr_t)residual | (uintptr_t)weight | (uintptr_t)y) & 15) != 0) return false;
+  const int vpt = (dim / V + 255) / 256;
+#define ROWS_LAUNCH(VPT)                                                                                          \
+  rmsnorm_row_kernel<T, ADD, VPT><<<(unsigned)rows, 256, 0, s>>>((const T*)x, (T*)residual, (const T*)weight, (T*)y, \
+                                                                 dim, eps)
+  if (vpt <= 1) ROWS_LAUNCH(1);
+  else if (vpt <= 2) ROWS_LAUNCH(2);
+  else if (vpt <= 4) ROWS_LAUNCH(4);
+  else if (vpt <= 8) ROWS_LAUNCH(8);
+  else return false;
+#undef ROWS_LAUNCH
+  return true;
+}
+
 extern "C" int holon_rmsnorm(const void* x, void* residual, const void* weight, void* y, int64_t rows, int dim,
                              float eps, int dtype, void* stream) {
   HOLON_CHECK(rows >= 0 && dim > 0, "rmsnorm: bad sizes rows=%lld dim=%d", (long long)rows, dim);
   if (rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  const int waves = 4;
+  bool done;
+  if (dtype == HOLON_F32)
+    done = residual ? launch_rmsnorm_rows<float, true>(x, residual, weight, y, rows, dim, eps, s)
+                    : launch_rmsnorm_rows<float, false>(x, residual, weight, y, rows, dim, eps, s);
+  else
+    done = residual ? launch_rmsnorm_rows<bf16_t, true>(x, residual, weight, y, rows, dim, eps, s)
+                    : launch_rmsnorm_rows<bf16_t, false>(x, residual, weight, y, rows, dim, eps, s);
+  if (done) {
+    HOLON_LAUNCH_OK();
+    return 0;
+  }
+  const int waves = 4;   // narrow or odd rows: one wave per row
   const unsigned grid = (unsigned)((rows + waves - 1) / waves);
 #define RMS_LAUNCH(T, ADD) \
   rmsnorm_kernel<T, ADD><<<grid, waves * WAVE, 0, s>>>((const T*)x, (T*)residual, (const T*)weight, (T*)y, rows, dim, eps)

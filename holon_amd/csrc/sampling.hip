@@ -18,7 +18,18 @@ __device__ ArgMax block_argmax(const float* __restrict__ row, int vocab, float i
   __shared__ ArgMax part[SAMPLE_THREADS / WAVE];
   __shared__ ArgMax result;
   ArgMax best{-INFINITY, 0x7fffffff};
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) best = better(best, ArgMax{row[i] * inv_temp, i});
+  if ((vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {   // 16-byte loads where the row allows
+    const float4* row4 = reinterpret_cast<const float4*>(row);
+    for (int i = threadIdx.x; i < vocab / 4; i += blockDim.x) {
+      const float4 v = row4[i];
+      best = better(best, ArgMax{v.x * inv_temp, 4 * i});
+      best = better(best, ArgMax{v.y * inv_temp, 4 * i + 1});
+      best = better(best, ArgMax{v.z * inv_temp, 4 * i + 2});
+      best = better(best, ArgMax{v.w * inv_temp, 4 * i + 3});
+    }
+  } else {
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) best = better(best, ArgMax{row[i] * inv_temp, i});
+  }
 #pragma unroll
   for (int o = WAVE / 2; o > 0; o >>= 1) {
     ArgMax other{__shfl_xor(best.v, o, WAVE), __shfl_xor(best.i, o, WAVE)};
