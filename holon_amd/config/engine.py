@@ -31,6 +31,8 @@ class EngineConfig:
     state_memory: int | None = _setting(None, "bytes for state pools; default: from memory_fraction")
     cache_tokens: int | None = _setting(None, "tokens of paged state per pool (overrides state_memory)")
     graphs: bool = _setting(True, "replay decode steps from HIP graphs, per batch-size bucket")
+    decode_weight_copy: bool = _setting(True, "keep a second copy of every projection in the tile layout that steps of "
+                                              "few rows stream fastest (doubles the weights' memory)")
 
     def __post_init__(self) -> None:
         for name in ("page_size", "max_seqs", "max_model_len", "max_step_tokens"):

@@ -303,18 +303,21 @@ __global__ void __launch_bounds__(64) attn_merge_kernel(const float* __restrict_
   float denom = 0.f;
   for (int s = 0; s < splits; ++s) denom += __shfl(w_s * l_s, s, WAVE);
   const float inv = denom > 0.f ? 1.0f / denom : 0.f;
-  for (int d0 = 4 * lane; d0 < head_dim; d0 += 4 * WAVE) {
+  for (int base = 0; base < head_dim; base += 4 * WAVE) {   // every lane walks the loop: the shuffles read all lanes
+    const int d0 = base + 4 * lane;
+    const bool mine = d0 < head_dim;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll 8
     for (int s = 0; s < splits; ++s) {
       const float w = __shfl(w_s, s, WAVE);
-      const f32x4_t v = *reinterpret_cast<const f32x4_t*>(po + (int64_t)s * head_dim + d0);
-      if (w > 0.f) acc += w * v;
+      if (mine && w > 0.f) acc += w * *reinterpret_cast<const f32x4_t*>(po + (int64_t)s * head_dim + d0);
     }
-    ushort4 o;
-    o.x = float_to_bf16(acc[0] * inv); o.y = float_to_bf16(acc[1] * inv);
-    o.z = float_to_bf16(acc[2] * inv); o.w = float_to_bf16(acc[3] * inv);
-    *reinterpret_cast<ushort4*>(out + ((int64_t)token * heads + h) * head_dim + d0) = o;
+    if (mine) {
+      ushort4 o;
+      o.x = float_to_bf16(acc[0] * inv); o.y = float_to_bf16(acc[1] * inv);
+      o.z = float_to_bf16(acc[2] * inv); o.w = float_to_bf16(acc[3] * inv);
+      *reinterpret_cast<ushort4*>(out + ((int64_t)token * heads + h) * head_dim + d0) = o;
+    }
   }
 }
 

@@ -5,13 +5,17 @@
 // v_mfma_f32_16x16x32_bf16 with the weights as A (16 rows x 32 k: lane l reads 16 contiguous bytes of row l%16) and
 // the activations as B (32 k x 16 tokens: lane l reads 16 contiguous bytes of token l%16); the result tile has weight
 // rows 4*(l/16)+r of token l%16 in lane l, i.e. 4 consecutive outputs of one token: one 8- or 16-byte store.
+//
+// Two weight layouts: rows [N, K] as the checkpoint stores them, and tiles [N/16, K/32, 64 lanes, 8] in which the
+// 16 bytes lane l needs for one product are at lane l's place, so that a wave's load is one contiguous kilobyte and a
+// tile's whole K extent is one contiguous run (measured: 6 to 7 TB/s against 4 to 5 for the row layout).
 #include "common.h"
 #include "holon_hip.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
-template <int MT, int WPB, int UNROLL, typename OutT>
+template <int MT, int WPB, int UNROLL, typename OutT, bool TILED>
 __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                 const bf16_t* __restrict__ w, OutT* __restrict__ y,
                                                                 int M, int N, int K) {
@@ -20,7 +24,10 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
   const int g = lane / 16, c = lane % 16;
   const int n0 = blockIdx.x * 16;
   const int kw = K / WPB;                       // this wave's slice of K (a multiple of 32)
-  const bf16_t* wp = w + (int64_t)(n0 + c) * K + (int64_t)wave * kw + 8 * g;
+  const int steps = kw / 32;
+  const bf16_t* wp = TILED ? w + ((int64_t)blockIdx.x * (K / 32) + (int64_t)wave * steps) * 512 + lane * 8
+                           : w + (int64_t)(n0 + c) * K + (int64_t)wave * kw + 8 * g;
+  constexpr int WSTEP = TILED ? 512 : 32;       // elements between one product's weights and the next
   const bf16_t* xp = x + (int64_t)c * K + (int64_t)wave * kw + 8 * g;
   f32x4_t acc[MT];
 #pragma unroll
@@ -29,12 +36,12 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
 #pragma unroll
   for (int t = 0; t < MT; ++t) have[t] = t * 16 + c < M;
 
-  const int steps = kw / 32;
   int s = 0;
   for (; s + UNROLL <= steps; s += UNROLL) {
     bf16x8_t wf[UNROLL], xf[UNROLL][MT];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) wf[u] = *reinterpret_cast<const bf16x8_t*>(wp + (s + u) * 32);
+    for (int u = 0; u < UNROLL; ++u)
+      wf[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp + (int64_t)(s + u) * WSTEP));
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
@@ -52,7 +59,7 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
       for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u][t], acc[t], 0, 0, 0);
   }
   for (; s < steps; ++s) {
-    const bf16x8_t wf = *reinterpret_cast<const bf16x8_t*>(wp + s * 32);
+    const bf16x8_t wf = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp + (int64_t)s * WSTEP));
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       bf16x8_t xf;
@@ -92,27 +99,36 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
   }
 }
 
-template <int MT, int WPB, typename OutT>
-static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, hipStream_t s) {
-  constexpr int UNROLL = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
-  gemm_skinny_kernel<MT, WPB, UNROLL, OutT><<<N / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (OutT*)y,
-                                                                         M, N, K);
+template <int MT, int WPB, int UNROLL, typename OutT>
+static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s) {
+  if (tiled)
+    gemm_skinny_kernel<MT, WPB, UNROLL, OutT, true><<<N / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
+                                                                                (OutT*)y, M, N, K);
+  else
+    gemm_skinny_kernel<MT, WPB, UNROLL, OutT, false><<<N / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
+                                                                                 (OutT*)y, M, N, K);
 }
 
+// How many waves share a tile, from the shapes alone (so a result never depends on M): wide outputs have tiles
+// enough to fill the GPU with few waves each and long loops; narrow ones split K 16 ways. Measured on MI355X.
 template <int MT, typename OutT>
-static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K, hipStream_t s) {
-  // enough waves to keep the memory system busy: aim for a few thousand, K split in multiples of 32
+static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s) {
   const int tiles = N / 16;
   int wpb = MT >= 3 ? 8 : 16;                  // 16 waves of 3 or 4 token tiles run out of registers
-  while (wpb > 1 && (K % (32 * wpb) != 0 || tiles * (wpb / 2) >= 4096)) wpb /= 2;
+  if (tiles >= 1024) wpb = 4;
+  while (wpb > 1 && K % (32 * wpb) != 0) wpb /= 2;
+  constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
   switch (wpb) {
     case 16:
-      if constexpr (MT < 3) launch_skinny<MT, 16, OutT>(x, w, y, M, N, K, s);
+      if constexpr (MT < 3) launch_skinny<MT, 16, U, OutT>(x, w, y, M, N, K, tiled, s);
       break;
-    case 8: launch_skinny<MT, 8, OutT>(x, w, y, M, N, K, s); break;
-    case 4: launch_skinny<MT, 4, OutT>(x, w, y, M, N, K, s); break;
-    case 2: launch_skinny<MT, 2, OutT>(x, w, y, M, N, K, s); break;
-    default: launch_skinny<MT, 1, OutT>(x, w, y, M, N, K, s); break;
+    case 8: launch_skinny<MT, 8, U, OutT>(x, w, y, M, N, K, tiled, s); break;
+    case 4:
+      if constexpr (MT == 1) launch_skinny<MT, 4, 16, OutT>(x, w, y, M, N, K, tiled, s);
+      else launch_skinny<MT, 4, U, OutT>(x, w, y, M, N, K, tiled, s);
+      break;
+    case 2: launch_skinny<MT, 2, U, OutT>(x, w, y, M, N, K, tiled, s); break;
+    default: launch_skinny<MT, 1, U, OutT>(x, w, y, M, N, K, tiled, s); break;
   }
   return 0;
 }
@@ -121,18 +137,37 @@ extern "C" int holon_gemm_skinny_supported(int M, int N, int K) {
   return M >= 1 && M <= 64 && N % 16 == 0 && K % 32 == 0 && K >= 32;
 }
 
-// out_f32: 1 writes float32, 0 bfloat16.
+// out_f32: 1 writes float32, 0 bfloat16. tiled: 1 when `w` is in the tile layout (see holon_tile_weight_bf16).
 extern "C" int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_f32,
-                                      void* stream) {
+                                      int tiled, void* stream) {
   HOLON_CHECK(holon_gemm_skinny_supported(M, N, K), "gemm (few rows): M=%d N=%d K=%d not served (M <= 64, N %% 16, K %% 32)",
               M, N, K);
   hipStream_t s = (hipStream_t)stream;
   const int mt = (M + 15) / 16;
 #define SKINNY(MT)                                                                 \
-  if (out_f32) pick_waves<MT, float>(x, w, y, M, N, K, s);                          \
-  else pick_waves<MT, bf16_t>(x, w, y, M, N, K, s)
+  if (out_f32) pick_waves<MT, float>(x, w, y, M, N, K, tiled != 0, s);              \
+  else pick_waves<MT, bf16_t>(x, w, y, M, N, K, tiled != 0, s)
   if (mt == 1) { SKINNY(1); } else if (mt == 2) { SKINNY(2); } else if (mt == 3) { SKINNY(3); } else { SKINNY(4); }
 #undef SKINNY
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+// tiled[t][s][l][e] = w[16 t + l % 16][32 s + 8 (l / 16) + e]: the layout the few-row product streams.
+__global__ void tile_weight_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ tiled, int N, int K) {
+  const int64_t chunks = (int64_t)N * K / 8;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * blockDim.x) {
+    const int lane = (int)(i % 64);
+    const int64_t ts = i / 64;
+    const int64_t step = ts % (K / 32), tile = ts / (K / 32);
+    const int64_t src = (tile * 16 + lane % 16) * K + step * 32 + 8 * (lane / 16);
+    *reinterpret_cast<uint4*>(tiled + i * 8) = *reinterpret_cast<const uint4*>(w + src);
+  }
+}
+
+extern "C" int holon_tile_weight_bf16(const void* w, void* tiled, int N, int K, void* stream) {
+  HOLON_CHECK(N > 0 && K > 0 && N % 16 == 0 && K % 32 == 0, "tile_weight: N=%d K=%d must be multiples of 16 and 32", N, K);
+  tile_weight_kernel<<<4096, 256, 0, (hipStream_t)stream>>>((const bf16_t*)w, (bf16_t*)tiled, N, K);
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -44,9 +44,12 @@ int holon_attention_decode_bf16(const void* q, void* out, const void* pages, con
                                 const int32_t* row_ids, int n_rows, int max_len, int heads, int kv_heads, int head_dim,
                                 int page_size, float scale, int window, float* part_o, float* part_ml, int splits,
                                 int keys_per_split, void* stream);
-// y[M, N] = x[M, K] w[N, K]^T for M <= 64 rows, bfloat16 in, float32 accumulation; out_f32 picks the output type.
+// y[M, N] = x[M, K] w[N, K]^T for M <= 64 rows, bfloat16 in, float32 accumulation; out_f32 picks the output type;
+// tiled says that `w` is holon_tile_weight_bf16's copy ([N/16, K/32, 64, 8]: lane-major 16-byte pieces).
 int holon_gemm_skinny_supported(int M, int N, int K);
-int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_f32, void* stream);
+int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_f32, int tiled,
+                           void* stream);
+int holon_tile_weight_bf16(const void* w, void* tiled, int N, int K, void* stream);
 int holon_argmax(const float* logits, int32_t* out, int rows, int vocab, void* stream);
 int holon_sample(const float* logits, int32_t* out, int rows, int vocab, const float* temperature,
                  const int32_t* top_k, const float* top_p, const float* min_p, const int64_t* seeds,

@@ -53,7 +53,8 @@ class Engine:
         self.eos = set(self.spec.eos_token_ids)
         shape = dict(page_size=cfg.page_size, max_seqs=cfg.max_seqs, max_model_len=cfg.max_model_len,
                      max_step_tokens=cfg.max_step_tokens)
-        self.model, _ = build_from_spec(self.spec, device=device, dtype=dtype, kernels=self.kernels, **shape)
+        self.model, _ = build_from_spec(self.spec, device=device, dtype=dtype, kernels=self.kernels,
+                                        decode_copy=cfg.decode_weight_copy, **shape)
         if random_config is not None:
             fill_random(self.model, self.spec, seed, device, dtype)
         else:

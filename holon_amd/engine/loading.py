@@ -51,9 +51,10 @@ class Loaded:
 
 
 def build_from_spec(spec: ModelSpec, *, device: torch.device, dtype: torch.dtype, kernels, page_size: int,
-                    max_seqs: int, max_model_len: int, max_step_tokens: int) -> tuple[Model, Build]:
+                    max_seqs: int, max_model_len: int, max_step_tokens: int, decode_copy: bool = True
+                    ) -> tuple[Model, Build]:
     build = Build(kernels=kernels, device=device, dtype=dtype, page_size=page_size, max_model_len=max_model_len,
-                  max_seqs=max_seqs, max_step_tokens=max_step_tokens)
+                  max_seqs=max_seqs, max_step_tokens=max_step_tokens, decode_copy=decode_copy)
     return build_model(spec, build), build
 
 

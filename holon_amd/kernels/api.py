@@ -52,8 +52,13 @@ class Kernels(Protocol):
     def add_rmsnorm(self, x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
         """residual += x in place (sum rounded to dtype), returns rmsnorm(residual) as a new tensor."""
 
-    def linear(self, x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-        """x [T, K] @ weight [N, K].T -> [T, N], float32 accumulation, rounded to out_dtype (default: x's)."""
+    def linear(self, x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None = None,
+               tiled: torch.Tensor | None = None) -> torch.Tensor:
+        """x [T, K] @ weight [N, K].T -> [T, N], float32 accumulation, rounded to out_dtype (default: x's).
+        `tiled`: what `tile_weight(weight)` returned, if anything."""
+
+    def tile_weight(self, weight: torch.Tensor) -> torch.Tensor | None:
+        """Once per weight after loading: a copy in the layout steps of few rows stream fastest, or None."""
 
     def silu_mul(self, gate_up: torch.Tensor) -> torch.Tensor:
         """gate_up [T, 2I] (gate columns first) -> [T, I] = round(silu(gate)) * up."""

@@ -65,7 +65,8 @@ class HipKernels:
             "holon_attention_decode_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P,
                                             _I, _I, _P],
             "holon_gemm_skinny_supported": [_I, _I, _I],
-            "holon_gemm_skinny_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
+            "holon_gemm_skinny_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "holon_tile_weight_bf16": [_P, _P, _I, _I, _P],
             "holon_argmax": [_P, _P, _I, _I, _P],
             "holon_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
         }
@@ -131,7 +132,18 @@ class HipKernels:
 
     skinny_rows = 16          # up to this many rows the hand-written weight-streaming product runs
 
-    def linear(self, x, weight, out_dtype=None):
+    def tile_weight(self, weight):
+        """A copy of `weight` [N, K] in the layout the few-row product streams fastest, or None when its shape or
+        dtype has no such layout (then `linear` reads the rows as they are)."""
+        n, k = weight.shape
+        if weight.dtype != torch.bfloat16 or not weight.is_cuda or n % 16 or k % 32 or k < 256:
+            return None
+        self._check(weight, "tile_weight")
+        tiled = torch.empty_like(weight)
+        self._call(self.lib.holon_tile_weight_bf16, weight.data_ptr(), tiled.data_ptr(), n, k, self._stream())
+        return tiled
+
+    def linear(self, x, weight, out_dtype=None, tiled=None):
         m, k = x.shape
         n = weight.shape[0]
         if weight.shape[1] != k:
@@ -140,8 +152,9 @@ class HipKernels:
                 and x.is_contiguous() and weight.is_contiguous() and self.lib.holon_gemm_skinny_supported(m, n, k)):
             to_f32 = out_dtype == torch.float32
             y = torch.empty((m, n), dtype=torch.float32 if to_f32 else torch.bfloat16, device=x.device)
-            self._call(self.lib.holon_gemm_skinny_bf16, x.data_ptr(), weight.data_ptr(), y.data_ptr(), m, n, k,
-                       int(to_f32), self._stream())
+            source = tiled if tiled is not None else weight
+            self._call(self.lib.holon_gemm_skinny_bf16, x.data_ptr(), source.data_ptr(), y.data_ptr(), m, n, k,
+                       int(to_f32), int(tiled is not None), self._stream())
             return y
         # the vendor library's product, float32 accumulation (no reduced-precision mode for float32 operands)
         y = torch.matmul(x, weight.t())

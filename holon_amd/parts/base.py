@@ -60,6 +60,7 @@ class Build:
     max_model_len: int = 8192
     max_seqs: int = 64
     max_step_tokens: int = 4096
+    decode_copy: bool = True                      # keep a second, tiled copy of every projection for decode steps
 
     def make(self, ref: PartRef, **site: Any) -> "Part":
         return part_class(ref)(self, **ref.get(), **site)
@@ -114,4 +115,7 @@ class Part:
                 t = getattr(part, name)
                 if t is not None:
                     total += t.numel() * t.element_size()
+            tiled = getattr(part, "tiled", None)
+            if tiled is not None:
+                total += tiled.numel() * tiled.element_size()
         return total

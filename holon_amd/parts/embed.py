@@ -27,11 +27,18 @@ class LMHead(Part):
         super().__init__(build)
         self.tied = tied
         self._embed = [embed]                     # in a list: the embedding part keeps the one owner of the tensor
+        self.tiled: torch.Tensor | None = None
         if not tied:
             self.declare("weight", (vocab, hidden))
 
+    def _weight(self) -> torch.Tensor:
+        return self._embed[0].weight if self.tied else self.weight
+
+    def finalize(self) -> None:
+        if self.build.decode_copy and self._weight() is not None:
+            self.tiled = self.kernels.tile_weight(self._weight())
+
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        weight = self._embed[0].weight if self.tied else self.weight
-        return self.kernels.linear(h, weight, torch.float32)
+        return self.kernels.linear(h, self._weight(), torch.float32, self.tiled)
 
     __call__ = forward

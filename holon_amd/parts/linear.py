@@ -12,9 +12,14 @@ class Linear(Part):
         super().__init__(build)
         self.inp, self.out = inp, out
         self.declare("weight", (out, inp))
+        self.tiled: torch.Tensor | None = None    # a second copy in the layout decode steps stream fastest
+
+    def finalize(self) -> None:
+        if self.weight is not None and self.build.decode_copy:
+            self.tiled = self.kernels.tile_weight(self.weight)
 
     def forward(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-        return self.kernels.linear(x, self.weight, out_dtype)
+        return self.kernels.linear(x, self.weight, out_dtype, self.tiled)
 
     __call__ = forward
 
@@ -24,5 +29,6 @@ class Linear(Part):
         merged = Linear(build, inp=parts[0].inp, out=sum(p.out for p in parts))
         merged.weight = torch.cat([p.weight for p in parts], dim=0)
         for p in parts:
-            p.weight = None
+            p.weight = p.tiled = None
+        merged.finalize()
         return merged

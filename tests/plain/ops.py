@@ -52,7 +52,10 @@ class TorchKernels:
         residual.add_(x)
         return _rmsnorm(residual, weight, eps)
 
-    def linear(self, x, weight, out_dtype=None):
+    def tile_weight(self, weight):
+        return None
+
+    def linear(self, x, weight, out_dtype=None, tiled=None):
         return (_up(x) @ _up(weight).T).to(out_dtype or x.dtype)
 
     def silu_mul(self, gate_up):

@@ -210,6 +210,11 @@ def test_linear(hip, dtype, monkeypatch):
         assert got.dtype == dtype and H.op_budget_usage(got, want, dtype, k) <= 1, (t, k, n)
         got32 = hip.linear(x, w, torch.float32)
         assert got32.dtype == torch.float32 and H.op_budget_usage(got32, want, dtype, k) <= 1
+        tiled = hip.tile_weight(w)
+        assert (tiled is None) == (dtype != torch.bfloat16 or n % 16 != 0 or k % 32 != 0 or k < 256)
+        if tiled is not None:                          # the tile layout is a permutation: the same bits come out
+            assert torch.equal(hip.linear(x, w, None, tiled), got)
+            assert torch.equal(hip.linear(x, w, torch.float32, tiled), got32)
     # exact arithmetic: activations in {-1, 0, 1} and weights in {-1, 0, 1} / 8 make every partial sum exact, so any
     # order of summation gives the same bits (plugins/tests/test_attention_kv_quant.py:244-261)
     g = torch.Generator().manual_seed(15)
