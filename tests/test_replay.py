@@ -142,3 +142,38 @@ def test_logits_do_not_depend_on_the_cut_in_float32(folders, device):
     for other in (parts, tail):
         b = torch.stack([other[k] for k in sorted(whole)])
         H.assert_fp32_close(b, a, "cut independence")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_trace_run_program(folders, tmp_path, dtype):
+    """bin/trace_run as a user runs it: steps on standard input, `done <step>` lines, logits files [wanted, vocab] as
+    little-endian float32; a step that wants nothing writes no file."""
+    import pathlib
+    import subprocess
+    import sys
+
+    import numpy as np
+    folder, name = folders["B-sharp"], "B-sharp"
+    requests = _requests(name, (40, 70, 33, 90))
+    trace = H.trace_mixed(requests, 3)
+    trace.steps[2]["entries"][0]["want"] = []                  # one step computes without reporting
+    dropped = trace.expect[2][: len(trace.steps[2]["entries"][0]["tokens"])]
+    trace.expect[2] = trace.expect[2][len(dropped):]
+    out = tmp_path / "out"
+    program = pathlib.Path(__file__).resolve().parent.parent / "bin" / "trace_run"
+    run = subprocess.run([sys.executable, str(program), "--model", str(folder), "--dtype", dtype, "--out", str(out),
+                          "--max-tokens", str(H.peak_live_tokens(trace)), "--page-size", "8"],
+                         input=trace.jsonl(), capture_output=True, text=True, timeout=110)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert run.stdout.split("\n")[:-1] == [f"done {i}" for i in range(len(trace.steps))]
+    vocab = MODELS[name][0]["vocab_size"]
+    got = {}
+    for i, expect in enumerate(trace.expect):
+        path = out / f"{i}.f32"
+        assert path.exists() == bool(expect)
+        if expect:
+            rows = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(len(expect), vocab))
+            got.update(zip(expect, rows))
+    assert len(got) == sum(map(len, requests.values())) - len(dropped)
+    _check(folder, dtype, requests, got, f"trace_run {dtype}")
