@@ -76,26 +76,36 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
   const int khalf = krow / 16, kin = krow % 16;
   const int max_page = a.table_stride - 1;
 
-  for (int kb = (key_lo / 32) * 32; kb <= key_hi; kb += 32) {
-    // the two pages this block touches (a block of 32 keys is two groups of 16; a group never straddles a page)
-    const int pi0 = min(kb / P, max_page), pi1 = min((kb + 16) / P, max_page);
-    const int64_t pg0 = (int64_t)trow[pi0] * page_stride, pg1 = (int64_t)trow[pi1] * page_stride;
-    const int off0 = kb % P, off1 = (kb + 16) % P;
-    const bf16_t* krowp = kbase + (khalf ? pg1 : pg0) + (int64_t)((khalf ? off1 : off0) + kin) * D + 8 * g;
-    bf16x8_t kf0[D / 32], kf1[D / 32];
+  // Keys of block kb for this lane: two fragments per 32 dims (the lane's key, and the key 4 further on).
+  auto load_keys = [&](int kb, bf16x8_t (&f0)[D / 32], bf16x8_t (&f1)[D / 32]) {
+    const int half_key = kb + 16 * khalf;
+    const int64_t pg = (int64_t)trow[min(half_key / P, max_page)] * page_stride;
+    const bf16_t* krowp = kbase + pg + (int64_t)(half_key % P + kin) * D + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < D / 32; ++ks) {
-      kf0[ks] = load8(krowp + ks * 32);
-      kf1[ks] = load8(krowp + 4 * D + ks * 32);   // the key 4 further on
+      f0[ks] = load8(krowp + ks * 32);
+      f1[ks] = load8(krowp + 4 * D + ks * 32);
     }
-    // values: lane group g needs keys 8g .. 8g+7 of the block, for dims dsub*16 + c
-    const bf16_t* vrowp = vbase + (g >= 2 ? pg1 : pg0) + (int64_t)c * P + (g >= 2 ? off1 : off0) + 8 * (g % 2);
+  };
+  const int kb_first = (key_lo / 32) * 32;
+  bf16x8_t kf0[D / 32], kf1[D / 32];
+  load_keys(kb_first, kf0, kf1);
+  for (int kb = kb_first; kb <= key_hi; kb += 32) {
+    // values of this block (lane group g needs keys 8g .. 8g+7, for dims dsub*16 + c) and the keys of the next one
+    // are requested before this block's products, so that their latency hides behind the matrix cores
+    const int vkey = kb + (g >= 2 ? 16 : 0);
+    const bf16_t* vrowp = vbase + (int64_t)trow[min(vkey / P, max_page)] * page_stride + (int64_t)c * P + vkey % P +
+                          8 * (g % 2);
+    bf16x8_t vf[D / 16];
+#pragma unroll
+    for (int ds = 0; ds < D / 16; ++ds) vf[ds] = load8(vrowp + (int64_t)ds * 16 * P);
+    bf16x8_t nf0[D / 32], nf1[D / 32];
+    const bool more = kb + 32 <= key_hi;
+    if (more) load_keys(kb + 32, nf0, nf1);
     bf16x8_t pb[NT];
-    bool any = false;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       if (kb > tile_last[t]) continue;   // every key of the block lies after every query of the tile
-      any = true;
       f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < D / 32; ++ks) {
@@ -131,14 +141,19 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
 #pragma unroll
       for (int ds = 0; ds < D / 16; ++ds) o[t][ds] *= alpha;
     }
-    if (!any) continue;
 #pragma unroll
     for (int ds = 0; ds < D / 16; ++ds) {
-      const bf16x8_t vf = load8(vrowp + (int64_t)ds * 16 * P);
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         if (kb > tile_last[t]) continue;
-        o[t][ds] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[t], o[t][ds], 0, 0, 0);
+        o[t][ds] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[ds], pb[t], o[t][ds], 0, 0, 0);
+      }
+    }
+    if (more) {
+#pragma unroll
+      for (int ks = 0; ks < D / 32; ++ks) {
+        kf0[ks] = nf0[ks];
+        kf1[ks] = nf1[ks];
       }
     }
   }
@@ -170,8 +185,11 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
   const TileMap tm = tile_map(group);
   const int hk = blockIdx.y / tm.head_blocks, hb = blockIdx.y % tm.head_blocks;
   const int qs = a.qstart[b], nq = a.qstart[b + 1] - qs, n = a.lens[b];
-  const int p_first = (blockIdx.x * 4 + wave) * NT * tm.pos_per_tile;   // first position index of this wave
-  if (p_first >= nq || n <= 0) return;
+  // Tiles of 16 rows along the row's positions. A wave takes NT of them: with NT = 2 the w-th from the start and the
+  // w-th from the end, so that every wave walks about the same number of keys under the causal mask.
+  const int n_tiles = (nq + tm.pos_per_tile - 1) / tm.pos_per_tile;
+  const int wi = blockIdx.x * 4 + wave;
+  if (n <= 0 || wi >= (n_tiles + NT - 1) / NT) return;
   const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
 
   bf16x8_t qf[NT][D / 32];
@@ -180,7 +198,9 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
   int key_hi = 0, key_lo = 0x7fffffff;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const int p0 = p_first + t * tm.pos_per_tile;
+    int tile = NT == 1 ? n_tiles - 1 - wi : (t == 0 ? wi : n_tiles - 1 - wi);
+    if (t == 1 && tile <= wi) tile = n_tiles;          // an odd count: the middle tile is the first one's alone
+    const int p0 = tile * tm.pos_per_tile;
     rr[t] = row_ref(tm, c, p0, hb, hk, group, qs, nq, n);
     qpos[t] = rr[t].valid ? rr[t].qpos : -1;   // an unused row sees no key
     const int last_qi = min(nq, p0 + tm.pos_per_tile) - 1;
@@ -346,8 +366,8 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
   a.scale_log2 = scale * 1.4426950408889634f; a.window = window;
   const TileMap tm = tile_map(heads / kv_heads);
   const int nt = head_dim == 256 ? 1 : 2;
-  const int pos_per_block = 4 * nt * tm.pos_per_tile;
-  dim3 grid((max_query + pos_per_block - 1) / pos_per_block, kv_heads * tm.head_blocks, n_rows);
+  const int tiles = (max_query + tm.pos_per_tile - 1) / tm.pos_per_tile;
+  dim3 grid(((tiles + nt - 1) / nt + 3) / 4, kv_heads * tm.head_blocks, n_rows);
   hipStream_t s = (hipStream_t)stream;
   if (head_dim == 64) attn_prefill_kernel<64, 2><<<grid, 256, 0, s>>>(a);
   else if (head_dim == 128) attn_prefill_kernel<128, 2><<<grid, 256, 0, s>>>(a);

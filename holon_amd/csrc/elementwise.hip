@@ -183,10 +183,46 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   }
 }
 
+// 16 bytes of gate and 16 bytes of up per thread (widths that are multiples of the vector).
+template <typename T>
+__global__ void silu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int64_t tokens, int inter) {
+  constexpr int V = Elem<T>::kVec;
+  const int per_row = inter / V;
+  const int64_t n = tokens * per_row;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = i / per_row;
+    const int c = (int)(i - t * per_row) * V;
+    const uint4 graw = *reinterpret_cast<const uint4*>(gu + t * 2 * inter + c);
+    const uint4 uraw = *reinterpret_cast<const uint4*>(gu + t * 2 * inter + inter + c);
+    const T* ge = reinterpret_cast<const T*>(&graw);
+    const T* ue = reinterpret_cast<const T*>(&uraw);
+    uint4 oraw;
+    T* oe = reinterpret_cast<T*>(&oraw);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const float g = Elem<T>::load(ge[j]);
+      const float sg = Elem<T>::round(g / (1.0f + expf(-g)));
+      oe[j] = Elem<T>::store(sg * Elem<T>::load(ue[j]));
+    }
+    *reinterpret_cast<uint4*>(out + t * inter + c) = oraw;
+  }
+}
+
 extern "C" int holon_silu_mul(const void* gate_up, void* out, int64_t tokens, int inter, int dtype, void* stream) {
   HOLON_CHECK(tokens >= 0 && inter > 0, "silu_mul: bad sizes");
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  const int vec = dtype == HOLON_F32 ? 4 : 8;
+  if (inter % vec == 0 && (((uintptr_t)gate_up | (uintptr_t)out) & 15) == 0) {
+    const int64_t nv = tokens * (inter / vec);
+    const unsigned vgrid = (unsigned)((nv + 255) / 256 < 16384 ? (nv + 255) / 256 : 16384);
+    if (dtype == HOLON_F32)
+      silu_mul_vec_kernel<float><<<vgrid, 256, 0, s>>>((const float*)gate_up, (float*)out, tokens, inter);
+    else
+      silu_mul_vec_kernel<bf16_t><<<vgrid, 256, 0, s>>>((const bf16_t*)gate_up, (bf16_t*)out, tokens, inter);
+    HOLON_LAUNCH_OK();
+    return 0;
+  }
   const int64_t n = tokens * inter;
   const unsigned grid = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
   if (dtype == HOLON_F32)
@@ -263,6 +299,58 @@ __global__ void qk_norm_rope_write_kernel(const T* qkv, int64_t qkv_stride, T* q
   }
 }
 
+// The same for head_dim 64, 128 or 256 with the whole head rotated (or not at all): each lane holds EPL = head_dim / 64
+// consecutive values; the rotation partner of a value sits 32 lanes away, so a shuffle replaces the LDS staging.
+template <typename T, int EPL>
+__global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
+    const T* qkv, int64_t qkv_stride, T* q_out, int heads, int kv_heads, const T* __restrict__ q_weight,
+    const T* __restrict__ k_weight, float eps, const float* __restrict__ table, const int32_t* __restrict__ positions,
+    T* __restrict__ pages, const int32_t* __restrict__ write_page, const int32_t* __restrict__ write_off,
+    int page_size, int total_heads) {
+  constexpr int D = EPL * WAVE;
+  const int w = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int t = blockIdx.x;
+  const int h = blockIdx.y * 4 + w;
+  if (h >= total_heads) return;   // no barrier below
+  const T* src = qkv + (int64_t)t * qkv_stride + (int64_t)h * D + lane * EPL;
+  float v[EPL];
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) v[j] = Elem<T>::load(src[j]);
+  if (h >= heads + kv_heads) {   // a value head: transposed inside the page
+    const int hk = h - heads - kv_heads;
+    T* dst = pages + (((int64_t)write_page[t] * 2 + 1) * kv_heads + hk) * (int64_t)page_size * D + write_off[t];
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) dst[(int64_t)(lane * EPL + j) * page_size] = src[j];
+    return;
+  }
+  const bool is_q = h < heads;
+  const T* weight = is_q ? q_weight : k_weight;
+  if (weight != nullptr) {
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) ss += v[j] * v[j];
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) v[j] = Elem<T>::round((v[j] * inv) * Elem<T>::load(weight[lane * EPL + j]));
+  }
+  if (table != nullptr) {
+    const float* cs = table + (int64_t)positions[t] * D;
+    const int i0 = (lane % 32) * EPL;   // index of the pair within the half
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+      const float other = __shfl_xor(v[j], 32, WAVE);
+      const float co = cs[i0 + j], si = cs[D / 2 + i0 + j];
+      v[j] = lane < 32 ? v[j] * co - other * si : v[j] * co + other * si;
+    }
+  }
+  T* dst = is_q ? q_out + ((int64_t)t * heads + h) * D + lane * EPL
+                : pages + (((int64_t)write_page[t] * 2 + 0) * kv_heads + (h - heads)) * (int64_t)page_size * D +
+                      (int64_t)write_off[t] * D + lane * EPL;
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) dst[j] = Elem<T>::store(v[j]);
+}
+
 extern "C" int holon_qk_norm_rope_write(const void* qkv, int64_t qkv_stride, void* q_out, int tokens, int heads,
                                         int kv_heads, int head_dim, const void* q_weight, const void* k_weight,
                                         float eps, const float* table, int rotary_dim, int max_positions,
@@ -281,6 +369,21 @@ extern "C" int holon_qk_norm_rope_write(const void* qkv, int64_t qkv_stride, voi
   const int total_heads = pages != nullptr ? heads + 2 * kv_heads : heads;
   dim3 grid(tokens, (total_heads + 3) / 4);
   hipStream_t s = (hipStream_t)stream;
+  if ((head_dim == 64 || head_dim == 128 || head_dim == 256) && (table == nullptr || rotary_dim == head_dim) &&
+      qkv != q_out) {
+#define QK_FAST(T, EPL)                                                                                            \
+  qk_norm_rope_write_fast_kernel<T, EPL><<<grid, 4 * WAVE, 0, s>>>(                                                 \
+      (const T*)qkv, qkv_stride, (T*)q_out, heads, kv_heads, (const T*)q_weight, (const T*)k_weight, eps, table,    \
+      positions, (T*)pages, write_page, write_off, page_size, total_heads)
+    if (dtype == HOLON_F32) {
+      if (head_dim == 64) QK_FAST(float, 1); else if (head_dim == 128) QK_FAST(float, 2); else QK_FAST(float, 4);
+    } else {
+      if (head_dim == 64) QK_FAST(bf16_t, 1); else if (head_dim == 128) QK_FAST(bf16_t, 2); else QK_FAST(bf16_t, 4);
+    }
+#undef QK_FAST
+    HOLON_LAUNCH_OK();
+    return 0;
+  }
 #define QK_LAUNCH(T)                                                                                              \
   qk_norm_rope_write_kernel<T><<<grid, 4 * WAVE, 0, s>>>((const T*)qkv, qkv_stride, (T*)q_out, heads, kv_heads,    \
                                                         head_dim, (const T*)q_weight, (const T*)k_weight, eps,    \
