@@ -326,11 +326,19 @@ __global__ void __launch_bounds__(64) attn_merge_kernel(const float* __restrict_
   for (int base = 0; base < head_dim; base += 4 * WAVE) {   // every lane walks the loop: the shuffles read all lanes
     const int d0 = base + 4 * lane;
     const bool mine = d0 < head_dim;
+    const float* src = po + (mine ? d0 : 0);
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 8
-    for (int s = 0; s < splits; ++s) {
-      const float w = __shfl(w_s, s, WAVE);
-      if (mine && w > 0.f) acc += w * *reinterpret_cast<const f32x4_t*>(po + (int64_t)s * head_dim + d0);
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+      // eight partials requested at once (unconditionally: an empty split's values are dropped below, not skipped,
+      // so that the loads do not wait for one another)
+      f32x4_t v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const f32x4_t*>(src + (int64_t)min(s0 + i, splits - 1) * head_dim);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float w = __shfl(w_s, min(s0 + i, splits - 1), WAVE);
+        if (s0 + i < splits && w > 0.f) acc += w * v[i];
+      }
     }
     if (mine) {
       ushort4 o;

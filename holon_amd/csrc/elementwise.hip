@@ -75,6 +75,13 @@ __global__ void __launch_bounds__(256) rmsnorm_row_kernel(const T* __restrict__ 
   uint4* rr = ADD ? reinterpret_cast<uint4*>(residual + row * dim) : nullptr;
   float vals[VPT][V];
   float ss = 0.f;
+  const uint4* wr = reinterpret_cast<const uint4*>(weight);
+  uint4 wraw[VPT];                              // requested now, needed after the reduction
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int v = threadIdx.x + i * 256;
+    if (v < nvec) wraw[i] = wr[v];
+  }
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int v = threadIdx.x + i * 256;
@@ -103,14 +110,12 @@ __global__ void __launch_bounds__(256) rmsnorm_row_kernel(const T* __restrict__ 
   __syncthreads();
   ss = ((part[0] + part[1]) + part[2]) + part[3];
   const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
-  const uint4* wr = reinterpret_cast<const uint4*>(weight);
   uint4* yr = reinterpret_cast<uint4*>(y + row * dim);
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int v = threadIdx.x + i * 256;
     if (v < nvec) {
-      const uint4 wraw = wr[v];
-      const T* we = reinterpret_cast<const T*>(&wraw);
+      const T* we = reinterpret_cast<const T*>(&wraw[i]);
       uint4 out;
       T* oe = reinterpret_cast<T*>(&out);
 #pragma unroll

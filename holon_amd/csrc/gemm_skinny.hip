@@ -153,6 +153,125 @@ extern "C" int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int
   return 0;
 }
 
+// The gated form: w = [gate rows; up rows] (2I rows), y[M, I] = round(silu(round(x gate^T))) * round(x up^T), the
+// roundings of the two-kernel composition. A block owns gate tile t and up tile t + I/16 and streams both.
+template <int MT, int WPB, int UNROLL, bool TILED>
+__global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t* __restrict__ x,
+                                                                    const bf16_t* __restrict__ w,
+                                                                    bf16_t* __restrict__ y, int M, int I, int K) {
+  __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * 2 * MT * WAVE : 1];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int g = lane / 16, c = lane % 16;
+  const int n0 = blockIdx.x * 16;
+  const int kw = K / WPB, steps = kw / 32;
+  const bf16_t* wp[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int64_t tile = blockIdx.x + (int64_t)h * (I / 16);
+    wp[h] = TILED ? w + (tile * (K / 32) + (int64_t)wave * steps) * 512 + lane * 8
+                  : w + (tile * 16 + c) * K + (int64_t)wave * kw + 8 * g;
+  }
+  constexpr int WSTEP = TILED ? 512 : 32;
+  const bf16_t* xp = x + (int64_t)c * K + (int64_t)wave * kw + 8 * g;
+  f32x4_t acc[2][MT];
+  bool have[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    acc[0][t] = acc[1][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    have[t] = t * 16 + c < M;
+  }
+  int s = 0;
+  for (; s + UNROLL <= steps; s += UNROLL) {
+    bf16x8_t wf[2][UNROLL], xf[UNROLL][MT];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u)
+        wf[h][u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp[h] + (int64_t)(s + u) * WSTEP));
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        if (have[t]) {
+          xf[u][t] = *reinterpret_cast<const bf16x8_t*>(xp + (int64_t)t * 16 * K + (s + u) * 32);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) xf[u][t][i] = (__bf16)0.f;
+        }
+      }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[0][u], xf[u][t], acc[0][t], 0, 0, 0);
+        acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[1][u], xf[u][t], acc[1][t], 0, 0, 0);
+      }
+  }
+  for (; s < steps; ++s) {
+    const bf16x8_t w0 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp[0] + (int64_t)s * WSTEP));
+    const bf16x8_t w1 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp[1] + (int64_t)s * WSTEP));
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      bf16x8_t xf;
+      if (have[t]) {
+        xf = *reinterpret_cast<const bf16x8_t*>(xp + (int64_t)t * 16 * K + s * 32);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xf[i] = (__bf16)0.f;
+      }
+      acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, xf, acc[0][t], 0, 0, 0);
+      acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, xf, acc[1][t], 0, 0, 0);
+    }
+  }
+  if (WPB > 1) {
+    if (wave > 0) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) red[(((wave - 1) * 2 + h) * MT + t) * WAVE + lane] = acc[h][t];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    for (int ww = 1; ww < WPB; ++ww)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[h][t] += red[(((ww - 1) * 2 + h) * MT + t) * WAVE + lane];
+  }
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + c;
+    if (m >= M) continue;
+    ushort4 o;
+    bf16_t* oe = reinterpret_cast<bf16_t*>(&o);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float gate = bf16_to_float(float_to_bf16(acc[0][t][r]));
+      const float up = bf16_to_float(float_to_bf16(acc[1][t][r]));
+      const float sg = bf16_to_float(float_to_bf16(gate / (1.0f + expf(-gate))));
+      oe[r] = float_to_bf16(sg * up);
+    }
+    *reinterpret_cast<ushort4*>(y + (int64_t)m * I + n0 + 4 * g) = o;
+  }
+}
+
+extern "C" int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int I, int K, int tiled,
+                                          void* stream) {
+  HOLON_CHECK(M >= 1 && M <= 32 && I % 16 == 0 && K % 128 == 0, "gated gemm (few rows): M=%d I=%d K=%d not served", M, I, K);
+  hipStream_t s = (hipStream_t)stream;
+  const bool few = I / 16 < 512;   // few tile pairs: four waves share each
+#define GLU(MT, WPB, U)                                                                                              \
+  if (tiled) gemm_skinny_glu_kernel<MT, WPB, U, true><<<I / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, \
+                                                                                 (bf16_t*)y, M, I, K);               \
+  else gemm_skinny_glu_kernel<MT, WPB, U, false><<<I / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,      \
+                                                                            (bf16_t*)y, M, I, K)
+  if (M <= 16) { if (few) { GLU(1, 4, 8); } else { GLU(1, 1, 8); } }
+  else { if (few) { GLU(2, 4, 4); } else { GLU(2, 1, 4); } }
+#undef GLU
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
 // tiled[t][s][l][e] = w[16 t + l % 16][32 s + 8 (l / 16) + e]: the layout the few-row product streams.
 __global__ void tile_weight_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ tiled, int N, int K) {
   const int64_t chunks = (int64_t)N * K / 8;

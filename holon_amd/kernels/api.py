@@ -60,6 +60,10 @@ class Kernels(Protocol):
     def tile_weight(self, weight: torch.Tensor) -> torch.Tensor | None:
         """Once per weight after loading: a copy in the layout steps of few rows stream fastest, or None."""
 
+    def linear_silu_mul(self, x: torch.Tensor, weight: torch.Tensor, tiled: torch.Tensor | None = None
+                        ) -> torch.Tensor | None:
+        """silu_mul(linear(x, weight)) fused, bit for bit the composition; None when not fused for this shape."""
+
     def silu_mul(self, gate_up: torch.Tensor) -> torch.Tensor:
         """gate_up [T, 2I] (gate columns first) -> [T, I] = round(silu(gate)) * up."""
 

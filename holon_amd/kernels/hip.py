@@ -67,6 +67,7 @@ class HipKernels:
             "holon_gemm_skinny_supported": [_I, _I, _I],
             "holon_gemm_skinny_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
             "holon_tile_weight_bf16": [_P, _P, _I, _I, _P],
+            "holon_gemm_skinny_glu_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
             "holon_argmax": [_P, _P, _I, _I, _P],
             "holon_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
         }
@@ -159,6 +160,20 @@ class HipKernels:
         # the vendor library's product, float32 accumulation (no reduced-precision mode for float32 operands)
         y = torch.matmul(x, weight.t())
         return y if out_dtype in (None, y.dtype) else y.to(out_dtype)
+
+    def linear_silu_mul(self, x, weight, tiled=None):
+        """silu_mul(linear(x, weight)) in one kernel for steps of few rows, with the roundings of the two kernels one
+        after the other; None when this shape is not fused (the caller then composes the two)."""
+        m, k = x.shape
+        two_i = weight.shape[0]
+        if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows
+                and two_i % 32 == 0 and k % 128 == 0 and k >= 256 and weight.shape[1] == k and x.is_contiguous()):
+            return None
+        y = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
+        source = tiled if tiled is not None else weight
+        self._call(self.lib.holon_gemm_skinny_glu_bf16, x.data_ptr(), source.data_ptr(), y.data_ptr(), m, two_i // 2, k,
+                   int(tiled is not None), self._stream())
+        return y
 
     def silu_mul(self, gate_up):
         self._check(gate_up, "silu_mul")

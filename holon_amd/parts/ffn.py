@@ -27,6 +27,9 @@ class SwiGLU(Part):
         self._children["gate_up"] = self.gate_up
 
     def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
-        return self.down_proj(self.kernels.silu_mul(self.gate_up(x)))
+        y = self.kernels.linear_silu_mul(x, self.gate_up.weight, self.gate_up.tiled)   # fused for steps of few rows
+        if y is None:
+            y = self.kernels.silu_mul(self.gate_up(x))
+        return self.down_proj(y)
 
     __call__ = forward

@@ -58,6 +58,9 @@ class TorchKernels:
     def linear(self, x, weight, out_dtype=None, tiled=None):
         return (_up(x) @ _up(weight).T).to(out_dtype or x.dtype)
 
+    def linear_silu_mul(self, x, weight, tiled=None):
+        return None
+
     def silu_mul(self, gate_up):
         gate, up = gate_up.chunk(2, dim=-1)
         return torch.nn.functional.silu(_up(gate)).to(gate.dtype) * up
