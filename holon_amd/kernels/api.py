@@ -62,7 +62,7 @@ class Kernels(Protocol):
 
     def linear_silu_mul(self, x: torch.Tensor, weight: torch.Tensor, tiled: torch.Tensor | None = None
                         ) -> torch.Tensor | None:
-        """silu_mul(linear(x, weight)) fused, bit for bit the composition; None when not fused for this shape."""
+        """silu_mul(linear(x, weight)) fused, with the composition's roundings; None when not fused for this shape."""
 
     def silu_mul(self, gate_up: torch.Tensor) -> torch.Tensor:
         """gate_up [T, 2I] (gate columns first) -> [T, I] = round(silu(gate)) * up."""

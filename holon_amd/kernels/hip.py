@@ -163,7 +163,7 @@ class HipKernels:
 
     def linear_silu_mul(self, x, weight, tiled=None):
         """silu_mul(linear(x, weight)) in one kernel for steps of few rows, with the roundings of the two kernels one
-        after the other; None when this shape is not fused (the caller then composes the two)."""
+        after the other (the sums over K may be split differently); None when this shape is not fused (the caller then composes the two)."""
         m, k = x.shape
         two_i = weight.shape[0]
         if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows

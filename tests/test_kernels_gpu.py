@@ -232,11 +232,17 @@ def test_fused_gate_up_is_the_two_kernels(hip, monkeypatch):
     for m, k, inter in ((1, 4096, 12288), (8, 4096, 12288), (16, 512, 208), (3, 1024, 1024), (5, 256, 48)):
         x = _randn(m, k, dtype=torch.bfloat16, seed=30)
         w = _randn(2 * inter, k, dtype=torch.bfloat16, seed=31, scale=0.05)
+        exact = PLAIN.silu_mul(PLAIN.linear(x.double(), w.double()))
         want = hip.silu_mul(hip.linear(x, w))
+        assert H.op_budget_usage(want, exact, torch.bfloat16, k) <= 1
+        both = []
         for tiled in (None, hip.tile_weight(w)):
             got = hip.linear_silu_mul(x, w, tiled)
-            assert got is not None and torch.equal(got, want), (m, k, inter, tiled is not None)
-        assert H.op_budget_usage(want, PLAIN.silu_mul(PLAIN.linear(x, w)).double(), torch.bfloat16, k) <= 1
+            assert got is not None and H.op_budget_usage(got, exact, torch.bfloat16, k) <= 1, (m, k, inter)
+            # the same roundings as the two kernels; the sums over K may be split differently
+            assert (got != want).float().mean() < 0.02
+            both.append(got)
+        assert torch.equal(both[0], both[1])           # the tile layout is a permutation of the same reads
     assert hip.linear_silu_mul(_randn(40, 256, dtype=torch.bfloat16), _randn(64, 256, dtype=torch.bfloat16)) is None
     assert hip.linear_silu_mul(_randn(4, 256, dtype=torch.float32), _randn(64, 256, dtype=torch.float32)) is None
 
