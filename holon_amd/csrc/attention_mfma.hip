@@ -248,6 +248,214 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
   }
 }
 
+// Prompt portions, staged through LDS: a block of four waves owns 4*NT consecutive tiles (for four heads a group: 32
+// positions with NT = 2) and walks the keys in stages of 32; each stage's keys and transposed values are copied from
+// the pages into LDS once per block (double buffered: the next stage's loads are in flight while this one is
+// multiplied) and every wave takes its matrix-core operands from there, so a key is read from the cache once per
+// block, not once per wave. Keys are stored in LDS in the order the two score products want their rows (lane c reads
+// row c, then row 16 + c), which with a row pitch of D + 8 makes the 16-byte reads conflict-free; value rows have a
+// pitch of 40. To even out the causal mask, a block does two position ranges: the b-th from the start and the b-th
+// from the end.
+template <int D, int NT>
+__global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
+  constexpr int KP = D + 8;    // pitch of a key row in LDS (elements)
+  constexpr int VP = 40;       // pitch of a value row: 32 keys + 8
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][32 * KP];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][D * VP];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, tid = threadIdx.x;
+  const int g = lane / 16, c = lane % 16;
+  const int b = a.row_ids[blockIdx.z];
+  const int group = a.heads / a.kv_heads;
+  const TileMap tm = tile_map(group);
+  const int hk = blockIdx.y / tm.head_blocks, hb = blockIdx.y % tm.head_blocks;
+  const int qs = a.qstart[b], nq = a.qstart[b + 1] - qs, n = a.lens[b];
+  const int n_tiles = (nq + tm.pos_per_tile - 1) / tm.pos_per_tile;
+  constexpr int TPB = 4 * NT;                                  // tiles a block owns per range
+  const int n_ranges = (n_tiles + TPB - 1) / TPB;
+  if (n <= 0 || (int)blockIdx.x >= (n_ranges + 1) / 2) return;   // uniform over the block
+  const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
+  const int P = a.page_size;
+  const int64_t plane = (int64_t)P * D;
+  const int64_t page_stride = 2 * (int64_t)a.kv_heads * plane;
+  const bf16_t* kbase = a.pages + (int64_t)hk * plane;
+  const bf16_t* vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
+  const int max_page = a.table_stride - 1;
+
+  // this thread's share of a stage's copy: 2 chunks of keys and 2 of values, 16 bytes each
+  constexpr int KCH = D / 8;                                   // chunks per key row
+  int k_key[2], k_col[2], k_dst[2], v_d[2], v_kc[2], v_dst[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = tid + 256 * i;
+    if (KCH * 32 > 256 * i + tid) {
+      k_key[i] = q / KCH;
+      k_col[i] = (q % KCH) * 8;
+    } else {
+      k_key[i] = -1;
+      k_col[i] = 0;
+    }
+    const int j = k_key[i] < 0 ? 0 : k_key[i];
+    const int row = (j % 8 < 4) ? 4 * (j / 8) + j % 8 : 16 + 4 * (j / 8) + (j % 8 - 4);
+    k_dst[i] = row * KP + k_col[i];
+    v_d[i] = (D * 4 > q) ? q / 4 : -1;                         // 4 chunks of 8 keys per value row
+    v_kc[i] = q % 4;
+    v_dst[i] = (v_d[i] < 0 ? 0 : v_d[i]) * VP + v_kc[i] * 8;
+  }
+  // D = 64: 256 key chunks and 256 value chunks, one round; D = 128: two rounds each; D = 256 would need four
+  static_assert(D == 64 || D == 128, "the LDS kernel copies at most two chunks of each kind per thread");
+
+  for (int pass = 0; pass < 2; ++pass) {
+    const int range = pass == 0 ? (int)blockIdx.x : n_ranges - 1 - (int)blockIdx.x;
+    if (pass == 1 && range <= (int)blockIdx.x) break;          // an odd count: the middle range was done in pass 0
+    bf16x8_t qf[NT][D / 32];
+    int qpos[NT], tile_last[NT];
+    RowRef rr[NT];
+    int key_hi = -1, key_lo = 0x7fffffff;                      // over the whole block (all waves walk the same stages)
+    {
+      const int p_lo = range * TPB * tm.pos_per_tile;
+      const int p_hi = min(nq, p_lo + TPB * tm.pos_per_tile) - 1;
+      key_hi = n - nq + p_hi;
+      key_lo = a.window > 0 ? max(0, n - nq + p_lo - a.window + 1) : 0;
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int tile = range * TPB + wave * NT + t;
+      const int p0 = tile * tm.pos_per_tile;
+      rr[t] = row_ref(tm, c, p0, hb, hk, group, qs, nq, n);
+      qpos[t] = rr[t].valid ? rr[t].qpos : -1;
+      tile_last[t] = p0 < nq ? n - nq + min(nq, p0 + tm.pos_per_tile) - 1 : -1;
+      const bf16_t* qp = a.q + ((int64_t)rr[t].token * a.heads + rr[t].head) * D + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < D / 32; ++ks) {
+        if (rr[t].valid) {
+          qf[t][ks] = load8(qp + ks * 32);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) qf[t][ks][i] = (__bf16)0.f;
+        }
+      }
+    }
+    f32x4_t o[NT][D / 16];
+    float m[NT], l[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      m[t] = -INFINITY;
+      l[t] = 0.f;
+#pragma unroll
+      for (int ds = 0; ds < D / 16; ++ds) o[t][ds] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    bf16x8_t kreg[2], vreg[2];
+    auto fetch = [&](int kb) {   // this thread's chunks of stage kb, into registers
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if (k_key[i] >= 0) {
+          const int key = kb + k_key[i];
+          kreg[i] = load8(kbase + (int64_t)trow[min(key / P, max_page)] * page_stride + (int64_t)(key % P) * D + k_col[i]);
+        }
+        if (v_d[i] >= 0) {
+          const int key = kb + v_kc[i] * 8;
+          vreg[i] = load8(vbase + (int64_t)trow[min(key / P, max_page)] * page_stride + (int64_t)v_d[i] * P + key % P);
+        }
+      }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if (k_key[i] >= 0) *reinterpret_cast<bf16x8_t*>(&k_lds[buf][k_dst[i]]) = kreg[i];
+        if (v_d[i] >= 0) *reinterpret_cast<bf16x8_t*>(&v_lds[buf][v_dst[i]]) = vreg[i];
+      }
+    };
+    const int kb_first = (key_lo / 32) * 32;
+    __syncthreads();             // the previous pass has finished reading both buffers
+    fetch(kb_first);
+    stash(0);
+    __syncthreads();
+    int buf = 0;
+    for (int kb = kb_first; kb <= key_hi; kb += 32, buf ^= 1) {
+      const bool more = kb + 32 <= key_hi;
+      if (more) fetch(kb + 32);
+      bool any = false;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) any = any || kb <= tile_last[t];
+      if (any) {
+        bf16x8_t kf0[D / 32], kf1[D / 32];
+#pragma unroll
+        for (int ks = 0; ks < D / 32; ++ks) {
+          kf0[ks] = *reinterpret_cast<const bf16x8_t*>(&k_lds[buf][c * KP + ks * 32 + 8 * g]);
+          kf1[ks] = *reinterpret_cast<const bf16x8_t*>(&k_lds[buf][(16 + c) * KP + ks * 32 + 8 * g]);
+        }
+        bf16x8_t pb[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          if (kb > tile_last[t]) continue;
+          f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < D / 32; ++ks) {
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf0[ks], qf[t][ks], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf1[ks], qf[t][ks], s1, 0, 0, 0);
+          }
+          const int qp = qpos[t];
+          const int first = a.window > 0 ? qp - a.window + 1 : 0;
+          float sv[8];
+          float mx = -INFINITY;
+#pragma unroll
+          for (int r = 0; r < 8; ++r) {
+            const int key = kb + 8 * g + r;
+            const float v = (r < 4 ? s0[r] : s1[r - 4]) * a.scale_log2;
+            sv[r] = (key <= qp && key >= first) ? v : -INFINITY;
+            mx = fmaxf(mx, sv[r]);
+          }
+          mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+          mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+          const float m_new = fmaxf(m[t], mx);
+          const float m_use = m_new == -INFINITY ? 0.f : m_new;
+          const float alpha = exp2f(m[t] - m_use);
+          m[t] = m_new;
+          float psum = 0.f;
+#pragma unroll
+          for (int r = 0; r < 8; ++r) {
+            const float p = exp2f(sv[r] - m_use);
+            psum += p;
+            pb[t][r] = (__bf16)p;
+          }
+          l[t] = l[t] * alpha + psum;
+#pragma unroll
+          for (int ds = 0; ds < D / 16; ++ds) o[t][ds] *= alpha;
+        }
+#pragma unroll
+        for (int ds = 0; ds < D / 16; ++ds) {
+          const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(ds * 16 + c) * VP + 8 * g]);
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            if (kb > tile_last[t]) continue;
+            o[t][ds] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[t], o[t][ds], 0, 0, 0);
+          }
+        }
+      }
+      if (more) stash(buf ^ 1);
+      __syncthreads();
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      float lt = l[t];
+      lt += __shfl_xor(lt, 16, WAVE);
+      lt += __shfl_xor(lt, 32, WAVE);
+      if (!rr[t].valid) continue;
+      const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+      bf16_t* op = a.out + ((int64_t)rr[t].token * a.heads + rr[t].head) * D + 4 * g;
+#pragma unroll
+      for (int ds = 0; ds < D / 16; ++ds) {
+        ushort4 w;
+        w.x = float_to_bf16(o[t][ds][0] * inv);
+        w.y = float_to_bf16(o[t][ds][1] * inv);
+        w.z = float_to_bf16(o[t][ds][2] * inv);
+        w.w = float_to_bf16(o[t][ds][3] * inv);
+        *reinterpret_cast<ushort4*>(op + ds * 16) = w;
+      }
+    }
+  }
+}
+
 // Decode rows: block (split, kv head x head block, row), one wave. Partials go to part_o / part_ml.
 template <int D>
 __global__ void __launch_bounds__(64) attn_decode_kernel(AttnArgs a) {
@@ -375,6 +583,14 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
   const TileMap tm = tile_map(heads / kv_heads);
   const int nt = head_dim == 256 ? 1 : 2;
   const int tiles = (max_query + tm.pos_per_tile - 1) / tm.pos_per_tile;
+  if (head_dim != 256 && tiles >= 16) {   // long portions: keys and values staged through LDS, shared by four waves
+    const int ranges = (tiles + 4 * nt - 1) / (4 * nt);
+    dim3 lgrid((ranges + 1) / 2, kv_heads * tm.head_blocks, n_rows);
+    if (head_dim == 64) attn_prefill_lds_kernel<64, 2><<<lgrid, 256, 0, (hipStream_t)stream>>>(a);
+    else attn_prefill_lds_kernel<128, 2><<<lgrid, 256, 0, (hipStream_t)stream>>>(a);
+    HOLON_LAUNCH_OK();
+    return 0;
+  }
   dim3 grid(((tiles + nt - 1) / nt + 3) / 4, kv_heads * tm.head_blocks, n_rows);
   hipStream_t s = (hipStream_t)stream;
   if (head_dim == 64) attn_prefill_kernel<64, 2><<<grid, 256, 0, s>>>(a);
