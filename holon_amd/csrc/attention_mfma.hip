@@ -248,6 +248,10 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
   }
 }
 
+// A barrier that waits for this wave's LDS traffic only. __syncthreads() also waits for every global load in flight
+// (vmcnt(0)), which would make each stage wait for the loads it has just requested for a later stage.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Prompt portions, staged through LDS: a block of four waves owns 4*NT consecutive tiles (for four heads a group: 32
 // positions with NT = 2) and walks the keys in stages of 32; each stage's keys and transposed values are copied from
 // the pages into LDS once per block (double buffered: the next stage's loads are in flight while this one is
@@ -262,6 +266,8 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
   constexpr int VP = 40;       // pitch of a value row: 32 keys + 8
   __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][32 * KP];
   __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][D * VP];
+  constexpr int PG = 4096;     // the row's first block-table entries, kept in LDS: page lookups then do not queue
+  __shared__ int32_t pg_lds[PG];   // behind the vector loads in flight
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, tid = threadIdx.x;
   const int g = lane / 16, c = lane % 16;
   const int b = a.row_ids[blockIdx.z];
@@ -279,30 +285,28 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
   const int64_t page_stride = 2 * (int64_t)a.kv_heads * plane;
   const bf16_t* kbase = a.pages + (int64_t)hk * plane;
   const bf16_t* vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
-  const int max_page = a.table_stride - 1;
+  const int max_page = min(a.table_stride, PG) - 1;
 
-  // this thread's share of a stage's copy: 2 chunks of keys and 2 of values, 16 bytes each
+  // every entry a stage can ask for: the last stage's second half may lie one page past the row's tokens (the table
+  // holds a valid page id there, the null page or any other: the keys are masked), so the whole row is copied
+  for (int i = tid; i < min(PG, a.table_stride); i += 256) pg_lds[i] = trow[i];
+  // this thread's share of a stage's copy: D/64 chunks of keys and as many of values, 16 bytes each
   constexpr int KCH = D / 8;                                   // chunks per key row
-  int k_key[2], k_col[2], k_dst[2], v_d[2], v_kc[2], v_dst[2];
+  constexpr int ROUNDS = D / 64;                               // 32 keys x D and D x 32 values: 4 D chunks each, 256 threads
+  static_assert(D == 64 || D == 128, "the LDS kernel copies one or two chunks of each kind per thread");
+  int k_key[ROUNDS], k_col[ROUNDS], k_dst[ROUNDS], v_d[ROUNDS], v_kc[ROUNDS], v_dst[ROUNDS];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < ROUNDS; ++i) {
     const int q = tid + 256 * i;
-    if (KCH * 32 > 256 * i + tid) {
-      k_key[i] = q / KCH;
-      k_col[i] = (q % KCH) * 8;
-    } else {
-      k_key[i] = -1;
-      k_col[i] = 0;
-    }
-    const int j = k_key[i] < 0 ? 0 : k_key[i];
+    k_key[i] = q / KCH;
+    k_col[i] = (q % KCH) * 8;
+    const int j = k_key[i];
     const int row = (j % 8 < 4) ? 4 * (j / 8) + j % 8 : 16 + 4 * (j / 8) + (j % 8 - 4);
     k_dst[i] = row * KP + k_col[i];
-    v_d[i] = (D * 4 > q) ? q / 4 : -1;                         // 4 chunks of 8 keys per value row
+    v_d[i] = q / 4;                                            // 4 chunks of 8 keys per value row
     v_kc[i] = q % 4;
-    v_dst[i] = (v_d[i] < 0 ? 0 : v_d[i]) * VP + v_kc[i] * 8;
+    v_dst[i] = v_d[i] * VP + v_kc[i] * 8;
   }
-  // D = 64: 256 key chunks and 256 value chunks, one round; D = 128: two rounds each; D = 256 would need four
-  static_assert(D == 64 || D == 128, "the LDS kernel copies at most two chunks of each kind per thread");
 
   for (int pass = 0; pass < 2; ++pass) {
     const int range = pass == 0 ? (int)blockIdx.x : n_ranges - 1 - (int)blockIdx.x;
@@ -344,36 +348,38 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
 #pragma unroll
       for (int ds = 0; ds < D / 16; ++ds) o[t][ds] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
-    bf16x8_t kreg[2], vreg[2];
-    auto fetch = [&](int kb) {   // this thread's chunks of stage kb, into registers
+    // Two register sets keep the loads of the next two stages in flight (a load from the cache takes longer than a
+    // stage's products; with one block per compute unit nothing else hides it). No branches around the loads: a
+    // stage past the end re-reads the last one.
+    struct Regs { bf16x8_t k[ROUNDS], v[ROUNDS]; };
+    Regs r0, r1;
+    const int kb_last = (key_hi / 32) * 32;
+    auto fetch = [&](int kb_want, Regs& r) {   // this thread's chunks of a stage, into registers
+      const int kb = min(kb_want, kb_last);
+      // a stage is two groups of 16 keys, each inside one page: two table entries, the same for every thread (scalar
+      // loads, which do not queue behind the vector loads in flight)
+      const int i0 = min(kb / P, max_page), i1 = min((kb + 16) / P, max_page);   // (kb <= key_hi < n: inside the row)
+      const int64_t pg0 = (int64_t)pg_lds[i0] * page_stride;   // (the host sends longer rows to the other kernel)
+      const int64_t pg1 = (int64_t)pg_lds[i1] * page_stride;
+      const int off0 = kb % P, off1 = (kb + 16) % P;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        if (k_key[i] >= 0) {
-          const int key = kb + k_key[i];
-          kreg[i] = load8(kbase + (int64_t)trow[min(key / P, max_page)] * page_stride + (int64_t)(key % P) * D + k_col[i]);
-        }
-        if (v_d[i] >= 0) {
-          const int key = kb + v_kc[i] * 8;
-          vreg[i] = load8(vbase + (int64_t)trow[min(key / P, max_page)] * page_stride + (int64_t)v_d[i] * P + key % P);
-        }
+      for (int i = 0; i < ROUNDS; ++i) {
+        const bool hi = k_key[i] >= 16;
+        r.k[i] = load8(kbase + (hi ? pg1 : pg0) + (int64_t)((hi ? off1 - 16 : off0) + k_key[i]) * D + k_col[i]);
+        const bool vhi = v_kc[i] >= 2;
+        r.v[i] = load8(vbase + (vhi ? pg1 : pg0) + (int64_t)v_d[i] * P + (vhi ? off1 : off0) + 8 * (v_kc[i] % 2));
       }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](int buf, const Regs& r) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        if (k_key[i] >= 0) *reinterpret_cast<bf16x8_t*>(&k_lds[buf][k_dst[i]]) = kreg[i];
-        if (v_d[i] >= 0) *reinterpret_cast<bf16x8_t*>(&v_lds[buf][v_dst[i]]) = vreg[i];
+      for (int i = 0; i < ROUNDS; ++i) {
+        *reinterpret_cast<bf16x8_t*>(&k_lds[buf][k_dst[i]]) = r.k[i];
+        *reinterpret_cast<bf16x8_t*>(&v_lds[buf][v_dst[i]]) = r.v[i];
       }
     };
-    const int kb_first = (key_lo / 32) * 32;
-    __syncthreads();             // the previous pass has finished reading both buffers
-    fetch(kb_first);
-    stash(0);
-    __syncthreads();
-    int buf = 0;
-    for (int kb = kb_first; kb <= key_hi; kb += 32, buf ^= 1) {
-      const bool more = kb + 32 <= key_hi;
-      if (more) fetch(kb + 32);
+    // One stage: LDS buffer `buf` holds the keys kb .. kb+31. `next` holds stage kb+32, which goes to the other
+    // buffer after the products and is then refilled with stage kb+96 (`other` holds kb+64 meanwhile).
+    auto stage = [&](int kb, int buf, Regs& next) {
       bool any = false;
 #pragma unroll
       for (int t = 0; t < NT; ++t) any = any || kb <= tile_last[t];
@@ -432,8 +438,20 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
           }
         }
       }
-      if (more) stash(buf ^ 1);
-      __syncthreads();
+      stash(buf ^ 1, next);
+      fetch(kb + 96, next);
+      lds_barrier();
+    };
+    const int kb_first = (key_lo / 32) * 32;
+    lds_barrier();               // the previous pass has finished reading both buffers
+    fetch(kb_first, r0);
+    fetch(kb_first + 32, r1);
+    stash(0, r0);
+    fetch(kb_first + 64, r0);
+    lds_barrier();
+    for (int kb = kb_first; kb <= key_hi; kb += 64) {   // even stages: buffer 0, next in r1; odd stages: buffer 1, r0
+      stage(kb, 0, r1);
+      if (kb + 32 <= key_hi) stage(kb + 32, 1, r0);
     }
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -568,8 +586,8 @@ extern "C" int holon_attention_mfma_supported(int head_dim, int page_size, int d
 extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void* pages, const int32_t* table,
                                             int table_stride, const int32_t* slots, const int32_t* lens,
                                             const int32_t* query_start, const int32_t* row_ids, int n_rows,
-                                            int max_query, int heads, int kv_heads, int head_dim, int page_size,
-                                            float scale, int window, void* stream) {
+                                            int max_query, int max_len, int heads, int kv_heads, int head_dim,
+                                            int page_size, float scale, int window, void* stream) {
   HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
@@ -583,7 +601,8 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
   const TileMap tm = tile_map(heads / kv_heads);
   const int nt = head_dim == 256 ? 1 : 2;
   const int tiles = (max_query + tm.pos_per_tile - 1) / tm.pos_per_tile;
-  if (head_dim != 256 && tiles >= 16) {   // long portions: keys and values staged through LDS, shared by four waves
+  if (head_dim != 256 && tiles >= 16 && max_len <= 4096 * page_size) {
+    // long portions: keys and values staged through LDS, shared by four waves (rows of up to 4096 pages)
     const int ranges = (tiles + 4 * nt - 1) / (4 * nt);
     dim3 lgrid((ranges + 1) / 2, kv_heads * tm.head_blocks, n_rows);
     if (head_dim == 64) attn_prefill_lds_kernel<64, 2><<<lgrid, 256, 0, (hipStream_t)stream>>>(a);

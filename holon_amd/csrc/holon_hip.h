@@ -34,8 +34,8 @@ int holon_attention_generic(const void* q, void* out, const void* pages, const i
 int holon_attention_mfma_supported(int head_dim, int page_size, int dtype);
 int holon_attention_prefill_bf16(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
                                  const int32_t* slots, const int32_t* lens, const int32_t* query_start,
-                                 const int32_t* row_ids, int n_rows, int max_query, int heads, int kv_heads,
-                                 int head_dim, int page_size, float scale, int window, void* stream);
+                                 const int32_t* row_ids, int n_rows, int max_query, int max_len, int heads,
+                                 int kv_heads, int head_dim, int page_size, float scale, int window, void* stream);
 // One query token per row; the keys are split over `splits` waves of `keys_per_split` keys (a multiple of 32) whose
 // partial results (part_o [n_rows, heads, splits, head_dim], part_ml [n_rows, heads, splits, 2], float32) are merged
 // in split order.

@@ -61,7 +61,8 @@ class HipKernels:
             "holon_kv_write": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
             "holon_attention_generic": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
             "holon_attention_mfma_supported": [_I, _I, _I],
-            "holon_attention_prefill_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+            "holon_attention_prefill_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I,
+                                             _P],
             "holon_attention_decode_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P,
                                             _I, _I, _P],
             "holon_gemm_skinny_supported": [_I, _I, _I],
@@ -248,7 +249,8 @@ class HipKernels:
                       rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr())
             if rows.n_chunk:
                 self._call(self.lib.holon_attention_prefill_bf16, *common, rows.chunk_rows.data_ptr(), rows.n_chunk,
-                           rows.max_chunk_query, hq, hkv, d, page_size, float(scale), int(window), self._stream())
+                           rows.max_chunk_query, rows.max_chunk_len, hq, hkv, d, page_size, float(scale), int(window),
+                           self._stream())
             if rows.n_decode:
                 span = rows.max_decode_len if not window else min(rows.max_decode_len, window + 31)
                 splits, per = self.decode_splits(rows.n_decode * hkv * ((hq // hkv + 15) // 16), span)
