@@ -57,13 +57,56 @@ __host__ __device__ inline TileMap tile_map(int group) {
   return m;
 }
 
+// One block of 32 keys for one tile, after the score products: mask (only where the block is not wholly visible),
+// running max and sum, the probabilities as the next product's B operand, and the rescale of what was summed so far
+// (only when some row's max moved: later blocks rarely move it, and the accumulators can then stay where the matrix
+// cores keep them). Lane (g, c): s0[r] is key kb+8g+r against query column c, s1[r] key kb+8g+4+r.
+template <int DS>
+__device__ __forceinline__ bf16x8_t softmax_block(const f32x4_t& s0, const f32x4_t& s1, bool whole, int kb, int g,
+                                                  int qp, int first, int key_lo, int key_hi, float scale_log2,
+                                                  float& m, float& l, f32x4_t (&o)[DS]) {
+  float sv[8];
+#pragma unroll
+  for (int r = 0; r < 8; ++r) sv[r] = (r < 4 ? s0[r] : s1[r - 4]) * scale_log2;
+  if (!whole) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int key = kb + 8 * g + r;
+      if (!(key <= qp && key >= first && key >= key_lo && key <= key_hi)) sv[r] = -INFINITY;
+    }
+  }
+  float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+  mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+  const float m_new = fmaxf(m, mx);
+  const float m_use = m_new == -INFINITY ? 0.f : m_new;   // nothing visible yet: keep everything at zero
+  bf16x8_t pb;
+  float psum = 0.f;
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const float p = __builtin_amdgcn_exp2f(sv[r] - m_use);   // arguments <= 0; results below 2^-126 flush to zero
+    psum += p;
+    pb[r] = (__bf16)p;
+  }
+  if (__any(m_new != m)) {
+    const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+    l *= alpha;
+#pragma unroll
+    for (int ds = 0; ds < DS; ++ds) o[ds] *= alpha;
+    m = m_new;
+  }
+  l += psum;
+  return pb;
+}
+
 // One wave: NT tiles against keys [key_lo, key_hi] (inclusive, as bounded per row by causality and the window).
 // On return o[t][dsub] holds the unnormalised O^T, m[t] the running max (base-2 scaled), l[t] this lane's share of
 // the sum (to be added over the four lane groups).
 template <int D, int NT>
 __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __restrict__ trow, int hk,
                                            const bf16x8_t (&qf)[NT][D / 32], const int (&qpos)[NT],
-                                           const int (&tile_last)[NT], int key_lo, int key_hi,
+                                           const int (&tile_last)[NT], const int (&tile_first)[NT], int key_lo,
+                                           int key_hi,
                                            f32x4_t (&o)[NT][D / 16], float (&m)[NT], float (&l)[NT]) {
   const int lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
@@ -112,34 +155,11 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
         s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf0[ks], qf[t][ks], s0, 0, 0, 0);
         s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf1[ks], qf[t][ks], s1, 0, 0, 0);
       }
-      // lane (g, c): s0[r] is key kb+8g+r against query column c, s1[r] key kb+8g+4+r
       const int qp = qpos[t];
       const int first = a.window > 0 ? qp - a.window + 1 : 0;
-      float sv[8];
-      float mx = -INFINITY;
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        const int key = kb + 8 * g + r;
-        const float v = (r < 4 ? s0[r] : s1[r - 4]) * a.scale_log2;
-        sv[r] = (key <= qp && key >= first && key >= key_lo && key <= key_hi) ? v : -INFINITY;
-        mx = fmaxf(mx, sv[r]);
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-      const float m_new = fmaxf(m[t], mx);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;   // nothing visible yet: keep everything at zero
-      const float alpha = exp2f(m[t] - m_use);
-      m[t] = m_new;
-      float psum = 0.f;
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        const float p = exp2f(sv[r] - m_use);
-        psum += p;
-        pb[t][r] = (__bf16)p;
-      }
-      l[t] = l[t] * alpha + psum;
-#pragma unroll
-      for (int ds = 0; ds < D / 16; ++ds) o[t][ds] *= alpha;
+      const bool whole = kb + 31 <= tile_first[t] && kb >= key_lo && kb + 31 <= key_hi &&
+                         (a.window <= 0 || kb >= tile_last[t] - a.window + 1);
+      pb[t] = softmax_block<D / 16>(s0, s1, whole, kb, g, qp, first, key_lo, key_hi, a.scale_log2, m[t], l[t], o[t]);
     }
 #pragma unroll
     for (int ds = 0; ds < D / 16; ++ds) {
@@ -193,7 +213,7 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
   const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
 
   bf16x8_t qf[NT][D / 32];
-  int qpos[NT], tile_last[NT];
+  int qpos[NT], tile_last[NT], tile_first[NT];   // a tile's rows sit at positions tile_first .. tile_last
   RowRef rr[NT];
   int key_hi = 0, key_lo = 0x7fffffff;
 #pragma unroll
@@ -205,6 +225,7 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
     qpos[t] = rr[t].valid ? rr[t].qpos : -1;   // an unused row sees no key
     const int last_qi = min(nq, p0 + tm.pos_per_tile) - 1;
     tile_last[t] = p0 < nq ? n - nq + last_qi : -1;
+    tile_first[t] = n - nq + p0;
     key_hi = max(key_hi, tile_last[t]);
     if (p0 < nq) key_lo = min(key_lo, a.window > 0 ? max(0, n - nq + p0 - a.window + 1) : 0);
     const bf16_t* qp = a.q + ((int64_t)rr[t].token * a.heads + rr[t].head) * D + 8 * g;
@@ -227,7 +248,7 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
 #pragma unroll
     for (int ds = 0; ds < D / 16; ++ds) o[t][ds] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
-  attn_tiles<D, NT>(a, trow, hk, qf, qpos, tile_last, key_lo, key_hi, o, m, l);
+  attn_tiles<D, NT>(a, trow, hk, qf, qpos, tile_last, tile_first, key_lo, key_hi, o, m, l);
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     float lt = l[t];
@@ -312,7 +333,7 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
     const int range = pass == 0 ? (int)blockIdx.x : n_ranges - 1 - (int)blockIdx.x;
     if (pass == 1 && range <= (int)blockIdx.x) break;          // an odd count: the middle range was done in pass 0
     bf16x8_t qf[NT][D / 32];
-    int qpos[NT], tile_last[NT];
+    int qpos[NT], tile_last[NT], tile_first[NT];
     RowRef rr[NT];
     int key_hi = -1, key_lo = 0x7fffffff;                      // over the whole block (all waves walk the same stages)
     {
@@ -328,6 +349,7 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
       rr[t] = row_ref(tm, c, p0, hb, hk, group, qs, nq, n);
       qpos[t] = rr[t].valid ? rr[t].qpos : -1;
       tile_last[t] = p0 < nq ? n - nq + min(nq, p0 + tm.pos_per_tile) - 1 : -1;
+      tile_first[t] = n - nq + p0;
       const bf16_t* qp = a.q + ((int64_t)rr[t].token * a.heads + rr[t].head) * D + 8 * g;
 #pragma unroll
       for (int ks = 0; ks < D / 32; ++ks) {
@@ -402,31 +424,8 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
           }
           const int qp = qpos[t];
           const int first = a.window > 0 ? qp - a.window + 1 : 0;
-          float sv[8];
-          float mx = -INFINITY;
-#pragma unroll
-          for (int r = 0; r < 8; ++r) {
-            const int key = kb + 8 * g + r;
-            const float v = (r < 4 ? s0[r] : s1[r - 4]) * a.scale_log2;
-            sv[r] = (key <= qp && key >= first) ? v : -INFINITY;
-            mx = fmaxf(mx, sv[r]);
-          }
-          mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-          mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-          const float m_new = fmaxf(m[t], mx);
-          const float m_use = m_new == -INFINITY ? 0.f : m_new;
-          const float alpha = exp2f(m[t] - m_use);
-          m[t] = m_new;
-          float psum = 0.f;
-#pragma unroll
-          for (int r = 0; r < 8; ++r) {
-            const float p = exp2f(sv[r] - m_use);
-            psum += p;
-            pb[t][r] = (__bf16)p;
-          }
-          l[t] = l[t] * alpha + psum;
-#pragma unroll
-          for (int ds = 0; ds < D / 16; ++ds) o[t][ds] *= alpha;
+          const bool whole = kb + 31 <= tile_first[t] && (a.window <= 0 || kb >= tile_last[t] - a.window + 1);
+          pb[t] = softmax_block<D / 16>(s0, s1, whole, kb, g, qp, first, 0, 0x7fffffff, a.scale_log2, m[t], l[t], o[t]);
         }
 #pragma unroll
         for (int ds = 0; ds < D / 16; ++ds) {
@@ -510,12 +509,12 @@ __global__ void __launch_bounds__(64) attn_decode_kernel(AttnArgs a) {
       for (int i = 0; i < 8; ++i) qf[0][ks][i] = (__bf16)0.f;
     }
   }
-  int qpos[1] = {rr.valid ? qp_row : -1}, tile_last[1] = {qp_row};
+  int qpos[1] = {rr.valid ? qp_row : -1}, tile_last[1] = {qp_row}, tile_first[1] = {qp_row};
   f32x4_t o[1][D / 16];
   float m[1] = {-INFINITY}, l[1] = {0.f};
 #pragma unroll
   for (int ds = 0; ds < D / 16; ++ds) o[0][ds] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  attn_tiles<D, 1>(a, trow, hk, qf, qpos, tile_last, max(key_lo, first), key_hi, o, m, l);
+  attn_tiles<D, 1>(a, trow, hk, qf, qpos, tile_last, tile_first, max(key_lo, first), key_hi, o, m, l);
   float lt = l[0];
   lt += __shfl_xor(lt, 16, WAVE);
   lt += __shfl_xor(lt, 32, WAVE);
