@@ -167,7 +167,7 @@ class HipKernels:
         after the other (the sums over K may be split differently); None when this shape is not fused (the caller then composes the two)."""
         m, k = x.shape
         two_i = weight.shape[0]
-        if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows
+        if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= min(self.skinny_rows, 32)
                 and two_i % 32 == 0 and k % 128 == 0 and k >= 256 and weight.shape[1] == k and x.is_contiguous()):
             return None
         y = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)

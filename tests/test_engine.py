@@ -171,3 +171,31 @@ def test_graph_replays_equal_eager_steps(folders, dtype):
         if graphs:
             assert engine.runner.graph_replays > 20 and len(engine.runner.graphs) >= 3
     assert outs[True] == outs[False]
+
+
+@pytest.mark.gpu
+def test_command_line_generates_and_sizes_its_cache(folders):
+    """`python -m holon_amd generate` on the GPU, the cache sized from free memory (no --cache-tokens)."""
+    import subprocess
+    import sys
+    plain = PlainQwen3(folders["Bu"])
+    prompts = [H.random_ids(n, 384, 90 + n) for n in (4, 11)]
+    cmd = [sys.executable, "-m", "holon_amd", "generate", str(folders["Bu"]), "--dtype", "float32", "--max-tokens", "6",
+           "--temperature", "0", "--ignore-eos", "--max-seqs", "2", "--max-model-len", "64", "--max-step-tokens", "32",
+           "--stats"]
+    for p in prompts:
+        cmd += ["--prompt-ids", " ".join(map(str, p))]
+    run = subprocess.run(cmd, capture_output=True, text=True, timeout=110)
+    assert run.returncode == 0, run.stderr[-2000:]
+    got = [[int(t) for t in line.split()] for line in run.stdout.strip().splitlines()]
+    assert got == [plain.greedy(p, 6) for p in prompts]
+    assert "for the cache" in run.stderr and '"preemptions": 0' in run.stderr
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import pathlib
+    import subprocess
+    import sys
+    bench = pathlib.Path(__file__).resolve().parent.parent / "bench.py"
+    run = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True, timeout=60)
+    assert run.returncode == 2 and len(run.stdout.strip().splitlines()) == 1 and "one GPU" in run.stdout
