@@ -59,8 +59,11 @@ class SamplingParams:
     ignore_eos: bool = False
     stop_token_ids: tuple[int, ...] = ()
     seed: int | None = None
+    logprobs: int | None = None          # with every generated token: its log-probability and the k most likely (k <= 32)
 
     def check(self) -> None:
+        if self.logprobs is not None and not 0 <= self.logprobs <= 32:
+            raise ValueError("logprobs must be between 0 and 32")
         if self.presence_penalty or self.frequency_penalty or self.repetition_penalty != 1:
             raise NotImplementedError("sampling penalties are not supported")
         if self.temperature < 0 or not 0 < self.top_p <= 1 or self.top_k < 0 or not 0 <= self.min_p <= 1:

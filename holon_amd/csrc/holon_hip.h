@@ -57,6 +57,10 @@ int holon_sample(const float* logits, int32_t* out, int rows, int vocab, const f
                  const int32_t* top_k, const float* top_p, const float* min_p, const int64_t* seeds,
                  const int64_t* positions, void* stream);
 
+// log_softmax of the raw logits: token_lp[r] for tokens[r], and the k (<= 32) largest with their ids, [rows, k].
+int holon_logprobs(const float* logits, const int32_t* tokens, int rows, int vocab, int k, float* token_lp,
+                   int32_t* top_ids, float* top_lp, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

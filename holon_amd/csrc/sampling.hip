@@ -303,3 +303,54 @@ extern "C" int holon_sample(const float* logits, int32_t* out, int rows, int voc
   HOLON_LAUNCH_OK();
   return 0;
 }
+
+// Log-probabilities of the raw logits (before temperature): for each row the log-probability of `token[r]` and the
+// `k` largest log-probabilities with their ids (ties: lower id first). One block per row; k passes of argmax over
+// the row with the tokens already taken masked out.
+#define LOGPROB_MAX_K 32
+__global__ void logprobs_kernel(const float* __restrict__ logits, const int32_t* __restrict__ tokens, int vocab, int k,
+                                float* __restrict__ token_lp, int32_t* __restrict__ top_ids,
+                                float* __restrict__ top_lp) {
+  const int r = blockIdx.x;
+  const float* row = logits + (int64_t)r * vocab;
+  const ArgMax top = block_argmax(row, vocab, 1.0f);
+  float part = 0.f;
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) part += expf(row[i] - top.v);
+  const float lse = top.v + logf(block_sum(part));
+  if (threadIdx.x == 0) token_lp[r] = row[tokens[r]] - lse;
+  __shared__ int taken[LOGPROB_MAX_K];
+  __shared__ ArgMax part_best[SAMPLE_THREADS / WAVE];
+  for (int j = 0; j < k; ++j) {
+    ArgMax best{-INFINITY, 0x7fffffff};
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+      bool skip = false;
+      for (int t = 0; t < j; ++t) skip = skip || taken[t] == i;
+      if (!skip) best = better(best, ArgMax{row[i], i});
+    }
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) {
+      ArgMax other{__shfl_xor(best.v, o, WAVE), __shfl_xor(best.i, o, WAVE)};
+      best = better(best, other);
+    }
+    if (threadIdx.x % WAVE == 0) part_best[threadIdx.x / WAVE] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      ArgMax b = part_best[0];
+      for (int w = 1; w < (int)blockDim.x / WAVE; ++w) b = better(b, part_best[w]);
+      taken[j] = b.i;
+      top_ids[(int64_t)r * k + j] = b.i == 0x7fffffff ? 0 : b.i;
+      top_lp[(int64_t)r * k + j] = b.v - lse;
+    }
+    __syncthreads();
+  }
+}
+
+extern "C" int holon_logprobs(const float* logits, const int32_t* tokens, int rows, int vocab, int k, float* token_lp,
+                              int32_t* top_ids, float* top_lp, void* stream) {
+  HOLON_CHECK(rows >= 0 && vocab > 0 && k >= 0 && k <= LOGPROB_MAX_K && k <= vocab, "logprobs: k=%d must be at most %d",
+              k, LOGPROB_MAX_K);
+  if (rows == 0) return 0;
+  logprobs_kernel<<<rows, SAMPLE_THREADS, 0, (hipStream_t)stream>>>(logits, tokens, vocab, k, token_lp, top_ids, top_lp);
+  HOLON_LAUNCH_OK();
+  return 0;
+}

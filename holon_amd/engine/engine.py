@@ -24,7 +24,7 @@ from ..config.engine import EngineConfig, SamplingParams
 from ..sampling.sampler import Sampler, sequence_seed
 from .batch import StepRow
 from .loading import Loaded, attach_cache, build_from_spec, default_kernels, torch_dtype
-from .request import Seq, Status, TokenDelta
+from .request import Logprobs, Seq, Status, TokenDelta
 from .scheduler import Scheduler
 
 
@@ -172,13 +172,18 @@ class Engine:
         if sampled:
             slots = np.array([seq.slot for seq, _ in sampled], dtype=np.int64)
             positions = np.array([seq.num_computed + n for seq, n in sampled], dtype=np.int64)
-            tokens = self.sampler.sample(logits, slots, positions).tolist()
+            drawn = self.sampler.sample(logits, slots, positions)
+            k = max((seq.params.logprobs if seq.params.logprobs is not None else -1) for seq, _ in sampled)
+            lps = [t.tolist() for t in self.kernels.logprobs(logits, drawn, k)] if k >= 0 else None
+            tokens = drawn.tolist()
         deltas, at = [], 0
         for seq, n, m in rows:
             seq.num_computed += n
             if not m:
                 continue
             token = tokens[at]
+            want = seq.params.logprobs
+            lp = None if want is None else Logprobs([lps[0][at]], [lps[1][at][:want]], [lps[2][at][:want]])
             at += 1
             if seq.status is not Status.RUNNING:
                 self.sched.finished_prefill(seq)
@@ -187,7 +192,7 @@ class Engine:
             if reason:
                 self.sched.finish(seq, reason)
                 self._live.pop(seq.rid, None)
-            deltas.append(TokenDelta(seq.rid, [token], reason))
+            deltas.append(TokenDelta(seq.rid, [token], reason, lp))
         return deltas
 
     def _finish_reason(self, seq: Seq, token: int) -> str | None:

@@ -32,9 +32,20 @@ class Seq:
 
 
 @dataclasses.dataclass
+class Logprobs:
+    """Per emitted token: its log-probability, and the ids and log-probabilities of the k most likely tokens (of the
+    raw logits, before temperature: std/holon_std/sampling/sampler.py:147-152)."""
+
+    token: list[float]
+    top_ids: list[list[int]]
+    top: list[list[float]]
+
+
+@dataclasses.dataclass
 class TokenDelta:
     """New tokens of one request; `finish_reason` ("stop" | "length" | "abort") on its last delta."""
 
     rid: str
     token_ids: list[int]
     finish_reason: str | None = None
+    logprobs: Logprobs | None = None

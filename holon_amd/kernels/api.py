@@ -92,6 +92,11 @@ class Kernels(Protocol):
     def argmax(self, logits: torch.Tensor) -> torch.Tensor:
         """logits [R, V] float32 -> [R] int32, the first maximal index of each row."""
 
+    def logprobs(self, logits: torch.Tensor, tokens: torch.Tensor, k: int
+                 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """log_softmax of the raw logits [R, V]: (the log-probability of tokens[r] [R], the k largest ids [R, k] int32,
+        their log-probabilities [R, k]); k <= 32; ties go to the lower id."""
+
     def sample(self, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
                min_p: torch.Tensor, seeds: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
         """One token per row [R] int32. temperature/top_p/min_p float32 [R], top_k int32 [R], seeds int64 [R],

@@ -71,6 +71,7 @@ class HipKernels:
             "holon_gemm_skinny_glu_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
             "holon_argmax": [_P, _P, _I, _I, _P],
             "holon_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
+            "holon_logprobs": [_P, _P, _I, _I, _I, _P, _P, _P, _P],
         }
         for name, args in sig.items():
             fn = getattr(lib, name)
@@ -281,6 +282,19 @@ class HipKernels:
         self._call(self.lib.holon_argmax, logits.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1],
                    self._stream())
         return out
+
+    def logprobs(self, logits, tokens, k):
+        self._check(logits, "logprobs logits", torch.float32)
+        self._check(tokens, "logprobs tokens", torch.int32)
+        r = logits.shape[0]
+        if tokens.shape != (r,) or not 0 <= k <= 32:
+            raise KernelError(f"logprobs: {tuple(tokens.shape)} tokens for {r} rows, k={k} (at most 32)")
+        token_lp = torch.empty((r,), dtype=torch.float32, device=logits.device)
+        top_ids = torch.empty((r, k), dtype=torch.int32, device=logits.device)
+        top_lp = torch.empty((r, k), dtype=torch.float32, device=logits.device)
+        self._call(self.lib.holon_logprobs, logits.data_ptr(), tokens.data_ptr(), r, logits.shape[1], k,
+                   token_lp.data_ptr(), top_ids.data_ptr(), top_lp.data_ptr(), self._stream())
+        return token_lp, top_ids, top_lp
 
     def sample(self, logits, temperature, top_k, top_p, min_p, seeds, positions):
         self._check(logits, "sample logits", torch.float32)

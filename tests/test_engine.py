@@ -199,3 +199,28 @@ def test_bench_refuses_more_than_one_gpu():
     bench = pathlib.Path(__file__).resolve().parent.parent / "bench.py"
     run = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True, timeout=60)
     assert run.returncode == 2 and len(run.stdout.strip().splitlines()) == 1 and "one GPU" in run.stdout
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_logprobs_of_generated_tokens(folders, device):
+    plain = PlainQwen3(folders["Bu"])
+    engine = _engine(folders["Bu"], device, page_size=8, max_seqs=2, max_model_len=64)
+    prompt = H.random_ids(9, 384, 3)
+    engine.add(prompt, SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True, logprobs=3), rid="a")
+    engine.add(prompt[:5], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True), rid="b")
+    ids, got = list(prompt), []
+    while engine.has_work():
+        for d in engine.step():
+            if d.rid == "b":
+                assert d.logprobs is None
+                continue
+            want = plain.logits(ids)[-1].log_softmax(-1)
+            top = want.topk(3)
+            assert d.logprobs.top_ids == [top.indices.tolist()] and d.token_ids == [int(top.indices[0])]
+            torch.testing.assert_close(torch.tensor(d.logprobs.top[0]), top.values, rtol=1e-4, atol=1e-4)
+            torch.testing.assert_close(torch.tensor(d.logprobs.token), top.values[:1], rtol=1e-4, atol=1e-4)
+            ids += d.token_ids
+            got += d.token_ids
+    assert len(got) == 4
+    with pytest.raises(ValueError):
+        engine.add(prompt, SamplingParams(logprobs=33))

@@ -247,6 +247,19 @@ def test_fused_gate_up_is_the_two_kernels(hip, monkeypatch):
     assert hip.linear_silu_mul(_randn(4, 256, dtype=torch.float32), _randn(64, 256, dtype=torch.float32)) is None
 
 
+def test_logprobs_kernel(hip):
+    g = torch.Generator().manual_seed(40)
+    for rows, vocab, k in ((3, 151_936, 20), (5, 97, 5), (2, 40, 0), (1, 33, 32)):
+        logits = (torch.randn(rows, vocab, generator=g) * 3).cuda()
+        logits[0, 7] = logits[0, 3] = logits[0].max() + 1                 # a tie at the top: the lower id first
+        tokens = torch.randint(0, vocab, (rows,), generator=g).to(torch.int32).cuda()
+        lp, ids, top = hip.logprobs(logits, tokens, k)
+        want_lp, want_ids, want_top = PLAIN.logprobs(logits.double(), tokens, k)
+        assert ids.tolist() == want_ids.tolist()
+        torch.testing.assert_close(lp.double(), want_lp.double(), rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(top.double(), want_top.double(), rtol=1e-5, atol=1e-5)
+
+
 def test_argmax_and_sampling(hip):
     from tests.plain import sampling as S
     g = torch.Generator().manual_seed(20)
