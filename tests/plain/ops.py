@@ -118,7 +118,7 @@ class TorchKernels:
 
     def logprobs(self, logits, tokens, k):
         lp = (logits if logits.dtype == torch.float64 else logits.float()).log_softmax(-1)
-        order = lp.argsort(-1, descending=True, stable=True)[:, :k]
+        order = lp.argsort(dim=-1, descending=True, stable=True)[:, :k]
         return lp.gather(-1, tokens.long()[:, None])[:, 0], order.to(torch.int32), lp.gather(-1, order)
 
     def sample(self, logits, temperature, top_k, top_p, min_p, seeds, positions):
