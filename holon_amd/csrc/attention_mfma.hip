@@ -601,11 +601,12 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
   const int nt = head_dim == 256 ? 1 : 2;
   const int tiles = (max_query + tm.pos_per_tile - 1) / tm.pos_per_tile;
   if (head_dim != 256 && tiles >= 16 && max_len <= 4096 * page_size) {
-    // long portions: keys and values staged through LDS, shared by four waves (rows of up to 4096 pages)
-    const int ranges = (tiles + 4 * nt - 1) / (4 * nt);
+    // long portions: keys and values staged through LDS, shared by four waves (rows of up to 4096 pages). One tile a
+    // wave: measured faster than two (more blocks in flight matter more than sharing each stage among more rows).
+    const int ranges = (tiles + 3) / 4;
     dim3 lgrid((ranges + 1) / 2, kv_heads * tm.head_blocks, n_rows);
-    if (head_dim == 64) attn_prefill_lds_kernel<64, 2><<<lgrid, 256, 0, (hipStream_t)stream>>>(a);
-    else attn_prefill_lds_kernel<128, 2><<<lgrid, 256, 0, (hipStream_t)stream>>>(a);
+    if (head_dim == 64) attn_prefill_lds_kernel<64, 1><<<lgrid, 256, 0, (hipStream_t)stream>>>(a);
+    else attn_prefill_lds_kernel<128, 1><<<lgrid, 256, 0, (hipStream_t)stream>>>(a);
     HOLON_LAUNCH_OK();
     return 0;
   }
