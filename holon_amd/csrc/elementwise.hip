@@ -356,6 +356,58 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
   for (int j = 0; j < EPL; ++j) dst[j] = Elem<T>::store(v[j]);
 }
 
+// Values of 16 consecutive tokens of one kv head into the cache. Inside a page values are stored transposed
+// ([D, P]), so a token alone writes D scattered elements; 16 tokens that fill consecutive places of one page are
+// transposed through LDS and written as 32 contiguous bytes per dim.
+template <typename T>
+__global__ void __launch_bounds__(256) v_write_group_kernel(const T* __restrict__ qkv, int64_t qkv_stride, int v_col0,
+                                                            int tokens, int kv_heads, int head_dim,
+                                                            T* __restrict__ pages,
+                                                            const int32_t* __restrict__ write_page,
+                                                            const int32_t* __restrict__ write_off, int page_size) {
+  __shared__ T tile[16][MAX_HEAD_DIM + 8];
+  __shared__ int together;
+  const int t0 = blockIdx.x * 16, hk = blockIdx.y, tid = threadIdx.x;
+  const int count = min(16, tokens - t0);
+  if (tid == 0) {
+    int ok = count == 16 && write_off[t0] % 8 == 0 && write_off[t0] + 16 <= page_size;
+    for (int j = 1; ok && j < 16; ++j)
+      ok = write_page[t0 + j] == write_page[t0] && write_off[t0 + j] == write_off[t0] + j;
+    together = ok;
+  }
+  const int per_row = head_dim / 8;   // head_dim % 8 == 0 (checked by the host)
+  for (int q = tid; q < count * per_row; q += 256) {
+    const int tk = q / per_row, c8 = (q % per_row) * 8;
+    const T* src = qkv + (int64_t)(t0 + tk) * qkv_stride + v_col0 + (int64_t)hk * head_dim + c8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) tile[tk][c8 + j] = src[j];
+  }
+  __syncthreads();
+  const int64_t plane = (int64_t)page_size * head_dim;
+  if (together) {
+    T* base = pages + (((int64_t)write_page[t0] * 2 + 1) * kv_heads + hk) * plane + write_off[t0];
+    for (int r = tid; r < head_dim * 2; r += 256) {
+      const int d = r / 2, half = r % 2;
+      T out8[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) out8[j] = tile[half * 8 + j][d];
+      T* dst = base + (int64_t)d * page_size + half * 8;
+      if (sizeof(T) == 2) {
+        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(out8);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst[j] = out8[j];
+      }
+    }
+  } else {
+    for (int q = tid; q < count * head_dim; q += 256) {
+      const int tk = q % count, d = q / count;
+      pages[(((int64_t)write_page[t0 + tk] * 2 + 1) * kv_heads + hk) * plane + (int64_t)d * page_size +
+            write_off[t0 + tk]] = tile[tk][d];
+    }
+  }
+}
+
 extern "C" int holon_qk_norm_rope_write(const void* qkv, int64_t qkv_stride, void* q_out, int tokens, int heads,
                                         int kv_heads, int head_dim, const void* q_weight, const void* k_weight,
                                         float eps, const float* table, int rotary_dim, int max_positions,
@@ -376,10 +428,15 @@ extern "C" int holon_qk_norm_rope_write(const void* qkv, int64_t qkv_stride, voi
   hipStream_t s = (hipStream_t)stream;
   if ((head_dim == 64 || head_dim == 128 || head_dim == 256) && (table == nullptr || rotary_dim == head_dim) &&
       qkv != q_out) {
+    // many tokens: values go through their own kernel, 16 tokens at a time (contiguous writes); the heads kernel then
+    // covers queries and keys only
+    const bool split_v = pages != nullptr && tokens >= 64;
+    const int fast_heads = split_v ? heads + kv_heads : total_heads;
+    grid = dim3(tokens, (fast_heads + 3) / 4);
 #define QK_FAST(T, EPL)                                                                                            \
   qk_norm_rope_write_fast_kernel<T, EPL><<<grid, 4 * WAVE, 0, s>>>(                                                 \
       (const T*)qkv, qkv_stride, (T*)q_out, heads, kv_heads, (const T*)q_weight, (const T*)k_weight, eps, table,    \
-      positions, (T*)pages, write_page, write_off, page_size, total_heads)
+      positions, (T*)pages, write_page, write_off, page_size, fast_heads)
     if (dtype == HOLON_F32) {
       if (head_dim == 64) QK_FAST(float, 1); else if (head_dim == 128) QK_FAST(float, 2); else QK_FAST(float, 4);
     } else {
@@ -387,6 +444,17 @@ extern "C" int holon_qk_norm_rope_write(const void* qkv, int64_t qkv_stride, voi
     }
 #undef QK_FAST
     HOLON_LAUNCH_OK();
+    if (split_v) {
+      dim3 vgrid((tokens + 15) / 16, kv_heads);
+      const int v_col0 = (heads + kv_heads) * head_dim;
+      if (dtype == HOLON_F32)
+        v_write_group_kernel<float><<<vgrid, 256, 0, s>>>((const float*)qkv, qkv_stride, v_col0, tokens, kv_heads,
+                                                          head_dim, (float*)pages, write_page, write_off, page_size);
+      else
+        v_write_group_kernel<bf16_t><<<vgrid, 256, 0, s>>>((const bf16_t*)qkv, qkv_stride, v_col0, tokens, kv_heads,
+                                                           head_dim, (bf16_t*)pages, write_page, write_off, page_size);
+      HOLON_LAUNCH_OK();
+    }
     return 0;
   }
 #define QK_LAUNCH(T)                                                                                              \

@@ -167,25 +167,29 @@ def test_attention_finds_a_far_key(hip, dtype):
 def test_fused_norm_rope_write_is_the_three_ops(hip, dtype, geometry):
     from holon_amd.parts.positions import rope_table
     heads, kv_heads, head_dim, page = geometry
-    t, units = 45, 40
-    qkv = _randn(t, (heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=8)
-    qw, kw = _randn(head_dim, dtype=dtype, seed=9), _randn(head_dim, dtype=dtype, seed=10)
     table = rope_table(4096, head_dim, 1e6).cuda()
     rng = np.random.default_rng(0)
-    where = rng.permutation(units * page)[:t]
-    pos = torch.as_tensor(rng.integers(0, 4096, t).astype(np.int32)).cuda()
-    wp, wo = (torch.as_tensor((where // page).astype(np.int32)).cuda(), torch.as_tensor((where % page).astype(np.int32)).cuda())
-    for use_norm, use_rope in ((True, True), (False, True), (True, False), (False, False)):
-        pages_h = torch.zeros(units, 2, kv_heads, page * head_dim, dtype=dtype).cuda()
-        pages_p = pages_h.clone()
-        args = (heads, kv_heads, head_dim, qw if use_norm else None, kw if use_norm else None, 1e-6,
-                table if use_rope else None, pos)
-        got = hip.qk_norm_rope_write(qkv, *args, pages_h, wp, wo, page)
-        want = PLAIN.qk_norm_rope_write(qkv, *args, pages_p, wp, wo, page)
-        assert H.op_budget_usage(got, want, dtype, head_dim) <= 1
-        assert H.op_budget_usage(pages_h, pages_p, dtype, head_dim) <= 1
-        assert torch.equal(pages_h == 0, pages_p == 0), "a cache entry outside the written ones changed"
-        assert torch.equal(pages_h[:, 1], pages_p[:, 1]), "values are copied bit for bit"
+    qw, kw = _randn(head_dim, dtype=dtype, seed=9), _randn(head_dim, dtype=dtype, seed=10)
+    # few tokens at scattered places; many tokens at consecutive places (whole pages and ragged ends); many scattered
+    layouts = [(45, rng.permutation(40 * page)[:45]), (200, np.arange(200) + 3 * page), (130, np.arange(130) + 5),
+               (100, rng.permutation(40 * page)[:100])]
+    for t, where in layouts:
+        units = int(where.max()) // page + 2
+        qkv = _randn(t, (heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=8)
+        pos = torch.as_tensor(rng.integers(0, 4096, t).astype(np.int32)).cuda()
+        wp, wo = (torch.as_tensor((where // page).astype(np.int32)).cuda(), torch.as_tensor((where % page).astype(np.int32)).cuda())
+        for use_norm, use_rope in ((True, True), (False, True), (True, False), (False, False)):
+            pages_h = torch.zeros(units, 2, kv_heads, page * head_dim, dtype=dtype).cuda()
+            pages_p = pages_h.clone()
+            args = (heads, kv_heads, head_dim, qw if use_norm else None, kw if use_norm else None, 1e-6,
+                    table if use_rope else None, pos)
+            got = hip.qk_norm_rope_write(qkv, *args, pages_h, wp, wo, page)
+            want = PLAIN.qk_norm_rope_write(qkv, *args, pages_p, wp, wo, page)
+            assert H.op_budget_usage(got, want, dtype, head_dim) <= 1
+            assert H.op_budget_usage(pages_h, pages_p, dtype, head_dim) <= 1
+            assert torch.equal(pages_h == 0, pages_p == 0), "a cache entry outside the written ones changed"
+            assert torch.equal(pages_h[:, 1], pages_p[:, 1]), "values are copied bit for bit"
+    t = 45
     # queries only (a run that reads another run's cache)
     got = hip.qk_norm_rope_write(qkv, heads, kv_heads, head_dim, qw, kw, 1e-6, table, pos, None, None, None, page)
     want = PLAIN.qk_norm_rope_write(qkv, heads, kv_heads, head_dim, qw, kw, 1e-6, table, pos, None, None, None, page)
