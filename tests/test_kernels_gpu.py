@@ -189,7 +189,11 @@ def test_fused_norm_rope_write_is_the_three_ops(hip, dtype, geometry):
             assert H.op_budget_usage(pages_h, pages_p, dtype, head_dim) <= 1
             assert torch.equal(pages_h == 0, pages_p == 0), "a cache entry outside the written ones changed"
             assert torch.equal(pages_h[:, 1], pages_p[:, 1]), "values are copied bit for bit"
-    t = 45
+    t, where = layouts[0]
+    units = 42
+    qkv = _randn(t, (heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=8)
+    pos = torch.as_tensor(rng.integers(0, 4096, t).astype(np.int32)).cuda()
+    wp, wo = (torch.as_tensor((where // page).astype(np.int32)).cuda(), torch.as_tensor((where % page).astype(np.int32)).cuda())
     # queries only (a run that reads another run's cache)
     got = hip.qk_norm_rope_write(qkv, heads, kv_heads, head_dim, qw, kw, 1e-6, table, pos, None, None, None, page)
     want = PLAIN.qk_norm_rope_write(qkv, heads, kv_heads, head_dim, qw, kw, 1e-6, table, pos, None, None, None, page)
