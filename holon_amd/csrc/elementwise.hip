@@ -304,56 +304,76 @@ __global__ void qk_norm_rope_write_kernel(const T* qkv, int64_t qkv_stride, T* q
   }
 }
 
-// The same for head_dim 64, 128 or 256 with the whole head rotated (or not at all): each lane holds EPL = head_dim / 64
-// consecutive values; the rotation partner of a value sits 32 lanes away, so a shuffle replaces the LDS staging.
-template <typename T, int EPL>
+// The same for head_dim 64, 128 or 256 with the whole head rotated (or not at all): each lane holds 8 consecutive
+// values (one 16-byte load), LPH = head_dim / 8 lanes make a head, a wave holds 64 / LPH heads. The rotation partner
+// of a value sits LPH / 2 lanes away; norm sums run over the LPH lanes of a head. No LDS.
+template <typename T, int LPH>
 __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
     const T* qkv, int64_t qkv_stride, T* q_out, int heads, int kv_heads, const T* __restrict__ q_weight,
     const T* __restrict__ k_weight, float eps, const float* __restrict__ table, const int32_t* __restrict__ positions,
     T* __restrict__ pages, const int32_t* __restrict__ write_page, const int32_t* __restrict__ write_off,
     int page_size, int total_heads) {
-  constexpr int D = EPL * WAVE;
-  const int w = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  constexpr int D = LPH * 8;
+  constexpr int HPB = 256 / LPH;                     // heads a block covers
   const int t = blockIdx.x;
-  const int h = blockIdx.y * 4 + w;
-  if (h >= total_heads) return;   // no barrier below
-  const T* src = qkv + (int64_t)t * qkv_stride + (int64_t)h * D + lane * EPL;
-  float v[EPL];
+  const int h = blockIdx.y * HPB + threadIdx.x / LPH;
+  const int li = threadIdx.x % LPH;                  // lane within the head
+  const bool active = h < total_heads;               // (shuffles below are executed by every lane)
+  const int hh = active ? h : 0;
+  const T* src = qkv + (int64_t)t * qkv_stride + (int64_t)hh * D + li * 8;
+  float v[8];
+  if (sizeof(T) == 2) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(src);
+    const T* e = reinterpret_cast<const T*>(&raw);
 #pragma unroll
-  for (int j = 0; j < EPL; ++j) v[j] = Elem<T>::load(src[j]);
-  if (h >= heads + kv_heads) {   // a value head: transposed inside the page
-    const int hk = h - heads - kv_heads;
+    for (int j = 0; j < 8; ++j) v[j] = Elem<T>::load(e[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = Elem<T>::load(src[j]);
+  }
+  if (active && hh >= heads + kv_heads) {   // a value head: transposed inside the page
+    const int hk = hh - heads - kv_heads;
     T* dst = pages + (((int64_t)write_page[t] * 2 + 1) * kv_heads + hk) * (int64_t)page_size * D + write_off[t];
 #pragma unroll
-    for (int j = 0; j < EPL; ++j) dst[(int64_t)(lane * EPL + j) * page_size] = src[j];
-    return;
+    for (int j = 0; j < 8; ++j) dst[(int64_t)(li * 8 + j) * page_size] = Elem<T>::store(v[j]);
   }
-  const bool is_q = h < heads;
+  const bool is_v = hh >= heads + kv_heads;
+  const bool is_q = hh < heads;
   const T* weight = is_q ? q_weight : k_weight;
   if (weight != nullptr) {
     float ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < EPL; ++j) ss += v[j] * v[j];
-    ss = wave_sum(ss);
+    for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
+#pragma unroll
+    for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
     const float inv = 1.0f / sqrtf(ss / (float)D + eps);
 #pragma unroll
-    for (int j = 0; j < EPL; ++j) v[j] = Elem<T>::round((v[j] * inv) * Elem<T>::load(weight[lane * EPL + j]));
+    for (int j = 0; j < 8; ++j) v[j] = Elem<T>::round((v[j] * inv) * Elem<T>::load(weight[li * 8 + j]));
   }
   if (table != nullptr) {
     const float* cs = table + (int64_t)positions[t] * D;
-    const int i0 = (lane % 32) * EPL;   // index of the pair within the half
+    const int i0 = (li % (LPH / 2)) * 8;   // index of the pair within the half
 #pragma unroll
-    for (int j = 0; j < EPL; ++j) {
-      const float other = __shfl_xor(v[j], 32, WAVE);
+    for (int j = 0; j < 8; ++j) {
+      const float other = __shfl_xor(v[j], LPH / 2, WAVE);
       const float co = cs[i0 + j], si = cs[D / 2 + i0 + j];
-      v[j] = lane < 32 ? v[j] * co - other * si : v[j] * co + other * si;
+      v[j] = li < LPH / 2 ? v[j] * co - other * si : v[j] * co + other * si;
     }
   }
-  T* dst = is_q ? q_out + ((int64_t)t * heads + h) * D + lane * EPL
-                : pages + (((int64_t)write_page[t] * 2 + 0) * kv_heads + (h - heads)) * (int64_t)page_size * D +
-                      (int64_t)write_off[t] * D + lane * EPL;
+  if (!active || is_v) return;
+  T* dst = is_q ? q_out + ((int64_t)t * heads + hh) * D + li * 8
+                : pages + (((int64_t)write_page[t] * 2 + 0) * kv_heads + (hh - heads)) * (int64_t)page_size * D +
+                      (int64_t)write_off[t] * D + li * 8;
+  if (sizeof(T) == 2) {
+    uint4 out;
+    T* oe = reinterpret_cast<T*>(&out);
 #pragma unroll
-  for (int j = 0; j < EPL; ++j) dst[j] = Elem<T>::store(v[j]);
+    for (int j = 0; j < 8; ++j) oe[j] = Elem<T>::store(v[j]);
+    *reinterpret_cast<uint4*>(dst) = out;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dst[j] = Elem<T>::store(v[j]);
+  }
 }
 
 // Values of 16 consecutive tokens of one kv head into the cache. Inside a page values are stored transposed
@@ -430,17 +450,18 @@ extern "C" int holon_qk_norm_rope_write(const void* qkv, int64_t qkv_stride, voi
       qkv != q_out) {
     // many tokens: values go through their own kernel, 16 tokens at a time (contiguous writes); the heads kernel then
     // covers queries and keys only
-    const bool split_v = pages != nullptr && tokens >= 64;
+    const bool split_v = pages != nullptr && tokens >= 256;
     const int fast_heads = split_v ? heads + kv_heads : total_heads;
-    grid = dim3(tokens, (fast_heads + 3) / 4);
-#define QK_FAST(T, EPL)                                                                                            \
-  qk_norm_rope_write_fast_kernel<T, EPL><<<grid, 4 * WAVE, 0, s>>>(                                                 \
+    const int lph = head_dim / 8;
+    grid = dim3(tokens, (fast_heads + 256 / lph - 1) / (256 / lph));
+#define QK_FAST(T, LPH)                                                                                            \
+  qk_norm_rope_write_fast_kernel<T, LPH><<<grid, 256, 0, s>>>(                                                      \
       (const T*)qkv, qkv_stride, (T*)q_out, heads, kv_heads, (const T*)q_weight, (const T*)k_weight, eps, table,    \
       positions, (T*)pages, write_page, write_off, page_size, fast_heads)
     if (dtype == HOLON_F32) {
-      if (head_dim == 64) QK_FAST(float, 1); else if (head_dim == 128) QK_FAST(float, 2); else QK_FAST(float, 4);
+      if (head_dim == 64) QK_FAST(float, 8); else if (head_dim == 128) QK_FAST(float, 16); else QK_FAST(float, 32);
     } else {
-      if (head_dim == 64) QK_FAST(bf16_t, 1); else if (head_dim == 128) QK_FAST(bf16_t, 2); else QK_FAST(bf16_t, 4);
+      if (head_dim == 64) QK_FAST(bf16_t, 8); else if (head_dim == 128) QK_FAST(bf16_t, 16); else QK_FAST(bf16_t, 32);
     }
 #undef QK_FAST
     HOLON_LAUNCH_OK();
