@@ -65,9 +65,11 @@ template <int DS>
 __device__ __forceinline__ bf16x8_t softmax_block(const f32x4_t& s0, const f32x4_t& s1, bool whole, int kb, int g,
                                                   int qp, int first, int key_lo, int key_hi, float scale_log2,
                                                   float& m, float& l, f32x4_t (&o)[DS]) {
+  // m and the comparisons are in units of the raw scores' scale times log2(e); a score enters as one fused
+  // multiply-add, exp2(s * c - m)
   float sv[8];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) sv[r] = (r < 4 ? s0[r] : s1[r - 4]) * scale_log2;
+  for (int r = 0; r < 8; ++r) sv[r] = r < 4 ? s0[r] : s1[r - 4];
   if (!whole) {
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
@@ -78,13 +80,13 @@ __device__ __forceinline__ bf16x8_t softmax_block(const f32x4_t& s0, const f32x4
   float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
   mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
   mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-  const float m_new = fmaxf(m, mx);
+  const float m_new = fmaxf(m, mx * scale_log2);          // (scale > 0: the largest raw score is the largest scaled one)
   const float m_use = m_new == -INFINITY ? 0.f : m_new;   // nothing visible yet: keep everything at zero
   bf16x8_t pb;
   float psum = 0.f;
 #pragma unroll
   for (int r = 0; r < 8; ++r) {
-    const float p = __builtin_amdgcn_exp2f(sv[r] - m_use);   // arguments <= 0; results below 2^-126 flush to zero
+    const float p = __builtin_amdgcn_exp2f(fmaf(sv[r], scale_log2, -m_use));   // <= 0; below 2^-126 flushes to zero
     psum += p;
     pb[r] = (__bf16)p;
   }
@@ -381,8 +383,9 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
       // a stage is two groups of 16 keys, each inside one page: two table entries, the same for every thread (scalar
       // loads, which do not queue behind the vector loads in flight)
       const int i0 = min(kb / P, max_page), i1 = min((kb + 16) / P, max_page);   // (kb <= key_hi < n: inside the row)
-      const int64_t pg0 = (int64_t)pg_lds[i0] * page_stride;   // (the host sends longer rows to the other kernel)
-      const int64_t pg1 = (int64_t)pg_lds[i1] * page_stride;
+      // (uniform over the block: kept in scalar registers, so the 64-bit page offsets are scalar arithmetic)
+      const int64_t pg0 = (int64_t)__builtin_amdgcn_readfirstlane(pg_lds[i0]) * page_stride;
+      const int64_t pg1 = (int64_t)__builtin_amdgcn_readfirstlane(pg_lds[i1]) * page_stride;
       const int off0 = kb % P, off1 = (kb + 16) % P;
 #pragma unroll
       for (int i = 0; i < ROUNDS; ++i) {

@@ -12,6 +12,7 @@ sampler draws a token for every row that ended its prompt or decoded, the commit
 """
 from __future__ import annotations
 
+import dataclasses
 import itertools
 import secrets
 import sys
@@ -21,9 +22,13 @@ import torch
 
 from ..cache.pool import OutOfPages
 from ..config.engine import EngineConfig, SamplingParams
+from ..config.model import read_config_json
+from ..registry import resolve
 from ..sampling.sampler import Sampler, sequence_seed
+from ..weights.loader import load_weights
+from ..weights.random_init import fill_random
 from .batch import StepRow
-from .loading import Loaded, attach_cache, build_from_spec, default_kernels, torch_dtype
+from .loading import attach_cache, build_from_spec, default_kernels, torch_dtype
 from .request import Logprobs, Seq, Status, TokenDelta
 from .scheduler import Scheduler
 
@@ -40,10 +45,6 @@ def activation_bytes(spec, max_step_tokens: int, max_seqs: int, itemsize: int) -
 
 class Engine:
     def __init__(self, cfg: EngineConfig, kernels=None, *, random_config: dict | None = None, seed: int = 0) -> None:
-        from ..config.model import read_config_json
-        from ..registry import resolve
-        from ..weights.loader import load_weights
-        from ..weights.random_init import fill_random
         self.cfg = cfg
         device, dtype = torch.device(cfg.device), torch_dtype(cfg.dtype)
         self.device, self.dtype = device, dtype
@@ -117,7 +118,6 @@ class Engine:
         if rid in self._live:
             raise ValueError(f"request id {rid!r} is already in flight")
         seed = p.seed if p.seed is not None else secrets.randbits(63)
-        import dataclasses
         seq = Seq(rid=rid, tokens=list(token_ids), params=dataclasses.replace(p, seed=sequence_seed(seed, 0)))
         self._live[rid] = seq
         self.sched.add(seq)

@@ -19,9 +19,11 @@ import time
 CSRC = pathlib.Path(__file__).resolve().parent.parent / "csrc"
 IN_TREE = pathlib.Path(__file__).resolve().parent / "libholon_hip.so"
 ARCH = "gfx950"
-# packed float32 VALU ops are kept out of the generated code on purpose (see the flag's use below)
+# Packed float32 VALU ops are kept out of the generated code on purpose. Matrix-core accumulators are kept in
+# ordinary vector registers: with the accumulator file the compiler copies them back and forth around every
+# rescale of the attention kernels (a third of their vector instructions).
 HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
-             "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+             "-packed-fp32-ops", "-mllvm", "-amdgpu-mfma-vgpr-form=1", "-Wno-unused-command-line-argument"]
 
 
 def sources() -> list[pathlib.Path]:
