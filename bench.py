@@ -3,8 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--no-points]
 
-One JSON line: decoded tokens a second at the given batch (default 8) with every request near the context length
-BASELINE.json's configs[2] gives (4,096), plus the prefill of one 2,048-token prompt, the decode step's memory
+One JSON line: decoded tokens a second at the given batch (default 8) with every request near a context of 4,096 tokens
+(a 2,048-token prompt and 2,048 generated tokens), plus the prefill of one 2,048-token prompt, the decode step's memory
 roofline, and decode at batch 1 and 64. A step is one decode step of the engine: scheduling, the model, sampling and
 the commit. The engine is one process on one GPU; for --gpus > 1 a line says so and the exit code is 2.
 """

@@ -1,6 +1,7 @@
 """Generation through the entry point (`Engine`), against the plain model: greedy and seeded temperature sampling,
 chunked prompts, mixed steps, preemption, rejections. CPU cases run the plain kernel twins; `gpu` cases the HIP kernels.
-Workloads: the two tiny configurations' own (BASELINE.json configs 0 and 1) and the reference's engine tests
+Workloads: the two tiny configurations' own (3 prompts of 5/17/33 tokens with 16 greedy tokens; 4 prompts of
+1/8/31/64 tokens with portions of 16 beside decode tokens and seeded sampling) and the reference's engine tests
 (plugins/tests/test_engine.py:25-106)."""
 from __future__ import annotations
 
