@@ -78,6 +78,8 @@ def build(verbose: bool = True, force: bool = True) -> pathlib.Path:
         objdir = fallback_dir()
         objdir.mkdir(parents=True, exist_ok=True)
         target = objdir / "libholon_hip.so"
+    objdir = objdir / f"obj-{os.getpid()}"       # its own folder: two processes may build at the same time
+    objdir.mkdir(parents=True, exist_ok=True)
     cc = hipcc()
     srcs = sources()
     say(f"compiling {len(srcs)} HIP sources for {ARCH} into {target} (a minute or two the first time)")
@@ -96,12 +98,13 @@ def build(verbose: bool = True, force: bool = True) -> pathlib.Path:
 
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
         objs = list(pool.map(compile_one, srcs))
-    tmp = target.with_suffix(f".tmp{os.getpid()}")
+    tmp = target.parent / f"{target.name}.tmp{os.getpid()}"
     proc = subprocess.run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *map(str, objs), "-o", str(tmp)],
                           capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"linking libholon_hip.so failed:\n{proc.stderr[-4000:]}")
     os.replace(tmp, target)
+    shutil.rmtree(objdir, ignore_errors=True)
     (target.parent / (target.name + ".hash")).write_text(source_hash())
     say(f"built {target} in {time.time() - t0:.0f} s")
     return target
