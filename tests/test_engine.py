@@ -225,3 +225,30 @@ def test_logprobs_of_generated_tokens(folders, device):
     assert len(got) == 4
     with pytest.raises(ValueError):
         engine.add(prompt, SamplingParams(logprobs=33))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_end_of_sequence_tokens_stop_a_request(folders, tmp_path, device):
+    """eos_token_id of config.json and generation_config.json (an int or a list) ends a request with "stop" and the
+    token is delivered; ignore_eos generates on."""
+    import json
+    import shutil
+    plain = PlainQwen3(folders["Bu"])
+    prompt = H.random_ids(7, 384, 21)
+    free = plain.greedy(prompt, 8)
+    folder = tmp_path / "with-eos"
+    shutil.copytree(folders["Bu"], folder)
+    cfg = json.loads((folder / "config.json").read_text())
+    cfg["eos_token_id"] = free[2]
+    (folder / "config.json").write_text(json.dumps(cfg))
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": [free[2], free[5]]}))
+    engine = _engine(folder, device, page_size=8, max_seqs=2, max_model_len=64)
+    assert engine.eos == {free[2], free[5]}
+    rid = engine.add(prompt, SamplingParams(temperature=0.0, max_tokens=8))
+    deltas = []
+    while engine.has_work():
+        deltas += engine.step()
+    assert [t for d in deltas for t in d.token_ids] == free[: free.index(free[2]) + 1]
+    assert deltas[-1].finish_reason == "stop" and deltas[-1].rid == rid
+    out = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
+    assert out == [free]
