@@ -105,7 +105,8 @@ def _paged_case(rows, heads, kv_heads, head_dim, page, dtype, seed=0, max_seqs=8
     return q, pages, table.cuda(), attn
 
 
-GEOMETRIES = [(32, 8, 128), (16, 4, 256), (16, 8, 64), (6, 3, 32), (4, 1, 16), (5, 5, 48), (12, 2, 80)]
+GEOMETRIES = [(32, 8, 128), (16, 4, 256), (16, 8, 64), (6, 3, 32), (4, 1, 16), (5, 5, 48), (12, 2, 80),
+              (10, 2, 64), (40, 2, 128), (7, 7, 64), (6, 1, 128), (48, 2, 64)]   # groups of 5, 20, 1, 6 and 24 heads
 ROWSETS = [[(0, 1), (0, 17), (5, 16), (31, 33), (0, 64), (100, 7), (16, 16)],
            [(0, 1), (15, 1), (16, 1), (99, 1), (999, 1), (4096, 1)],
            [(63, 1), (200, 2), (17, 1), (0, 130), (1, 1)]]
