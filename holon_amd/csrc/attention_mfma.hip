@@ -492,8 +492,12 @@ __global__ void __launch_bounds__(64) attn_decode_kernel(AttnArgs a) {
   // the keys this row can see, cut into `splits` ranges of keys_per_split
   const int qp_row = n - 1;
   const int first = a.window > 0 ? max(0, qp_row - a.window + 1) : 0;
-  const int key_lo = (first / 32) * 32 + split * a.keys_per_split;
-  const int key_hi = min(qp_row, key_lo + a.keys_per_split - 1);
+  // every split gets an equal share of this row's own keys (a multiple of 32), whatever length the launch was
+  // shaped for: a row shorter than the longest one still keeps all its waves busy
+  const int base = (first / 32) * 32;
+  const int share = max(32, ((qp_row - base + a.splits) / a.splits + 31) / 32 * 32);
+  const int key_lo = base + split * share;
+  const int key_hi = min(qp_row, key_lo + share - 1);
   float* po = a.part_o + (((int64_t)ri * a.heads + rr.head) * a.splits + split) * D + 4 * g;
   float* pml = a.part_ml + (((int64_t)ri * a.heads + rr.head) * a.splits + split) * 2;
   if (n <= 0 || key_lo > key_hi) {   // an empty range: a partial that weighs nothing
