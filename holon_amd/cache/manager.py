@@ -6,6 +6,10 @@ pool, one block table, one storage tensor `[sites, pages, page_size * elems]` â€
 the group. Groups with different needs (all tokens, a window of them) have pools of their own; a windowed group gives
 pages back as soon as the window has passed them, a finished request gives back everything.
 
+With a prefix index (`enable_prefix`) full pages of tokens are shared between requests that start alike: `adopt` gives
+a new request the cached pages of its longest known prefix, `publish` hands the pages a request has filled to the
+index, and `reserve` evicts cached pages nobody uses when the pool runs short.
+
 core/holon/core/state.py:124-554 (`StateManager`: admit/reserve/release, `BlockTable`), core/holon/core/assembly.py:
 140-189 (grouping by declaration), std/holon_std/state/paged/kind.py:10-19 (pages needed).
 """
@@ -18,6 +22,7 @@ import torch
 
 from ..parts.base import PagedState, SlotState
 from .pool import OutOfPages, PagePool
+from .prefix import PrefixIndex
 
 
 @dataclasses.dataclass
@@ -49,6 +54,9 @@ class CacheManager:
         self._free_slots = list(range(max_seqs - 1, -1, -1))
         self._live: set[int] = set()
         self.computed = [0] * (max_seqs + 1)
+        self.prefix: PrefixIndex | None = None
+        self.chain: list[list[bytes] | None] = [None] * (max_seqs + 1)   # per slot: keys of the blocks it follows
+        self.tokens_saved = 0
         num_pages = -(-tokens // page_size) + 1
         if tokens < 1:
             raise ValueError("the cache needs room for at least one token")
@@ -93,6 +101,7 @@ class CacheManager:
         slot = self._free_slots.pop()
         self._live.add(slot)
         self.computed[slot] = 0
+        self.chain[slot] = [] if self.prefix is not None else None
         for _, _, t in self.slot_states:
             t[slot].zero_()
         return slot
@@ -109,7 +118,76 @@ class CacheManager:
             g.dirty.add(slot)
         self._live.remove(slot)
         self.computed[slot] = 0
+        self.chain[slot] = None
         self._free_slots.append(slot)
+
+    # -- shared prefixes ------------------------------------------------------------------------------------------
+    def enable_prefix(self, namespace: bytes) -> bool:
+        """Share full pages between requests that start with the same tokens. Only state that a page holds whole can
+        be shared: with a windowed group (whose early pages go) or fixed-size state (which no page restores) nothing
+        is, and this returns False."""
+        if self._live:
+            raise RuntimeError("the prefix index is set up before requests are admitted")
+        if not self.groups or self.slot_states or any(g.decl.window > 0 for g in self.groups):
+            return False
+        self.prefix = PrefixIndex(namespace, self.page_size, [g.pool for g in self.groups])
+        return True
+
+    def adopt(self, slot: int, tokens: list[int]) -> int:
+        """Give a freshly admitted request the cached pages of the longest prefix of `tokens` that the index knows,
+        always leaving one token to compute. Returns the tokens it now holds (core/holon/core/state.py:180-224)."""
+        if self.prefix is None:
+            return 0
+        if self.computed[slot] or any(g.count[slot] for g in self.groups):
+            raise RuntimeError(f"slot {slot} already holds tokens")
+        blocks = self.prefix.match(tokens, (len(tokens) - 1) // self.page_size)
+        for gid, g in enumerate(self.groups):
+            for i, e in enumerate(blocks):
+                g.pool.incref(e.pages[gid])
+                g.table[slot, i] = e.pages[gid]
+            g.count[slot] = len(blocks)
+            g.dirty.add(slot)
+        self.chain[slot] = [e.key for e in blocks]
+        self.computed[slot] = len(blocks) * self.page_size
+        self.tokens_saved += self.computed[slot]
+        return self.computed[slot]
+
+    def publish(self, slot: int, tokens: list[int]) -> None:
+        """Hand the pages that the request has filled since the last call to the index. Where another request stored
+        the same block first, the request takes that page for its own copy, which is given back
+        (core/holon/core/state.py:433-462)."""
+        chain = self.chain[slot]
+        if self.prefix is None or chain is None:
+            return
+        P, idx = self.page_size, self.prefix
+        for i in range(len(chain), min(self.computed[slot], len(tokens)) // P):
+            prev = chain[-1] if chain else None
+            block = tuple(tokens[i * P: (i + 1) * P])
+            key = idx.key(prev, block)
+            mine = tuple(int(g.table[slot, i]) for g in self.groups)
+            e = idx.get(key)
+            if e is None:
+                idx.store(key, prev, block, mine)
+            elif e.parent == prev and e.tokens == block:
+                if e.pages != mine:
+                    for g, theirs, own in zip(self.groups, e.pages, mine):
+                        g.pool.incref(theirs)
+                        g.table[slot, i] = theirs
+                        g.pool.decref(own)
+                        g.dirty.add(slot)
+                idx.touch(e)
+            else:                                     # two prefixes under one key: this request shares nothing further
+                self.chain[slot] = None
+                return
+            chain.append(key)
+
+    def flush_prefix(self) -> None:
+        """Forget every cached block (after the weights changed, say); live requests keep their pages but publish
+        nothing further."""
+        if self.prefix is not None:
+            self.prefix.flush()
+            for slot in self._live:
+                self.chain[slot] = None
 
     # -- pages ----------------------------------------------------------------------------------------------------
     def pages_needed(self, slot: int, total: int) -> list[int]:
@@ -124,8 +202,13 @@ class CacheManager:
         if total > self.max_model_len:
             raise ValueError(f"{total} tokens exceed max_model_len {self.max_model_len}")
         need = self.pages_needed(slot, total)
-        if any(n > g.pool.free for n, g in zip(need, self.groups)):
-            return False
+        short = max((n - g.pool.free for n, g in zip(need, self.groups)), default=0)
+        if short > 0:                   # cached pages nobody uses make room, a few more than needed at a time
+            if self.prefix is None:
+                return False
+            self.prefix.evict(max(short, self.groups[0].pool.usable // 64))
+            if any(n > g.pool.free for n, g in zip(need, self.groups)):
+                return False
         for n, g in zip(need, self.groups):
             if n:
                 pages = g.pool.alloc(n)
@@ -160,9 +243,18 @@ class CacheManager:
         """Whether releasing the requests in `victims` (slots) would let `slot` (None: a new request) keep `total`
         tokens (core/holon/core/state.py:478-497)."""
         want = -(-total // self.page_size)
-        for g in self.groups:
+        for gid, g in enumerate(self.groups):
             have = g.count[slot] if slot is not None else 0
-            freed = sum(g.count[v] - g.first[v] for v in victims)
+            if self.prefix is None:
+                freed = sum(g.count[v] - g.first[v] for v in victims)
+            else:                       # a page comes free when only the index, or nobody, would still hold it
+                dropped: dict[int, int] = {}
+                for v in victims:
+                    for p in g.table[v, g.first[v]: g.count[v]].tolist():
+                        dropped[p] = dropped.get(p, 0) + 1
+                cached = self.prefix.is_cached(gid)
+                freed = sum(1 for p in cached if g.pool.refs(p) - dropped.get(p, 0) == 1)
+                freed += sum(1 for p, n in dropped.items() if p not in cached and g.pool.refs(p) == n)
             if want - have > g.pool.free + freed:
                 return False
         return True
@@ -206,6 +298,11 @@ class CacheManager:
                     raise AssertionError(f"group {g.gid}: slot {slot}'s table does not match what it holds")
                 for p in inside.tolist():
                     held[p] = held.get(p, 0) + 1
+            if self.prefix is not None:
+                for e in self.prefix.entries.values():
+                    held[e.pages[g.gid]] = held.get(e.pages[g.gid], 0) + 1
+                    if e.parent is not None and e.parent not in self.prefix.entries:
+                        raise AssertionError(f"cached block {e.key.hex()} outlived the block before it")
             free = set(g.pool._free)
             if len(free) != len(g.pool._free):
                 raise AssertionError(f"group {g.gid}: a page is in the free list twice")

@@ -13,6 +13,7 @@ sampler draws a token for every row that ended its prompt or decoded, the commit
 from __future__ import annotations
 
 import dataclasses
+import hashlib
 import itertools
 import secrets
 import sys
@@ -66,6 +67,11 @@ class Engine:
         if not self.cache.fits_alone(cfg.max_model_len):
             raise OutOfPages(f"the cache holds {tokens} tokens, fewer than one request of max_model_len "
                              f"{cfg.max_model_len}; lower max_model_len or give the cache more memory")
+        if cfg.prefix_cache:
+            identity = repr((self.spec, cfg.dtype, cfg.page_size)).encode()
+            if not self.cache.enable_prefix(hashlib.blake2b(identity, digest_size=16).digest()):
+                print("holon_amd: this model keeps state that pages do not hold whole; prompts share nothing",
+                      file=sys.stderr)
         self.sampler = Sampler(self.kernels, cfg.max_seqs, device)
         self.sched = Scheduler(self.cache, cfg.max_step_tokens, cfg.max_model_len, cfg.chunk_with_decode,
                                on_admit=lambda seq: self.sampler.admit(seq.slot, seq.params))
@@ -137,7 +143,13 @@ class Engine:
         return {"waiting": len(self.sched.waiting), "running": len(self.sched.running),
                 "preemptions": self.sched.preemptions, "mixed_steps": self.sched.mixed_steps, "steps": self.steps,
                 "free_pages": min((g.pool.free for g in self.cache.groups), default=0),
-                "graphs": len(getattr(self.runner, "graphs", {}))}
+                "graphs": len(getattr(self.runner, "graphs", {})),
+                "prefix_tokens_saved": self.cache.tokens_saved,
+                "cached_pages": len(self.cache.prefix.entries) if self.cache.prefix is not None else 0}
+
+    def flush_prefix(self) -> None:
+        """Drop the cached prompt blocks (core/holon/core/engine.py:418-420)."""
+        self.cache.flush_prefix()
 
     def close(self) -> None:
         self._live.clear()
@@ -179,6 +191,7 @@ class Engine:
         deltas, at = [], 0
         for seq, n, m in rows:
             seq.num_computed += n
+            self.cache.publish(seq.slot, seq.tokens)
             if not m:
                 continue
             token = tokens[at]

@@ -87,6 +87,7 @@ class Scheduler:
         if slot is None:
             return False
         seq.slot = slot
+        seq.num_computed = self.cache.adopt(slot, seq.tokens)    # the cached start of its tokens is not run again
         if self.on_admit is not None:
             self.on_admit(seq)
         return True

@@ -33,8 +33,10 @@ def _engine(folder, device, **kw):
 
 
 def _released(engine):
+    """No request holds anything: every page is free or held by the prefix index alone."""
     engine.cache.check()
-    return all(g.pool.free == g.pool.usable for g in engine.cache.groups) and \
+    cached = len(engine.cache.prefix.entries) if engine.cache.prefix is not None else 0
+    return all(g.pool.free + cached == g.pool.usable for g in engine.cache.groups) and \
         engine.cache.free_slots == engine.cache.max_seqs
 
 
@@ -106,6 +108,38 @@ def test_preemption_changes_nothing(folders, device):
     assert _released(tight)
     greedy = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
     assert tight.generate(prompts, greedy) == roomy.generate(prompts, greedy)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_prompts_that_start_alike_share_their_cache_and_generate_the_same(folders, device):
+    """Four prompts over one 37-token start, then the same four again, with sampling: every draw is still the plain
+    model's at the plain uniform. The second round (and, within a round, every prompt admitted after the first has
+    published) computes only what the cache does not hold; a tight pool evicts cached pages and preempts between."""
+    plain = PlainQwen3(folders["Bu"])
+    start = H.random_ids(37, 384, 90)
+    prompts = [start + H.random_ids(n, 384, 91 + n) for n in (1, 6, 12, 3)] + [start[:33]]
+    params = SamplingParams(temperature=0.7, seed=11, max_tokens=10, ignore_eos=True)
+    want = [_plain_sampled(plain, p, 10, 11, 0.7) for p in prompts]
+    shape = dict(page_size=4, max_seqs=3, max_step_tokens=24, max_model_len=64)
+    engine = _engine(folders["Bu"], device, **shape)
+    assert engine.generate(prompts, params) == want
+    first = engine.stats()["prefix_tokens_saved"]
+    assert first >= 36                                     # the third and later prompts were admitted after a publish
+    assert engine.generate(prompts, params) == want
+    assert engine.stats()["prefix_tokens_saved"] - first >= 4 * 36 + 32      # all but a tail of every prompt
+    assert _released(engine)
+    two = engine.generate([prompts[1], prompts[1]], params)                 # the same prompt twice, side by side
+    assert two == [want[1], want[1]]
+    off = _engine(folders["Bu"], device, prefix_cache=False, **shape)
+    assert off.generate(prompts, params) == want and off.stats()["prefix_tokens_saved"] == 0
+    tight = _engine(folders["Bu"], device, cache_tokens=72, **shape)        # 18 pages: one request of 64, little more
+    assert tight.generate(prompts, params) == want
+    assert tight.generate(prompts[::-1], params) == want[::-1]
+    assert tight.cache.prefix.evictions > 0 and tight.stats()["preemptions"] > 0
+    assert _released(tight)
+    tight.flush_prefix()
+    assert all(g.pool.free == g.pool.usable for g in tight.cache.groups)
+    assert tight.generate(prompts[:2], params) == want[:2]
 
 
 @pytest.mark.parametrize("device", DEVICES)

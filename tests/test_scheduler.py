@@ -15,9 +15,11 @@ from holon_amd.model import Site
 from holon_amd.parts.base import PagedState
 
 
-def _sched(tokens=64, page=4, max_seqs=4, max_model_len=32, max_step_tokens=16, chunk_with_decode=0):
+def _sched(tokens=64, page=4, max_seqs=4, max_model_len=32, max_step_tokens=16, chunk_with_decode=0, prefix=False):
     cache = CacheManager([Site(run=0, layer=0)], [[PagedState("kv", 2)]], page_size=page, max_seqs=max_seqs,
                          max_model_len=max_model_len, tokens=tokens, device=torch.device("cpu"), dtype=torch.float32)
+    if prefix:
+        assert cache.enable_prefix(b"sched")
     return Scheduler(cache, max_step_tokens, max_model_len, chunk_with_decode), cache
 
 
@@ -30,6 +32,7 @@ def _commit(sched, cache, rows):
     for seq, n, m in rows:
         cache.advance(seq.slot, seq.num_computed + n)
         seq.num_computed += n
+        cache.publish(seq.slot, seq.tokens)
         if m:
             if seq.status is not Status.RUNNING:
                 sched.finished_prefill(seq)
@@ -112,14 +115,16 @@ def test_a_request_alone_that_cannot_grow_preempts_itself_and_the_engine_would_r
     assert sched.schedule() is None or a.status is Status.PREEMPTED
 
 
+@pytest.mark.parametrize("prefix", [False, True], ids=["", "shared-prefixes"])
 @pytest.mark.parametrize("mode", [0, 5])
 @pytest.mark.parametrize("seed", range(12))
-def test_every_request_finishes_under_random_traffic(seed, mode):
+def test_every_request_finishes_under_random_traffic(seed, mode, prefix):
+    """Prompts are 0, 1, 2, ...: each is the start of every longer one, so with a prefix index most admissions hit."""
     rng = random.Random(seed)
     max_len = 32
     sched, cache = _sched(tokens=rng.choice([32, 40, 64, 96]), page=rng.choice([1, 4, 8]), max_seqs=rng.choice([2, 4]),
                           max_model_len=max_len, max_step_tokens=rng.choice([12, 16, 40]) if not mode else 16,
-                          chunk_with_decode=mode)
+                          chunk_with_decode=mode, prefix=prefix)
     assert cache.fits_alone(max_len)
     seqs = [_seq(i, rng.randint(1, 24), max_tokens=rng.randint(1, 12)) for i in range(14)]
     pending = list(seqs)
@@ -145,4 +150,7 @@ def test_every_request_finishes_under_random_traffic(seed, mode):
         cache.check()
     assert all(s.status is Status.FINISHED for s in seqs)
     assert all(len(s.tokens) - s.prompt_len == min(s.params.max_tokens, max_len - s.prompt_len) for s in seqs)
+    if prefix:
+        assert cache.tokens_saved > 0
+        cache.flush_prefix()
     assert all(g.pool.free == g.pool.usable for g in cache.groups) and cache.free_slots == cache.max_seqs
