@@ -56,15 +56,20 @@ class SamplingParams:
     presence_penalty: float = 0.0        # penalties are refused when set, as the reference refuses them
     frequency_penalty: float = 0.0
     repetition_penalty: float = 1.0
+    n: int = 1                           # sequences drawn for the prompt; sequence i uses `sequence_seed(seed, i)`
     max_tokens: int | None = None
     ignore_eos: bool = False
     stop_token_ids: tuple[int, ...] = ()
     seed: int | None = None
     logprobs: int | None = None          # with every generated token: its log-probability and the k most likely (k <= 32)
+    prompt_logprobs: int | None = None   # the same for the prompt's own tokens, each given the tokens before it
 
     def check(self) -> None:
-        if self.logprobs is not None and not 0 <= self.logprobs <= 32:
-            raise ValueError("logprobs must be between 0 and 32")
+        for name in ("logprobs", "prompt_logprobs"):
+            if getattr(self, name) is not None and not 0 <= getattr(self, name) <= 32:
+                raise ValueError(f"{name} must be between 0 and 32")
+        if self.n < 1:
+            raise ValueError(f"n must be >= 1, got {self.n}")
         if self.presence_penalty or self.frequency_penalty or self.repetition_penalty != 1:
             raise NotImplementedError("sampling penalties are not supported")
         if self.temperature < 0 or not 0 < self.top_p <= 1 or self.top_k < 0 or not 0 <= self.min_p <= 1:

@@ -33,6 +33,8 @@ from .loading import attach_cache, build_from_spec, default_kernels, torch_dtype
 from .request import Logprobs, Seq, Status, TokenDelta
 from .scheduler import Scheduler
 
+PROMPT_LOGPROB_PORTION = 256        # core/holon/core/executor.py:645-666 takes the prompt's logits in pieces as small
+
 
 def activation_bytes(spec, max_step_tokens: int, max_seqs: int, itemsize: int) -> int:
     """An upper estimate of what one step allocates beside weights and cache: a few copies of the widest activation
@@ -74,10 +76,17 @@ class Engine:
                       file=sys.stderr)
         self.sampler = Sampler(self.kernels, cfg.max_seqs, device)
         self.sched = Scheduler(self.cache, cfg.max_step_tokens, cfg.max_model_len, cfg.chunk_with_decode,
-                               on_admit=lambda seq: self.sampler.admit(seq.slot, seq.params))
+                               on_admit=self._on_admit)
         self._ids = itertools.count()
-        self._live: dict[str, Seq] = {}
+        self._live: dict[str, list[Seq]] = {}
+        self._siblings: dict[Seq, list[Seq]] = {}         # n > 1: waiting until the first sequence's prompt is cached
+        self._prompt_lp: dict[Seq, Logprobs] = {}         # sequences still gathering prompt log-probabilities
         self.steps = 0
+
+    def _on_admit(self, seq: Seq) -> None:
+        self.sampler.admit(seq.slot, seq.params)
+        if seq.cached_tokens is None:                     # the first admission's hit; later ones are recomputation
+            seq.cached_tokens = seq.num_computed
 
     @classmethod
     def from_random(cls, config_json: dict, seed: int, cfg: EngineConfig, kernels=None) -> "Engine":
@@ -123,21 +132,50 @@ class Engine:
         rid = rid if rid is not None else str(next(self._ids))
         if rid in self._live:
             raise ValueError(f"request id {rid!r} is already in flight")
-        seed = p.seed if p.seed is not None else secrets.randbits(63)
-        seq = Seq(rid=rid, tokens=list(token_ids), params=dataclasses.replace(p, seed=sequence_seed(seed, 0)))
-        self._live[rid] = seq
-        self.sched.add(seq)
+        base = p.seed if p.seed is not None else secrets.randbits(63)
+        for i in range(p.n):                # a concrete seed per sequence: its draws depend on nothing else
+            child = dataclasses.replace(p, seed=sequence_seed(base, i),
+                                        prompt_logprobs=p.prompt_logprobs if i == 0 else None)
+            seq = Seq(rid=rid, tokens=list(token_ids), params=child, index=i)
+            self._live.setdefault(rid, []).append(seq)
+            if child.prompt_logprobs is not None:         # every position computed, in portions whose logits stay small
+                seq.share_prefix, seq.portion_cap = False, PROMPT_LOGPROB_PORTION
+                self._prompt_lp[seq] = Logprobs([], [], [])
+            if i == 0 or self.cache.prefix is None:
+                self.sched.add(seq)
+                first = seq
+            else:                                         # siblings start from the first sequence's cached prompt
+                self._siblings.setdefault(first, []).append(seq)
         return rid
 
     def has_work(self) -> bool:
         return bool(self.sched.waiting or self.sched.running)
 
+    def idle_for(self) -> float | None:
+        """How long a serving loop may wait for new requests before its next `step`: 0 while a request can run, None
+        (as long as it likes) when there is no work."""
+        return 0.0 if self.has_work() else None
+
+    def drain(self) -> list[TokenDelta]:
+        """Nothing runs on the device after this returns. Every step is committed before `step` returns, so there is
+        never one in flight."""
+        if self.device.type == "cuda":
+            torch.cuda.synchronize(self.device)
+        return []
+
     def abort(self, rid: str, reason: str = "abort") -> list[TokenDelta]:
-        seq = self._live.pop(rid, None)
-        if seq is None or seq.status is Status.FINISHED:
-            return []
-        self.sched.finish(seq, reason)
-        return [TokenDelta(rid, [], reason)]
+        """Finish every sequence of request `rid` now: one delta each, siblings that never started included."""
+        deltas = []
+        for seq in self._live.pop(rid, []):
+            for sibling in self._siblings.pop(seq, []):
+                sibling.status = Status.FINISHED
+                deltas.append(TokenDelta(rid, [], reason, index=sibling.index))
+            if seq.status is Status.FINISHED:
+                continue
+            self.sched.finish(seq, reason)
+            self._prompt_lp.pop(seq, None)
+            deltas.append(TokenDelta(rid, [], reason, index=seq.index))
+        return deltas
 
     def stats(self) -> dict[str, int]:
         return {"waiting": len(self.sched.waiting), "running": len(self.sched.running),
@@ -155,7 +193,9 @@ class Engine:
         self._live.clear()
 
     def generate(self, prompts: list[list[int]], params: SamplingParams | None = None) -> list[list[int]]:
-        """Token ids generated for each prompt."""
+        """Token ids generated for each prompt (one sequence per prompt)."""
+        if params is not None and params.n != 1:
+            raise ValueError("generate() returns one sequence per prompt; step() streams n > 1")
         rids = [self.add(p, params) for p in prompts]
         out: dict[str, list[int]] = {r: [] for r in rids}
         pending = set(rids)
@@ -175,10 +215,25 @@ class Engine:
             if self.has_work():
                 raise RuntimeError("the scheduler made no progress with requests pending")
             return []
-        step_rows = [StepRow(seq.slot, seq.num_computed, seq.tokens[seq.num_computed: seq.num_computed + n],
-                             [n - 1] if m else []) for seq, n, m in rows]
+        step_rows, owed, places, at = [], [], [], 0
+        for seq, n, m in rows:
+            want = list(range(*self._prompt_places(seq, n))) if seq in self._prompt_lp else []
+            if want:
+                owed.append((seq, at, len(want), seq.tokens[seq.num_computed + want[0] + 1:
+                                                            seq.num_computed + want[-1] + 2]))
+            at += len(want)
+            if m:
+                places.append(at)
+                want.append(n - 1)
+                at += 1
+            step_rows.append(StepRow(seq.slot, seq.num_computed, seq.tokens[seq.num_computed: seq.num_computed + n],
+                                     want))
         logits = self.runner.run(step_rows)
         self.steps += 1
+        for seq, lo, count, targets in owed:
+            self._gather_prompt_logprobs(seq, logits[lo: lo + count], targets)
+        if owed and places:
+            logits = logits.index_select(0, torch.tensor(places, device=logits.device))
         sampled = [(seq, n) for seq, n, m in rows if m]
         tokens: list[int] = []
         if sampled:
@@ -201,12 +256,37 @@ class Engine:
             if seq.status is not Status.RUNNING:
                 self.sched.finished_prefill(seq)
             seq.tokens.append(token)
+            for sibling in reversed(self._siblings.pop(seq, [])):         # its prompt is cached now
+                self.sched.add(sibling, front=True)
             reason = self._finish_reason(seq, token)
             if reason:
                 self.sched.finish(seq, reason)
-                self._live.pop(seq.rid, None)
-            deltas.append(TokenDelta(seq.rid, [token], reason, lp))
+                live = self._live.get(seq.rid, [])
+                if seq in live:
+                    live.remove(seq)
+                if not live:
+                    self._live.pop(seq.rid, None)
+            first = not seq.reported
+            seq.reported = True
+            deltas.append(TokenDelta(seq.rid, [token], reason, lp, seq.index,
+                                     self._prompt_lp.pop(seq, None) if first else None,
+                                     seq.cached_tokens if first else None))
         return deltas
+
+    def _prompt_places(self, seq: Seq, n: int) -> tuple[int, int]:
+        """The places among the next `n` tokens of `seq` whose logits predict a prompt token not yet recorded (a
+        request preempted in its prompt computes some again). core/holon/core/engine.py:588-602."""
+        start, have = seq.num_computed, len(self._prompt_lp[seq].token)
+        lo, hi = max(start, have), min(start + n, seq.prompt_len - 1)
+        return (lo - start, hi - start) if lo < hi else (0, 0)
+
+    def _gather_prompt_logprobs(self, seq: Seq, logits: torch.Tensor, targets: list[int]) -> None:
+        acc, k = self._prompt_lp[seq], seq.params.prompt_logprobs
+        tokens = torch.tensor(targets, dtype=torch.int32, device=logits.device)
+        lp, ids, top = (t.tolist() for t in self.kernels.logprobs(logits.contiguous(), tokens, k))
+        acc.token += lp
+        acc.top_ids += [row[:k] for row in ids]
+        acc.top += [row[:k] for row in top]
 
     def _finish_reason(self, seq: Seq, token: int) -> str | None:
         p = seq.params

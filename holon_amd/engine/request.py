@@ -25,6 +25,11 @@ class Seq:
     num_computed: int = 0                # tokens whose state is in the cache
     status: Status = Status.WAITING
     finish_reason: str | None = None
+    index: int = 0                       # which of its request's `n` sequences
+    portion_cap: int = 0                 # most prompt tokens one step runs of it (0: what the budget allows)
+    share_prefix: bool = True            # False: every position is computed, whatever the cache holds
+    cached_tokens: int | None = None     # what the prefix cache served at its first admission
+    reported: bool = False               # its first delta has gone out
 
     def __post_init__(self) -> None:
         if not self.prompt_len:
@@ -49,3 +54,6 @@ class TokenDelta:
     token_ids: list[int]
     finish_reason: str | None = None
     logprobs: Logprobs | None = None
+    index: int = 0                       # which of the request's `n` sequences
+    prompt_logprobs: Logprobs | None = None   # with the first delta: prompt positions 1 .. n-1 (the first has no context)
+    cached_tokens: int | None = None     # with the first delta: tokens the prefix cache served at the first admission

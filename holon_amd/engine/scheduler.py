@@ -58,7 +58,7 @@ class Scheduler:
         for seq in list(self.waiting):
             if budget <= 0 or (seq.slot < 0 and not self._fit(seq, None)):
                 break                                           # first come first served: nobody skips ahead
-            n = min(len(seq.tokens) - seq.num_computed, budget)
+            n = min(len(seq.tokens) - seq.num_computed, budget, seq.portion_cap or budget)
             if not self._fit(seq, seq.num_computed + n):
                 break
             rows.append((seq, n, int(seq.num_computed + n == len(seq.tokens))))
@@ -87,7 +87,8 @@ class Scheduler:
         if slot is None:
             return False
         seq.slot = slot
-        seq.num_computed = self.cache.adopt(slot, seq.tokens)    # the cached start of its tokens is not run again
+        if seq.share_prefix:                       # the cached start of its tokens is not run again
+            seq.num_computed = self.cache.adopt(slot, seq.tokens)
         if self.on_admit is not None:
             self.on_admit(seq)
         return True

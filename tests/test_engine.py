@@ -262,6 +262,64 @@ def test_logprobs_of_generated_tokens(folders, device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_several_sequences_of_one_prompt_and_prompt_logprobs(folders, device):
+    """`n` sequences of one prompt: sequence i draws with `sequence_seed(seed, i)`; with the prefix cache the siblings
+    start from the first one's cached prompt. `prompt_logprobs`: every prompt token's log-probability given the tokens
+    before it, with the first delta; such a request computes every position, in portions, also when it is preempted
+    in its prompt and runs part of it again."""
+    plain = PlainQwen3(folders["Bu"])
+    prompt = H.random_ids(29, 384, 123)
+    engine = _engine(folders["Bu"], device, page_size=4, max_seqs=4, max_step_tokens=10, max_model_len=48)
+    params = SamplingParams(temperature=0.8, seed=5, n=3, max_tokens=6, ignore_eos=True, prompt_logprobs=2)
+    rid = engine.add(prompt, params)
+    out, first = {0: [], 1: [], 2: []}, {}
+    while engine.has_work():
+        for d in engine.step():
+            assert d.rid == rid
+            first.setdefault(d.index, d)
+            assert (d.cached_tokens is None) == (d is not first[d.index])
+            out[d.index] += d.token_ids
+    assert out == {i: _plain_sampled(plain, prompt, 6, S.sequence_seed(5, i), 0.8) for i in range(3)}
+    assert len({tuple(o) for o in out.values()}) == 3
+    assert [first[i].cached_tokens for i in range(3)] == [0, 28, 28]        # 7 whole pages of the 29 tokens
+    want = plain.logits(prompt)[:-1].log_softmax(-1)
+    top = want.topk(2)
+    lp = first[0].prompt_logprobs
+    assert first[1].prompt_logprobs is None and len(lp.token) == 28
+    assert lp.top_ids == top.indices.tolist()
+    torch.testing.assert_close(torch.tensor(lp.top), top.values, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(torch.tensor(lp.token), want.gather(-1, torch.tensor(prompt[1:])[:, None])[:, 0],
+                               rtol=1e-4, atol=1e-4)
+    assert _released(engine)
+    with pytest.raises(ValueError):
+        engine.generate([prompt], params)
+    with pytest.raises(ValueError):
+        engine.add(prompt, SamplingParams(n=0))
+    engine.add(prompt, params, rid="gone")
+    engine.step()
+    assert sorted(d.index for d in engine.abort("gone")) == [0, 1, 2] and not engine.has_work()
+    assert engine.idle_for() is None and engine.drain() == [] and _released(engine)
+    # preempted in its prompt: the older requests grow, the youngest gives way and later runs its prompt again
+    tight = _engine(folders["Bu"], device, page_size=4, max_seqs=3, max_step_tokens=10, max_model_len=48,
+                    cache_tokens=60, chunk_with_decode=6, prefix_cache=False)
+    greedy = SamplingParams(temperature=0.0, max_tokens=14, ignore_eos=True)
+    for n in (12, 9):
+        tight.add(H.random_ids(n, 384, 130 + n), greedy)
+    for _ in range(2):
+        tight.step()
+    tight.add(prompt, SamplingParams(temperature=0.0, max_tokens=3, ignore_eos=True, prompt_logprobs=0), rid="lp")
+    got = None
+    while tight.has_work():
+        for d in tight.step():
+            if d.rid == "lp" and d.prompt_logprobs is not None:
+                got = d.prompt_logprobs
+    assert tight.stats()["preemptions"] > 0
+    assert got.top_ids == [[]] * 28
+    torch.testing.assert_close(torch.tensor(got.token), want.gather(-1, torch.tensor(prompt[1:])[:, None])[:, 0],
+                               rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_end_of_sequence_tokens_stop_a_request(folders, tmp_path, device):
     """eos_token_id of config.json and generation_config.json (an int or a list) ends a request with "stop" and the
     token is delivered; ignore_eos generates on."""
