@@ -15,7 +15,9 @@
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
-template <int MT, int WPB, int UNROLL, typename OutT, bool TILED>
+// RESID: y is the residual stream, y = round(y + round(product)) in place: the add that the next norm's kernel would
+// have done, with its roundings.
+template <int MT, int WPB, int UNROLL, typename OutT, bool TILED, bool RESID = false>
 __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                 const bf16_t* __restrict__ w, OutT* __restrict__ y,
                                                                 int M, int N, int K) {
@@ -94,24 +96,35 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
       ushort4 o;
       o.x = float_to_bf16(acc[t][0]); o.y = float_to_bf16(acc[t][1]);
       o.z = float_to_bf16(acc[t][2]); o.w = float_to_bf16(acc[t][3]);
+      if constexpr (RESID) {
+        const ushort4 r = *reinterpret_cast<const ushort4*>(yp);
+        o.x = float_to_bf16(bf16_to_float(r.x) + bf16_to_float(o.x));
+        o.y = float_to_bf16(bf16_to_float(r.y) + bf16_to_float(o.y));
+        o.z = float_to_bf16(bf16_to_float(r.z) + bf16_to_float(o.z));
+        o.w = float_to_bf16(bf16_to_float(r.w) + bf16_to_float(o.w));
+      }
       *reinterpret_cast<ushort4*>(yp) = o;
     }
   }
 }
 
-template <int MT, int WPB, int UNROLL, typename OutT>
+template <int MT, int WPB, int UNROLL, typename OutT, bool RESID>
 static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s) {
-  if (tiled)
-    gemm_skinny_kernel<MT, WPB, UNROLL, OutT, true><<<N / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
+  const dim3 grid(N / 16), block(WPB * 64);
+  if constexpr (RESID)
+    gemm_skinny_kernel<MT, WPB, UNROLL, OutT, true, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
                                                                                 (OutT*)y, M, N, K);
+  else if (tiled)
+    gemm_skinny_kernel<MT, WPB, UNROLL, OutT, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
+                                                                          (OutT*)y, M, N, K);
   else
-    gemm_skinny_kernel<MT, WPB, UNROLL, OutT, false><<<N / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                                 (OutT*)y, M, N, K);
+    gemm_skinny_kernel<MT, WPB, UNROLL, OutT, false><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
+                                                                           (OutT*)y, M, N, K);
 }
 
 // How many waves share a tile, from the shapes alone (so a result never depends on M): wide outputs have tiles
 // enough to fill the GPU with few waves each and long loops; narrow ones split K 16 ways. Measured on MI355X.
-template <int MT, typename OutT>
+template <int MT, typename OutT, bool RESID = false>
 static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s) {
   const int tiles = N / 16;
   int wpb = MT >= 3 ? 8 : 16;                  // 16 waves of 3 or 4 token tiles run out of registers
@@ -120,15 +133,15 @@ static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K
   constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
   switch (wpb) {
     case 16:
-      if constexpr (MT < 3) launch_skinny<MT, 16, U, OutT>(x, w, y, M, N, K, tiled, s);
+      if constexpr (MT < 3) launch_skinny<MT, 16, U, OutT, RESID>(x, w, y, M, N, K, tiled, s);
       break;
-    case 8: launch_skinny<MT, 8, U, OutT>(x, w, y, M, N, K, tiled, s); break;
+    case 8: launch_skinny<MT, 8, U, OutT, RESID>(x, w, y, M, N, K, tiled, s); break;
     case 4:
-      if constexpr (MT == 1) launch_skinny<MT, 4, 16, OutT>(x, w, y, M, N, K, tiled, s);
-      else launch_skinny<MT, 4, U, OutT>(x, w, y, M, N, K, tiled, s);
+      if constexpr (MT == 1) launch_skinny<MT, 4, 16, OutT, RESID>(x, w, y, M, N, K, tiled, s);
+      else launch_skinny<MT, 4, U, OutT, RESID>(x, w, y, M, N, K, tiled, s);
       break;
-    case 2: launch_skinny<MT, 2, U, OutT>(x, w, y, M, N, K, tiled, s); break;
-    default: launch_skinny<MT, 1, U, OutT>(x, w, y, M, N, K, tiled, s); break;
+    case 2: launch_skinny<MT, 2, U, OutT, RESID>(x, w, y, M, N, K, tiled, s); break;
+    default: launch_skinny<MT, 1, U, OutT, RESID>(x, w, y, M, N, K, tiled, s); break;
   }
   return 0;
 }
@@ -149,6 +162,17 @@ extern "C" int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int
   else pick_waves<MT, bf16_t>(x, w, y, M, N, K, tiled != 0, s)
   if (mt == 1) { SKINNY(1); } else if (mt == 2) { SKINNY(2); } else if (mt == 3) { SKINNY(3); } else { SKINNY(4); }
 #undef SKINNY
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+// residual[M, N] += x[M, K] w^T in place (the product rounded, then the sum rounded), for one tile of rows (M <= 16)
+// over tiled weights: the output projection's product and the residual add that follows it, in one kernel.
+extern "C" int holon_gemm_skinny_add_bf16(const void* x, const void* w_tiled, void* residual, int M, int N, int K,
+                                          void* stream) {
+  HOLON_CHECK(M >= 1 && M <= 16 && holon_gemm_skinny_supported(M, N, K),
+              "gemm (few rows, added to the residual): M=%d N=%d K=%d not served (M <= 16, N %% 16, K %% 32)", M, N, K);
+  pick_waves<1, bf16_t, true>(x, w_tiled, residual, M, N, K, true, (hipStream_t)stream);
   HOLON_LAUNCH_OK();
   return 0;
 }

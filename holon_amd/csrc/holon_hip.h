@@ -49,6 +49,9 @@ int holon_attention_decode_bf16(const void* q, void* out, const void* pages, con
 int holon_gemm_skinny_supported(int M, int N, int K);
 int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_f32, int tiled,
                            void* stream);
+// residual[M, N] = round(residual + round(x w^T)) in place, M <= 16, tiled weights: the product and the residual add
+// that follows it in one kernel.
+int holon_gemm_skinny_add_bf16(const void* x, const void* w_tiled, void* residual, int M, int N, int K, void* stream);
 // y[M, I] = round(silu(round(x gate^T))) * round(x up^T) with w = [gate; up] ([2I, K]), M <= 32.
 int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int I, int K, int tiled, void* stream);
 int holon_tile_weight_bf16(const void* w, void* tiled, int N, int K, void* stream);

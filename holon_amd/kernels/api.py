@@ -60,6 +60,11 @@ class Kernels(Protocol):
     def tile_weight(self, weight: torch.Tensor) -> torch.Tensor | None:
         """Once per weight after loading: a copy in the layout steps of few rows stream fastest, or None."""
 
+    def linear_add(self, x: torch.Tensor, weight: torch.Tensor, tiled: torch.Tensor | None, residual: torch.Tensor
+                   ) -> bool:
+        """residual += linear(x, weight) in place in one kernel: the product rounded to dtype, then the sum rounded,
+        as the add of `add_rmsnorm` does. False when not fused for this shape; then nothing was done."""
+
     def linear_silu_mul(self, x: torch.Tensor, weight: torch.Tensor, tiled: torch.Tensor | None = None
                         ) -> torch.Tensor | None:
         """silu_mul(linear(x, weight)) fused, with the composition's roundings; None when not fused for this shape."""

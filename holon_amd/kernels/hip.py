@@ -68,6 +68,7 @@ class HipKernels:
             "holon_gemm_skinny_supported": [_I, _I, _I],
             "holon_gemm_skinny_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
             "holon_tile_weight_bf16": [_P, _P, _I, _I, _P],
+            "holon_gemm_skinny_add_bf16": [_P, _P, _P, _I, _I, _I, _P],
             "holon_gemm_skinny_glu_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
             "holon_argmax": [_P, _P, _I, _I, _P],
             "holon_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
@@ -162,6 +163,19 @@ class HipKernels:
         # the vendor library's product, float32 accumulation (no reduced-precision mode for float32 operands)
         y = torch.matmul(x, weight.t())
         return y if out_dtype in (None, y.dtype) else y.to(out_dtype)
+
+    def linear_add(self, x, weight, tiled, residual):
+        (m, k), n = x.shape, weight.shape[0]
+        if not (tiled is not None and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                and residual.dtype == torch.bfloat16 and 1 <= m <= min(self.skinny_rows, 16) and weight.shape[1] == k
+                and k >= 256 and x.is_contiguous() and residual.is_contiguous()
+                and self.lib.holon_gemm_skinny_supported(m, n, k)):
+            return False
+        if tuple(residual.shape) != (m, n):
+            raise KernelError(f"linear_add: residual {tuple(residual.shape)} for a product of {(m, n)}")
+        self._call(self.lib.holon_gemm_skinny_add_bf16, x.data_ptr(), tiled.data_ptr(), residual.data_ptr(), m, n, k,
+                   self._stream())
+        return True
 
     def linear_silu_mul(self, x, weight, tiled=None):
         """silu_mul(linear(x, weight)) in one kernel for steps of few rows, with the roundings of the two kernels one

@@ -69,6 +69,8 @@ class Build:
 class Part:
     """Base of all parts. Subclasses call `declare` for tensors and `attach` for sub-parts in `__init__`."""
 
+    adds_residual = False     # its forward accepts `residual=h`: it may add its result into h and return None
+
     def __init__(self, build: Build) -> None:
         self.build = build
         self.kernels = build.kernels

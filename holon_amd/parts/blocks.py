@@ -23,12 +23,11 @@ class PreNorm(Part):
 
     def forward(self, h: torch.Tensor, delta: torch.Tensor | None, step, site
                 ) -> tuple[torch.Tensor, torch.Tensor | None]:
-        """The residual stream is `h + delta` on entry and on return; `h` is updated in place."""
-        if delta is None:
-            a = self.input_norm(h)
-        else:
-            a, h = self.input_norm.add(delta, h)
-        x, h = self.post_norm.add(self.mixer(a, step, site), h)
-        return h, self.ffn(x, step)
+        """The residual stream is `h + delta` on entry and on return; `h` is updated in place. A part that can add
+        its result into `h` inside its own kernel (`adds_residual`) is given `h`; it returns None when it did."""
+        a = self.input_norm(h) if delta is None else self.input_norm.add(delta, h)[0]
+        mixed = self.mixer(a, step, site, **({"residual": h} if self.mixer.adds_residual else {}))
+        x = self.post_norm(h) if mixed is None else self.post_norm.add(mixed, h)[0]
+        return h, self.ffn(x, step, **({"residual": h} if self.ffn.adds_residual else {}))
 
     __call__ = forward

@@ -26,10 +26,12 @@ class SwiGLU(Part):
         self.drop("up_proj")
         self._children["gate_up"] = self.gate_up
 
-    def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
+    adds_residual = True
+
+    def forward(self, x: torch.Tensor, step=None, residual: torch.Tensor | None = None) -> torch.Tensor | None:
         y = self.kernels.linear_silu_mul(x, self.gate_up.weight, self.gate_up.tiled)   # fused for steps of few rows
         if y is None:
             y = self.kernels.silu_mul(self.gate_up(x))
-        return self.down_proj(y)
+        return self.down_proj(y, residual=residual)
 
     __call__ = forward

@@ -18,7 +18,12 @@ class Linear(Part):
         if self.weight is not None and self.build.decode_copy:
             self.tiled = self.kernels.tile_weight(self.weight)
 
-    def forward(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, out_dtype: torch.dtype | None = None, residual: torch.Tensor | None = None
+                ) -> torch.Tensor | None:
+        """x W^T. With `residual`, the product is added into it in place when one kernel can do both (steps of few
+        rows), and None is returned; otherwise the product is returned and the add is the caller's."""
+        if residual is not None and out_dtype is None and self.kernels.linear_add(x, self.weight, self.tiled, residual):
+            return None
         return self.kernels.linear(x, self.weight, out_dtype, self.tiled)
 
     __call__ = forward

@@ -54,7 +54,9 @@ class GQA(Part):
                 and pos["position"] in ("rope", "none"):
             self._fused = {"eps": norm["eps"], "table": pos["table"]}
 
-    def forward(self, x: torch.Tensor, step, site) -> torch.Tensor:
+    adds_residual = True
+
+    def forward(self, x: torch.Tensor, step, site, residual: torch.Tensor | None = None) -> torch.Tensor | None:
         k = self.kernels
         t, hq, hkv, d = x.shape[0], self.heads, self.kv_heads, self.head_dim
         view = step.paged[site.group]
@@ -77,6 +79,6 @@ class GQA(Part):
                 v = qkv[:, (hq + hkv) * d:].contiguous().view(t, hkv, d)
                 k.kv_write(kk, v, pages, view.write_page, view.write_off, view.page_size)
         out = k.paged_attention(q, pages, view.table, step.rows, view.page_size, self.scale, self.window)
-        return self.o_proj(out.view(t, hq * d))
+        return self.o_proj(out.view(t, hq * d), residual=residual)
 
     __call__ = forward

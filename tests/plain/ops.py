@@ -58,6 +58,10 @@ class TorchKernels:
     def linear(self, x, weight, out_dtype=None, tiled=None):
         return (_up(x) @ _up(weight).T).to(out_dtype or x.dtype)
 
+    def linear_add(self, x, weight, tiled, residual):
+        residual.copy_((_up(residual) + _up(self.linear(x, weight))).to(residual.dtype))
+        return True
+
     def linear_silu_mul(self, x, weight, tiled=None):
         return None
 

@@ -256,6 +256,34 @@ def test_fused_gate_up_is_the_two_kernels(hip, monkeypatch):
     assert hip.linear_silu_mul(_randn(4, 256, dtype=torch.float32), _randn(64, 256, dtype=torch.float32)) is None
 
 
+def test_product_added_into_the_residual(hip):
+    """`linear_add` = the few-row product, rounded, added into the residual, rounded: the bits of the two kernels one
+    after the other, since the product is the same kernel's."""
+    from holon_amd.kernels.hip import KernelError
+    bf = torch.bfloat16
+    for m, k, n in ((1, 4096, 6144), (8, 4096, 4096), (16, 12288, 4096), (3, 256, 48), (5, 1024, 208), (2, 4096, 24576)):
+        x, w = _randn(m, k, dtype=bf, seed=50), _randn(n, k, dtype=bf, seed=51, scale=0.05)
+        tiled = hip.tile_weight(w)
+        res = _randn(m, n, dtype=bf, seed=53, scale=2.0)
+        exact = res.double() + (x.double() @ w.double().T).to(bf).double()
+        want = (res.float() + hip.linear(x, w, None, tiled).float()).to(bf)
+        mine = res.clone()
+        assert hip.linear_add(x, w, tiled, mine) is True
+        assert torch.equal(mine, want), (m, k, n)
+        assert H.op_budget_usage(mine, exact, bf, k) <= 1, (m, k, n)
+    # what is not served is left to the kernels one after the other, and nothing is touched
+    w = _randn(512, 4096, dtype=bf, seed=55, scale=0.02)
+    tiled = hip.tile_weight(w)
+    res = _randn(17, 512, dtype=bf)
+    keep = res.clone()
+    assert hip.linear_add(_randn(17, 4096, dtype=bf), w, tiled, res) is False and torch.equal(res, keep)
+    assert hip.linear_add(_randn(4, 4096, dtype=bf), w, None, res[:4].contiguous()) is False
+    f32 = torch.float32
+    assert hip.linear_add(_randn(4, 256, dtype=f32), _randn(64, 256, dtype=f32), None, _randn(4, 64, dtype=f32)) is False
+    with pytest.raises(KernelError):
+        hip.linear_add(_randn(16, 4096, dtype=bf), w, tiled, _randn(16, 500, dtype=bf))
+
+
 def test_logprobs_kernel(hip):
     g = torch.Generator().manual_seed(40)
     for rows, vocab, k in ((3, 151_936, 20), (5, 97, 5), (2, 40, 0), (1, 33, 32)):
