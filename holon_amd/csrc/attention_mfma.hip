@@ -531,53 +531,63 @@ __global__ void __launch_bounds__(64) attn_decode_kernel(AttnArgs a) {
   if (g == 0) { pml[0] = m[0]; pml[1] = lt; }
 }
 
-// out[row, head, :] = sum_i 2^(m_i - M) o_i / sum_i 2^(m_i - M) l_i, splits in index order. One wave per (row, head):
-// lane s holds split s's weight (at most 64 splits), every lane a few dims of the output.
-__global__ void __launch_bounds__(64) attn_merge_kernel(const float* __restrict__ part_o,
-                                                        const float* __restrict__ part_ml, bf16_t* __restrict__ out,
-                                                        const int32_t* __restrict__ row_ids,
-                                                        const int32_t* __restrict__ qstart, int heads, int splits,
-                                                        int head_dim) {
-  const int ri = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+// out[row, head, :] = sum_i 2^(m_i - M) o_i / sum_i 2^(m_i - M) l_i over the splits (at most 64). One block of four
+// waves per (row, head): thread (group, d4) adds the partials of splits group, group + NG, ... for four dims, all of
+// its loads under way at once; the groups' sums are then added in group order. The order of every sum depends on
+// the number of splits and the head size alone.
+template <int D>
+__global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict__ part_o,
+                                                         const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+                                                         const int32_t* __restrict__ row_ids,
+                                                         const int32_t* __restrict__ qstart, int heads, int splits) {
+  constexpr int LANES = D / 4;            // threads across one partial
+  constexpr int NG = 256 / LANES;         // groups of splits
+  constexpr int PER = (64 + NG - 1) / NG; // splits a thread may own
+  __shared__ float weight[64];
+  __shared__ float inv_denom;
+  __shared__ f32x4_t sums[NG][LANES];
+  const int ri = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int token = qstart[row_ids[ri]];
   const float* ml = part_ml + ((int64_t)ri * heads + h) * splits * 2;
-  const float* po = part_o + ((int64_t)ri * heads + h) * splits * head_dim;
-  float m_s = -INFINITY, l_s = 0.f;
-  if (lane < splits) {
-    const float2 v = *reinterpret_cast<const float2*>(ml + 2 * lane);
-    m_s = v.x;
-    l_s = v.y;
+  const float* po = part_o + ((int64_t)ri * heads + h) * splits * D;
+  const int group = tid / LANES, d0 = 4 * (tid % LANES);
+  f32x4_t v[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i)            // asked for before the weights are known: an empty split's values are dropped
+    v[i] = *reinterpret_cast<const f32x4_t*>(po + (int64_t)min(group + i * NG, splits - 1) * D + d0);
+  if (tid < WAVE) {
+    float m_s = -INFINITY, l_s = 0.f;
+    if (tid < splits) {
+      const float2 x = *reinterpret_cast<const float2*>(ml + 2 * tid);
+      m_s = x.x;
+      l_s = x.y;
+    }
+    if (!(l_s > 0.f)) m_s = -INFINITY;
+    const float big = wave_max(m_s);
+    const float w_s = l_s > 0.f ? exp2f(m_s - big) : 0.f;
+    float denom = 0.f;                     // in split order
+    for (int s = 0; s < splits; ++s) denom += __shfl(w_s * l_s, s, WAVE);
+    weight[tid] = w_s;
+    if (tid == 0) inv_denom = denom > 0.f ? 1.0f / denom : 0.f;
   }
-  if (!(l_s > 0.f)) m_s = -INFINITY;
-  const float big = wave_max(m_s);
-  const float w_s = l_s > 0.f ? exp2f(m_s - big) : 0.f;
-  // the denominator in split order
-  float denom = 0.f;
-  for (int s = 0; s < splits; ++s) denom += __shfl(w_s * l_s, s, WAVE);
-  const float inv = denom > 0.f ? 1.0f / denom : 0.f;
-  for (int base = 0; base < head_dim; base += 4 * WAVE) {   // every lane walks the loop: the shuffles read all lanes
-    const int d0 = base + 4 * lane;
-    const bool mine = d0 < head_dim;
-    const float* src = po + (mine ? d0 : 0);
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < splits; s0 += 8) {
-      // eight partials requested at once (unconditionally: an empty split's values are dropped below, not skipped,
-      // so that the loads do not wait for one another)
-      f32x4_t v[8];
+  __syncthreads();
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const f32x4_t*>(src + (int64_t)min(s0 + i, splits - 1) * head_dim);
+  for (int i = 0; i < PER; ++i) {
+    const int sp = group + i * NG;
+    const float w = sp < splits ? weight[sp] : 0.f;
+    if (w > 0.f) acc += w * v[i];
+  }
+  sums[group][tid % LANES] = acc;
+  __syncthreads();
+  if (group == 0) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float w = __shfl(w_s, min(s0 + i, splits - 1), WAVE);
-        if (s0 + i < splits && w > 0.f) acc += w * v[i];
-      }
-    }
-    if (mine) {
-      ushort4 o;
-      o.x = float_to_bf16(acc[0] * inv); o.y = float_to_bf16(acc[1] * inv);
-      o.z = float_to_bf16(acc[2] * inv); o.w = float_to_bf16(acc[3] * inv);
-      *reinterpret_cast<ushort4*>(out + ((int64_t)token * heads + h) * head_dim + d0) = o;
-    }
+    for (int gq = 1; gq < NG; ++gq) acc += sums[gq][tid];
+    const float inv = inv_denom;
+    ushort4 o;
+    o.x = float_to_bf16(acc[0] * inv); o.y = float_to_bf16(acc[1] * inv);
+    o.z = float_to_bf16(acc[2] * inv); o.w = float_to_bf16(acc[3] * inv);
+    *reinterpret_cast<ushort4*>(out + ((int64_t)token * heads + h) * D + d0) = o;
   }
 }
 
@@ -656,7 +666,12 @@ extern "C" int holon_attention_decode_bf16(const void* q, void* out, const void*
   else attn_decode_kernel<256><<<grid, 64, 0, s>>>(a);
   HOLON_LAUNCH_OK();
   dim3 mgrid(n_rows, heads);
-  attn_merge_kernel<<<mgrid, 64, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits, head_dim);
+  if (head_dim == 64)
+    attn_merge_kernel<64><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits);
+  else if (head_dim == 128)
+    attn_merge_kernel<128><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits);
+  else
+    attn_merge_kernel<256><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits);
   HOLON_LAUNCH_OK();
   return 0;
 }
