@@ -142,6 +142,56 @@ def test_prompts_that_start_alike_share_their_cache_and_generate_the_same(folder
     assert tight.generate(prompts[:2], params) == want[:2]
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_traffic_generates_what_the_plain_model_generates(folders, seed):
+    """Requests arrive while others run: prompts that share starts, pools so tight that cached pages are evicted and
+    requests preempted, portions beside decode rows or not, several sequences of a prompt. Every sequence is the
+    plain model's, drawn at the plain uniforms, whatever happened to it on the way (CPU twins of the kernels)."""
+    import random
+    rng = random.Random(seed)
+    plain = PlainQwen3(folders["Bu"])
+    page = rng.choice([4, 8])
+    max_len = 64
+    mixed = rng.choice([0, 6])
+    engine = _engine(folders["Bu"], "cpu", page_size=page, max_seqs=rng.choice([2, 3, 5]), max_model_len=max_len,
+                     max_step_tokens=rng.choice([16, 24]), chunk_with_decode=mixed,
+                     cache_tokens=rng.choice([64, 96, 160]), prefix_cache=rng.random() < 0.8)
+    starts = [H.random_ids(40, 384, 1000 * seed + i) for i in range(2)]
+    todo = []
+    for i in range(10):
+        cut = rng.randrange(0, 30)
+        prompt = rng.choice(starts)[:cut] + H.random_ids(rng.randrange(1, 12), 384, 2000 * seed + i)
+        greedy = rng.random() < 0.4
+        params = SamplingParams(temperature=0.0 if greedy else 0.9, seed=50 + i, ignore_eos=True,
+                                max_tokens=rng.randrange(1, 14), n=1 if greedy else rng.choice([1, 1, 2]),
+                                top_k=rng.choice([0, 0, 20]))
+        todo.append((f"r{i}", prompt, params))
+    want = {}
+    for rid, prompt, p in todo:
+        for i in range(p.n):
+            want[rid, i] = plain.greedy(prompt, p.max_tokens) if p.greedy else \
+                _plain_sampled(plain, prompt, p.max_tokens, S.sequence_seed(p.seed, i), p.temperature, top_k=p.top_k)
+    got = {key: [] for key in want}
+    done = set()
+    pending = list(todo)
+    for _ in range(3000):
+        while pending and rng.random() < 0.3:
+            rid, prompt, p = pending.pop(0)
+            engine.add(prompt, p, rid=rid)
+        if not engine.has_work():
+            if not pending:
+                break
+            continue
+        for d in engine.step():
+            got[d.rid, d.index] += d.token_ids
+            if d.finish_reason:
+                assert d.finish_reason == "length" and (d.rid, d.index) not in done
+                done.add((d.rid, d.index))
+        engine.cache.check()
+    assert done == set(want) and got == want
+    assert _released(engine)
+
+
 @pytest.mark.parametrize("device", DEVICES)
 def test_rejections_and_limits(folders, device):
     engine = _engine(folders["Bu"], device, page_size=4, max_seqs=3, max_step_tokens=10, max_model_len=40)
