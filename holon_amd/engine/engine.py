@@ -33,6 +33,7 @@ from .loading import attach_cache, build_from_spec, default_kernels, torch_dtype
 from .request import Logprobs, Seq, Status, TokenDelta
 from .scheduler import Scheduler
 
+CACHED_PREFIX_TOKENS = 1 << 22      # with a prefix cache the pools grow to this many tokens, if memory allows
 PROMPT_LOGPROB_PORTION = 256        # core/holon/core/executor.py:645-666 takes the prompt's logits in pieces as small
 
 
@@ -115,7 +116,9 @@ class Engine:
                   f"{max(budget, 0) / 2**30:.1f} GiB for the cache ({per_token} B a token)", file=sys.stderr)
         else:
             budget = cfg.max_seqs * cfg.max_model_len * per_token
-        tokens = min(budget // per_token, cfg.max_seqs * cfg.max_model_len)
+        live = cfg.max_seqs * cfg.max_model_len          # live requests never hold more; what is beyond keeps prompts
+        shared = CACHED_PREFIX_TOKENS if cfg.prefix_cache and self.device.type == "cuda" else 0    # others may start with
+        tokens = min(budget // per_token, max(live, shared))
         return max(int(tokens), 0) // cfg.page_size * cfg.page_size or cfg.page_size
 
     # -- requests -------------------------------------------------------------------------------------------------
