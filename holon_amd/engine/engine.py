@@ -37,16 +37,6 @@ CACHED_PREFIX_TOKENS = 1 << 22      # with a prefix cache the pools grow to this
 PROMPT_LOGPROB_PORTION = 256        # core/holon/core/executor.py:645-666 takes the prompt's logits in pieces as small
 
 
-def activation_bytes(spec, max_step_tokens: int, max_seqs: int, itemsize: int) -> int:
-    """An upper estimate of what one step allocates beside weights and cache: a few copies of the widest activation
-    per token, and float32 logits for the rows that sample."""
-    width = spec.hidden
-    for layer in spec.layers:
-        m, f = layer.mixer.get(), layer.ffn.get()
-        width = max(width, 2 * f.get("inter", 0), (m.get("heads", 0) + 2 * m.get("kv_heads", 0)) * m.get("head_dim", 0))
-    return max_step_tokens * (3 * width + 6 * spec.hidden) * itemsize + 3 * max_seqs * spec.vocab * 4 + (256 << 20)
-
-
 class Engine:
     def __init__(self, cfg: EngineConfig, kernels=None, *, random_config: dict | None = None, seed: int = 0) -> None:
         self.cfg = cfg
@@ -109,17 +99,56 @@ class Engine:
         if cfg.state_memory is not None:
             budget = cfg.state_memory
         elif self.device.type == "cuda":
+            peak = self._profile_step()
             free, _ = torch.cuda.mem_get_info(self.device)
-            item = torch.empty((), dtype=self.dtype).element_size()
-            budget = int(free * cfg.memory_fraction) - activation_bytes(self.spec, cfg.max_step_tokens, cfg.max_seqs, item)
-            print(f"holon_amd: weights {self.model.nbytes() / 2**30:.2f} GiB, {free / 2**30:.1f} GiB free, "
-                  f"{max(budget, 0) / 2**30:.1f} GiB for the cache ({per_token} B a token)", file=sys.stderr)
+            budget = int(free * cfg.memory_fraction) - peak
+            print(f"holon_amd: weights {self.model.nbytes() / 2**30:.2f} GiB, {free / 2**30:.1f} GiB free, a step takes "
+                  f"up to {peak / 2**30:.2f} GiB, {max(budget, 0) / 2**30:.1f} GiB for the cache ({per_token} B a token)",
+                  file=sys.stderr)
         else:
             budget = cfg.max_seqs * cfg.max_model_len * per_token
         live = cfg.max_seqs * cfg.max_model_len          # live requests never hold more; what is beyond keeps prompts
         shared = CACHED_PREFIX_TOKENS if cfg.prefix_cache and self.device.type == "cuda" else 0    # others may start with
         tokens = min(budget // per_token, max(live, shared))
         return max(int(tokens), 0) // cfg.page_size * cfg.page_size or cfg.page_size
+
+    def _profile_step(self) -> int:
+        """Bytes the largest steps allocate beside weights and cache, measured on a cache just large enough for them
+        (core/holon/core/executor.py:208-234): a step of `max_step_tokens` prompt tokens over as many rows as fit,
+        every row sampled, and a step of `max_seqs` decode rows, sampled with filters and log-probabilities."""
+        cfg, device = self.cfg, self.device
+        longest = cfg.max_model_len - 1
+        rows = min(cfg.max_seqs, max(1, -(-cfg.max_step_tokens // longest)))
+        per_row = min(longest, cfg.max_step_tokens // rows)
+        pages = rows * -(-(per_row + 1) // cfg.page_size) + cfg.max_seqs
+        cache, runner = attach_cache(self.model, device=device, dtype=self.dtype, kernels=self.kernels,
+                                     cache_tokens=pages * cfg.page_size, graphs=False, page_size=cfg.page_size,
+                                     max_seqs=cfg.max_seqs, max_model_len=cfg.max_model_len,
+                                     max_step_tokens=cfg.max_step_tokens)
+        sampler = Sampler(self.kernels, cfg.max_seqs, device)
+        torch.cuda.synchronize(device)
+        torch.cuda.reset_peak_memory_stats(device)
+        base = torch.cuda.memory_allocated(device)
+        slots = [cache.admit() for _ in range(min(cfg.max_seqs, cfg.max_step_tokens))]
+        params = SamplingParams(temperature=1.0, top_k=50, top_p=0.9, min_p=0.01, seed=0)
+        for slot in slots:
+            sampler.admit(slot, params)
+        for slot in slots[:rows]:
+            cache.reserve(slot, per_row)
+        runner.run([StepRow(slot, 0, [0] * per_row, [per_row - 1]) for slot in slots[:rows]])
+        for slot in slots:
+            cache.reserve(slot, cache.computed[slot] + 1)
+        logits = runner.run([StepRow(slot, cache.computed[slot], [0], [0]) for slot in slots])
+        where = np.array(slots, dtype=np.int64)
+        drawn = sampler.sample(logits, where, np.array([cache.computed[s] for s in slots], dtype=np.int64))
+        self.kernels.logprobs(logits, drawn, 32)
+        torch.cuda.synchronize(device)
+        peak = torch.cuda.max_memory_allocated(device) - base
+        del logits, drawn, runner, cache, sampler
+        for site in self.model.sites:
+            site.detach()
+        torch.cuda.empty_cache()
+        return int(peak * 1.1) + (64 << 20)           # the allocator's rounding and fragmentation
 
     # -- requests -------------------------------------------------------------------------------------------------
     def add(self, token_ids: list[int], params: SamplingParams | None = None, rid: str | None = None) -> str:

@@ -23,6 +23,10 @@ class Site:
     pages: torch.Tensor | None = None             # this site's page storage [num_pages, P * elems]
     slot_state: dict[str, torch.Tensor] = dataclasses.field(default_factory=dict)   # name -> [S+1, *shape]
 
+    def detach(self) -> None:
+        """Forget the storage a cache manager gave (before another one is made for the same model)."""
+        self.group, self.pages, self.slot_state = None, None, {}
+
 
 class Model(Part):
     def __init__(self, spec: ModelSpec, build: Build) -> None:
