@@ -54,6 +54,7 @@ class CacheManager:
         self._free_slots = list(range(max_seqs - 1, -1, -1))
         self._live: set[int] = set()
         self.computed = [0] * (max_seqs + 1)
+        self._capacity = [0] * (max_seqs + 1)          # tokens each slot's pages hold (kept beside the groups' counts)
         self.prefix: PrefixIndex | None = None
         self.chain: list[list[bytes] | None] = [None] * (max_seqs + 1)   # per slot: keys of the blocks it follows
         self.tokens_saved = 0
@@ -117,7 +118,7 @@ class CacheManager:
             g.first[slot] = g.count[slot] = 0
             g.dirty.add(slot)
         self._live.remove(slot)
-        self.computed[slot] = 0
+        self.computed[slot] = self._capacity[slot] = 0
         self.chain[slot] = None
         self._free_slots.append(slot)
 
@@ -148,7 +149,7 @@ class CacheManager:
             g.count[slot] = len(blocks)
             g.dirty.add(slot)
         self.chain[slot] = [e.key for e in blocks]
-        self.computed[slot] = len(blocks) * self.page_size
+        self.computed[slot] = self._capacity[slot] = len(blocks) * self.page_size
         self.tokens_saved += self.computed[slot]
         return self.computed[slot]
 
@@ -215,13 +216,15 @@ class CacheManager:
                 g.table[slot, g.count[slot]: g.count[slot] + n] = pages
                 g.count[slot] += n
                 g.dirty.add(slot)
+        self._capacity[slot] = min(g.count[slot] for g in self.groups) * self.page_size if self.groups \
+            else self.max_model_len
         return True
 
     def capacity(self, slot: int) -> int:
         """Tokens the request's pages hold (the smallest over groups)."""
         if not self.groups:
             return self.max_model_len
-        return min(g.count[slot] for g in self.groups) * self.page_size
+        return self._capacity[slot]
 
     def advance(self, slot: int, computed: int) -> None:
         """The request now has `computed` tokens in the cache: pages a window has passed are given back."""

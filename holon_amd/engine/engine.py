@@ -276,9 +276,12 @@ class Engine:
             lps = [t.tolist() for t in self.kernels.logprobs(logits, drawn, k)] if k >= 0 else None
             tokens = drawn.tolist()
         deltas, at = [], 0
+        chains, page = self.cache.chain, self.cache.page_size
         for seq, n, m in rows:
             seq.num_computed += n
-            self.cache.publish(seq.slot, seq.tokens)
+            chain = chains[seq.slot]                  # (the check `publish` starts with, without the call: per row, per step)
+            if chain is not None and min(seq.num_computed, len(seq.tokens)) // page > len(chain):
+                self.cache.publish(seq.slot, seq.tokens)
             if not m:
                 continue
             token = tokens[at]

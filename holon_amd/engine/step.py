@@ -42,6 +42,8 @@ class StepRunner:
         self.vocab = model.spec.vocab
         self.steps = 0
         self.pinned = device.type == "cuda"
+        self._stages: list[tuple[torch.Tensor, torch.cuda.Event] | None] = [None, None]
+        self._turn = 0
         self.use_graphs = graphs and device.type == "cuda"
         self.graphs: dict[tuple[int, int], _Graph] = {}
         self.graph_replays = 0
@@ -51,13 +53,17 @@ class StepRunner:
                 ) -> tuple[list[np.ndarray], dict]:
         """The int32 arrays of a step, in a fixed order, and the host-side facts about them."""
         cache = self.cache
-        total = int(counts.sum())
-        qstart = np.concatenate(([0], np.cumsum(counts)))
-        token_row = np.repeat(np.arange(len(slots)), counts)
-        positions = np.repeat(starts, counts) + (np.arange(total) - np.repeat(qstart[:-1], counts))
+        total, n = int(counts.sum()), len(slots)
+        if total == n:                             # one token a row: the step's shape is the batch's
+            rows = np.arange(n + 1)
+            qstart, token_row, positions, decode, chunk = rows, rows[:n], starts, rows[:n], rows[:0]
+        else:
+            qstart = np.concatenate(([0], np.cumsum(counts)))
+            token_row = np.repeat(np.arange(n), counts)
+            positions = np.repeat(starts, counts) + (np.arange(total) - np.repeat(qstart[:-1], counts))
+            decode = np.flatnonzero(counts == 1)
+            chunk = np.flatnonzero(counts > 1)
         lens = starts + counts
-        decode = np.flatnonzero(counts == 1)
-        chunk = np.flatnonzero(counts > 1)
         arrays = [tokens, positions, token_row, slots, starts, lens, qstart, decode, chunk]
         for g in cache.groups:
             page, off = cache.write_targets(g.gid, slots[token_row], positions)
@@ -68,18 +74,33 @@ class StepRunner:
                      max_chunk_len=int(lens[chunk].max()) if len(chunk) else 0)
         return arrays, facts
 
-    def _to_device(self, arrays: list[np.ndarray], arena: torch.Tensor | None = None) -> list[torch.Tensor]:
-        """Several int32 arrays to the device in one copy (into `arena`, a buffer of fixed address, when given)."""
+    def _to_device(self, arrays: list[np.ndarray], arena: torch.Tensor | None = None, views: bool = True
+                   ) -> list[torch.Tensor]:
+        """Several int32 arrays to the device in one copy (into `arena`, a buffer of fixed address, when given). The
+        host side is one of two pinned buffers used in turn; a buffer is written again only after its last copy ran."""
         sizes = [a.size for a in arrays]
-        flat = np.concatenate([a.astype(np.int32, copy=False).ravel() for a in arrays])
-        host = torch.from_numpy(flat)
+        total = sum(sizes)
         if self.pinned:
-            host = host.pin_memory()
+            stage = self._stages[self._turn]
+            self._turn ^= 1
+            if stage is None or stage[0].numel() < total:
+                stage = (torch.empty(max(total, 4096) * 2, dtype=torch.int32).pin_memory(), torch.cuda.Event())
+                self._stages[self._turn ^ 1] = stage
+            else:
+                stage[1].synchronize()
+            host = stage[0][:total]
+        else:
+            host = torch.empty(total, dtype=torch.int32)
+        np.concatenate([a.ravel() for a in arrays], out=host.numpy(), casting="unsafe")
         if arena is None:
             dev = host.to(self.device, non_blocking=True)
         else:
-            dev = arena[: flat.size]
+            dev = arena[:total]
             dev.copy_(host, non_blocking=True)
+        if self.pinned:
+            stage[1].record()
+        if not views:                              # a graph's step already holds its views of the arena
+            return []
         out, at = [], 0
         for n in sizes:
             out.append(dev[at: at + n])
@@ -101,32 +122,35 @@ class StepRunner:
         if not rows:
             raise ValueError("a step needs at least one row")
         cache = self.cache
-        counts = np.array([len(r.tokens) for r in rows], dtype=np.int64)
-        if (counts < 1).any():
-            raise ValueError("every row of a step brings at least one token")
-        total = int(counts.sum())
-        if total > self.max_step_tokens:
-            raise ValueError(f"the step has {total} tokens; max_step_tokens is {self.max_step_tokens}")
-        if len({r.slot for r in rows}) != len(rows):
-            raise ValueError("a request appears twice in one step")
-        slots = np.array([r.slot for r in rows], dtype=np.int64)
-        starts = np.array([r.start for r in rows], dtype=np.int64)
-        for r, n in zip(rows, counts):
-            if r.start != cache.computed[r.slot]:
-                raise ValueError(f"slot {r.slot}: the row starts at {r.start}, the cache holds {cache.computed[r.slot]}")
-            if r.start + n > cache.capacity(r.slot):
+        computed, paged = cache.computed, bool(cache.groups)
+        slots, starts, counts, wanted, flat = [], [], [], [], []
+        at = 0
+        for b, r in enumerate(rows):
+            n = len(r.tokens)
+            if n < 1:
+                raise ValueError("every row of a step brings at least one token")
+            if r.start != computed[r.slot]:
+                raise ValueError(f"slot {r.slot}: the row starts at {r.start}, the cache holds {computed[r.slot]}")
+            if paged and r.start + n > cache.capacity(r.slot):
                 raise RuntimeError(f"slot {r.slot}: no pages reserved for tokens up to {r.start + n}")
-        tokens = np.concatenate([np.asarray(r.tokens, dtype=np.int64) for r in rows])
+            for w in r.want:
+                if not 0 <= w < n:
+                    raise ValueError(f"row {b}: wanted place {w} is not among its {n} tokens")
+                wanted.append(at + w)
+            slots.append(r.slot)
+            starts.append(r.start)
+            counts.append(n)
+            flat.extend(r.tokens)
+            at += n
+        if at > self.max_step_tokens:
+            raise ValueError(f"the step has {at} tokens; max_step_tokens is {self.max_step_tokens}")
+        if len(set(slots)) != len(slots):
+            raise ValueError("a request appears twice in one step")
+        tokens = np.array(flat, dtype=np.int64)
         if tokens.min() < 0 or tokens.max() >= self.vocab:
             raise ValueError(f"token ids must lie in [0, {self.vocab})")
-        qstart = np.concatenate(([0], np.cumsum(counts)))
-        wanted = []
-        for b, r in enumerate(rows):
-            for w in r.want:
-                if not 0 <= w < counts[b]:
-                    raise ValueError(f"row {b}: wanted place {w} is not among its {counts[b]} tokens")
-                wanted.append(qstart[b] + w)
-        return slots, starts, counts, tokens, np.asarray(wanted, dtype=np.int64)
+        return (np.array(slots, dtype=np.int64), np.array(starts, dtype=np.int64), np.array(counts, dtype=np.int64),
+                tokens, np.array(wanted, dtype=np.int64))
 
     def prepare(self, rows: list[StepRow]) -> tuple[Step, np.ndarray]:
         """Device inputs of a step, and the flat indices of the tokens whose logits are wanted (in row order, then in
@@ -185,7 +209,7 @@ class StepRunner:
             g = _Graph(arena=arena, step=self._step(self._to_device(arrays, arena), facts, slots, starts, counts))
             self.graphs[key] = g
         else:
-            self._to_device(arrays, g.arena)
+            self._to_device(arrays, g.arena, views=False)
         g.runs += 1
         if g.graph is None and g.runs == 1:        # the first step of a bucket: eagerly, on the fixed buffers
             return self._forward(g.step, None)[:n]
