@@ -1,0 +1,131 @@
+"""Decode and prefill throughput of the engine at the Qwen3-8B shape with random weights, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--no-points]
+    python -m holon_amd bench ...          (the same)
+
+One JSON line: decoded tokens a second at the given batch (default 8) with every request near a context of 4,096 tokens
+(a 2,048-token prompt and 2,048 generated tokens), plus the prefill of one 2,048-token prompt, the decode step's memory
+roofline, and decode at batch 1 and 64. A step is one decode step of the engine: scheduling, the model, sampling and
+the commit. The engine is one process on one GPU; for --gpus > 1 a line says so and the exit code is 2.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+HBM_GBS = 8000.0                 # MI355X published peaks
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
+QWEN3_8B = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 36, "hidden_size": 4096,
+            "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 12288,
+            "vocab_size": 151936, "rope_theta": 1e6, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
+            "max_position_embeddings": 40960}
+CONTEXT, PROMPT = 4096, 2048
+
+
+def main(argv: list[str] | None = None) -> int:
+    ap = argparse.ArgumentParser(prog="bench", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"],
+                    help="fewer layers than the configuration has (recorded in config)")
+    ap.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-graphs", action="store_true")
+    a = ap.parse_args(argv)
+    if a.gpus != 1:
+        print(f"bench.py: this engine serves on one GPU; --gpus {a.gpus} is not a configuration it has", flush=True)
+        return 2
+
+    import torch
+
+    from .config import EngineConfig, SamplingParams
+    from .engine.engine import Engine
+    from .kernels import build as kernel_build
+
+    if kernel_build.find_library() is None:
+        kernel_build.build()
+    cfg_json = dict(QWEN3_8B, num_hidden_layers=a.layers)
+    max_batch = max(a.batch, 1 if a.no_points else 64)
+    engine = Engine.from_random(cfg_json, seed=0, cfg=EngineConfig(
+        model="random:qwen3-8b", device="cuda:0", dtype=a.dtype, page_size=16, max_seqs=max_batch,
+        max_model_len=CONTEXT + 16, max_step_tokens=4096, cache_tokens=max_batch * (CONTEXT + 16),
+        graphs=not a.no_graphs))
+    spec, c = engine.spec, cfg_json
+    item = 2 if a.dtype == "bfloat16" else 4
+    g = torch.Generator().manual_seed(0)
+    greedy = lambda n: SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True)
+
+    def decode(batch: int, steps: int, warmup: int) -> tuple[float, float]:
+        """(ms per decode step, mean context) for `batch` requests whose contexts end at CONTEXT."""
+        start = CONTEXT - steps - warmup - 1
+        for _ in range(batch):
+            engine.add(torch.randint(0, c["vocab_size"], (start,), generator=g).tolist(), greedy(steps + warmup + 1))
+        while engine.sched.waiting:                              # prompts, cut by the step budget
+            engine.step()
+        for _ in range(warmup):
+            engine.step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            engine.step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        while engine.has_work():
+            engine.step()
+        return ms, start + 1 + warmup + steps / 2
+
+    def prefill(tokens: int) -> float:
+        best = float("inf")
+        for _ in range(3):                     # another prompt each time: nothing of it is in the prefix cache
+            ids = torch.randint(0, c["vocab_size"], (tokens,), generator=g).tolist()
+            engine.add(ids, greedy(1))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            engine.step()
+            torch.cuda.synchronize()
+            best = min(best, (time.perf_counter() - t0) * 1e3)
+            assert not engine.has_work()
+        return best
+
+    h, hq, hkv, d, inter, v, layers = (c["hidden_size"], c["num_attention_heads"], c["num_key_value_heads"],
+                                       c["head_dim"], c["intermediate_size"], c["vocab_size"], a.layers)
+    layer_params = h * (hq + 2 * hkv) * d + hq * d * h + 3 * h * inter
+    weight_bytes = (layers * (layer_params + 2 * h + 2 * d) + h + h * v) * item      # every weight a decode step reads
+    kv_token_bytes = layers * 2 * hkv * d * item
+    pre_ms = prefill(PROMPT)
+    pre_flops = layers * (2 * PROMPT * layer_params + 2 * hq * d * PROMPT * PROMPT) + 2 * h * v
+    ms, ctx = decode(a.batch, a.steps, a.warmup)
+    step_bytes = weight_bytes + a.batch * ctx * kv_token_bytes
+    achieved = step_bytes / (ms * 1e-3) / 1e9
+    points = {}
+    if not a.no_points:
+        for b in (1, 64):
+            pms, _ = decode(b, min(a.steps, 32), min(a.warmup, 4))
+            points[f"decode_b{b}"] = round(b / (pms * 1e-3), 1)
+    line = {
+        "metric": "decode tok/s at batch 8 (context 4,096), Qwen3-8B shape", "value": round(a.batch / (ms * 1e-3), 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (random weights, uniform random token ids)",
+        "config": {"model": "Qwen3-8B shape", "layers": layers, "layers_of_config": QWEN3_8B["num_hidden_layers"],
+                   "hidden": h, "heads": hq, "kv_heads": hkv, "head_dim": d, "intermediate": inter, "vocab": v,
+                   "tied": False, "global_batch": a.batch, "seq_len": CONTEXT, "prompt_len": PROMPT, "page_size": 16,
+                   "parallelism": "single GPU", "graphs": not a.no_graphs, "mean_context": round(ctx, 1)},
+        "prefill": {"value": round(PROMPT / (pre_ms * 1e-3), 1), "tokens": PROMPT, "ms": round(pre_ms, 3),
+                    "frac": round(pre_flops / (pre_ms * 1e-3) / PEAK_FLOPS[a.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBS, 4)},
+        "points": points,
+    }
+    if engine.stats()["prefix_tokens_saved"]:
+        raise RuntimeError("the prefix cache served part of a timed prompt: the figures above would count work not done")
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

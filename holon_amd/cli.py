@@ -4,6 +4,7 @@
     random           write a model folder with random weights from a configuration and a seed
     replay           trace replay (what bin/trace_run runs)
     models           the architectures this build serves
+    bench            decode and prefill throughput at the Qwen3-8B shape (what bench.py at the repository's root runs)
 
 Engine flags are made from `EngineConfig`'s fields, one flag a field with the field's help line, booleans as
 --x / --no-x, as the reference's `holon serve` makes them (core/holon/core/cli.py:52-80).
@@ -44,18 +45,32 @@ def _ids(text: str) -> list[int]:
     return [int(t) for t in text.replace(",", " ").split()]
 
 
+def _tokenizer(folder: str):
+    """The checkpoint's own tokenizer (tokenizer.json), for prompts given as text. core/holon/api/frontend.py:55-70
+    keeps tokenisation outside the engine; so does this: the engine sees ids only."""
+    path = pathlib.Path(folder) / "tokenizer.json"
+    if not path.is_file():
+        raise SystemExit(f"--prompt needs {path}; give token ids with --prompt-ids instead")
+    from tokenizers import Tokenizer
+    return Tokenizer.from_file(str(path))
+
+
 def generate_main(argv: list[str]) -> int:
-    ap = argparse.ArgumentParser(prog="holon_amd generate", description="Generate token ids for prompts of token ids.")
+    ap = argparse.ArgumentParser(prog="holon_amd generate", description="Generate tokens for prompts of token ids "
+                                 "(printed as ids) or of text (printed as text, with the folder's tokenizer.json).")
     ap.add_argument("model", help="model folder (config.json, *.safetensors)")
     ap.add_argument("--prompt-ids", action="append", default=[], metavar="IDS",
                     help="a prompt as token ids separated by spaces or commas; may be given several times")
     ap.add_argument("--prompt-file", help="a file with one prompt of token ids per line")
+    ap.add_argument("--prompt", action="append", default=[], metavar="TEXT",
+                    help="a prompt as text, encoded with the model folder's tokenizer.json; may be given several times")
     ap.add_argument("--max-tokens", type=int, default=16)
     ap.add_argument("--temperature", type=float, default=0.0)
     ap.add_argument("--top-k", type=int, default=0)
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--min-p", type=float, default=0.0)
     ap.add_argument("--seed", type=int, default=None)
+    ap.add_argument("--n", type=int, default=1, help="sequences per prompt, printed one a line in order")
     ap.add_argument("--ignore-eos", action=argparse.BooleanOptionalAction, default=False)
     ap.add_argument("--stats", action="store_true", help="print the engine's counters to stderr at the end")
     engine_flags(ap.add_argument_group("engine"))
@@ -63,14 +78,24 @@ def generate_main(argv: list[str]) -> int:
     prompts = [_ids(p) for p in a.prompt_ids]
     if a.prompt_file:
         prompts += [_ids(line) for line in pathlib.Path(a.prompt_file).read_text().splitlines() if line.strip()]
+    as_text = len(prompts)                          # prompts from here on were given as text and are answered as text
+    tokenizer = _tokenizer(a.model) if a.prompt else None
+    prompts += [tokenizer.encode(text).ids for text in a.prompt]
     if not prompts:
-        ap.error("give at least one prompt (--prompt-ids or --prompt-file)")
+        ap.error("give at least one prompt (--prompt-ids, --prompt-file or --prompt)")
     from .engine.engine import Engine
     engine = Engine(engine_config(a.model, a))
     params = SamplingParams(temperature=a.temperature, top_k=a.top_k, top_p=a.top_p, min_p=a.min_p, seed=a.seed,
-                            max_tokens=a.max_tokens, ignore_eos=a.ignore_eos)
-    for out in engine.generate(prompts, params):
-        print(" ".join(str(t) for t in out), flush=True)
+                            max_tokens=a.max_tokens, ignore_eos=a.ignore_eos, n=a.n)
+    rids = [engine.add(p, params) for p in prompts]
+    out: dict[tuple[str, int], list[int]] = {(rid, i): [] for rid in rids for i in range(a.n)}
+    while engine.has_work():
+        for d in engine.step():
+            out[d.rid, d.index] += d.token_ids
+    for at, rid in enumerate(rids):
+        for i in range(a.n):
+            ids = out[rid, i]
+            print(tokenizer.decode(ids) if at >= as_text else " ".join(str(t) for t in ids), flush=True)
     if a.stats:
         print(json.dumps(engine.stats()), file=sys.stderr)
     engine.close()
@@ -133,7 +158,13 @@ def models_main(argv: list[str]) -> int:
     return 0
 
 
-COMMANDS = {"generate": generate_main, "random": random_main, "replay": replay_main, "models": models_main}
+def bench_main(argv: list[str]) -> int:
+    from .benchmark import main as bench
+    return bench(argv)
+
+
+COMMANDS = {"generate": generate_main, "random": random_main, "replay": replay_main, "models": models_main,
+            "bench": bench_main}
 
 
 def main(argv: list[str] | None = None) -> int:

@@ -277,6 +277,35 @@ def test_command_line_generates_and_sizes_its_cache(folders):
     assert "for the cache" in run.stderr and '"preemptions": 0' in run.stderr
 
 
+@pytest.mark.gpu
+def test_command_line_takes_text_with_the_folders_tokenizer(folders, tmp_path):
+    """`--prompt TEXT` is encoded with the folder's tokenizer.json and answered as text; `--n` sequences a prompt, one
+    a line. The tokenizer is a word list made here ("w0" ... "w383"), so ids and words map one to one."""
+    import shutil
+    import subprocess
+    import sys
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    plain = PlainQwen3(folders["Bu"])
+    folder = tmp_path / "with-tokenizer"
+    shutil.copytree(folders["Bu"], folder)
+    tok = Tokenizer(models.WordLevel({f"w{i}": i for i in range(384)}, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.WhitespaceSplit()
+    tok.save(str(folder / "tokenizer.json"))
+    prompt = H.random_ids(9, 384, 77)
+    cmd = [sys.executable, "-m", "holon_amd", "generate", str(folder), "--dtype", "float32", "--max-tokens", "5",
+           "--temperature", "0.8", "--seed", "3", "--n", "2", "--ignore-eos", "--max-seqs", "4", "--max-model-len", "64",
+           "--cache-tokens", "256", "--prompt", " ".join(f"w{t}" for t in prompt), "--prompt-ids",
+           " ".join(map(str, prompt))]
+    run = subprocess.run(cmd, capture_output=True, text=True, timeout=110)
+    assert run.returncode == 0, run.stderr[-2000:]
+    want = [_plain_sampled(plain, prompt, 5, S.sequence_seed(3, i), 0.8) for i in range(2)]
+    lines = run.stdout.strip().splitlines()
+    assert lines[:2] == [" ".join(map(str, w)) for w in want]                 # the prompt given as ids, answered as ids
+    assert lines[2:] == [" ".join(f"w{t}" for t in w) for w in want]          # the prompt given as text, as text
+    missing = subprocess.run(cmd[:4] + [str(folders["Bu"]), "--prompt", "w1"], capture_output=True, text=True, timeout=110)
+    assert missing.returncode != 0 and "tokenizer.json" in missing.stderr
+
+
 def test_bench_refuses_more_than_one_gpu():
     import pathlib
     import subprocess
