@@ -31,6 +31,7 @@ class EngineConfig:
     state_memory: int | None = _setting(None, "bytes for state pools; default: from memory_fraction")
     cache_tokens: int | None = _setting(None, "tokens of paged state per pool (overrides state_memory)")
     prefix_cache: bool = _setting(True, "reuse cached prompt blocks across requests")
+    overlap: bool = _setting(True, "schedule and launch the next step while the last one runs")
     graphs: bool = _setting(True, "replay decode steps from HIP graphs, per batch-size bucket")
     decode_weight_copy: bool = _setting(True, "keep a second copy of every projection in the tile layout that steps of "
                                               "few rows stream fastest (doubles the weights' memory)")

@@ -4,11 +4,17 @@
 #include "holon_hip.h"
 
 // ---------------------------------------------------------------------------------------------------------------
+// take_slot / last_token (both or neither): token t is last_token[take_slot[t]] where take_slot[t] >= 0, a token that
+// the previous step drew and that never left the device.
 template <typename T>
-__global__ void embedding_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table, T* __restrict__ out,
-                                 int hidden) {
+__global__ void embedding_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ take_slot,
+                                 const int32_t* __restrict__ last_token, const T* __restrict__ table,
+                                 T* __restrict__ out, int hidden, int vocab) {
   const int64_t t = blockIdx.x;
-  const T* src = table + (int64_t)ids[t] * hidden;
+  int id = ids[t];
+  if (take_slot != nullptr && take_slot[t] >= 0) id = last_token[take_slot[t]];
+  id = min(max(id, 0), vocab - 1);             // (the host checks the ids it sends; a drawn token is in range)
+  const T* src = table + (int64_t)id * hidden;
   T* dst = out + t * hidden;
   constexpr int V = Elem<T>::kVec;
   if (hidden % V == 0) {
@@ -20,15 +26,19 @@ __global__ void embedding_kernel(const int32_t* __restrict__ ids, const T* __res
   }
 }
 
-extern "C" int holon_embedding(const int32_t* ids, const void* table, void* out, int tokens, int hidden, int vocab,
-                               int dtype, void* stream) {
+extern "C" int holon_embedding(const int32_t* ids, const int32_t* take_slot, const int32_t* last_token,
+                               const void* table, void* out, int tokens, int hidden, int vocab, int dtype,
+                               void* stream) {
   HOLON_CHECK(tokens >= 0 && hidden > 0 && vocab > 0, "embedding: bad sizes tokens=%d hidden=%d", tokens, hidden);
+  HOLON_CHECK((take_slot == nullptr) == (last_token == nullptr), "embedding: slots to take tokens from need the tokens");
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == HOLON_F32)
-    embedding_kernel<float><<<tokens, 256, 0, s>>>(ids, (const float*)table, (float*)out, hidden);
+    embedding_kernel<float><<<tokens, 256, 0, s>>>(ids, take_slot, last_token, (const float*)table, (float*)out,
+                                                   hidden, vocab);
   else
-    embedding_kernel<bf16_t><<<tokens, 256, 0, s>>>(ids, (const bf16_t*)table, (bf16_t*)out, hidden);
+    embedding_kernel<bf16_t><<<tokens, 256, 0, s>>>(ids, take_slot, last_token, (const bf16_t*)table, (bf16_t*)out,
+                                                    hidden, vocab);
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -10,8 +10,10 @@ extern "C" {
 const char* holon_last_error(void);
 int holon_abi_version(void);
 
-int holon_embedding(const int32_t* ids, const void* table, void* out, int tokens, int hidden, int vocab, int dtype,
-                    void* stream);
+// out[t] = table[ids[t]]; with take_slot and last_token (both or neither), token t is last_token[take_slot[t]] where
+// take_slot[t] >= 0: a token the previous step drew and left on the device.
+int holon_embedding(const int32_t* ids, const int32_t* take_slot, const int32_t* last_token, const void* table, void* out,
+                    int tokens, int hidden, int vocab, int dtype, void* stream);
 // y = rmsnorm(x) over rows of `dim`; with `residual`: residual += x (rounded), y = rmsnorm(residual).
 int holon_rmsnorm(const void* x, void* residual, const void* weight, void* y, int64_t rows, int dim, float eps,
                   int dtype, void* stream);
@@ -56,6 +58,9 @@ int holon_gemm_skinny_add_bf16(const void* x, const void* w_tiled, void* residua
 int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int I, int K, int tiled, void* stream);
 int holon_tile_weight_bf16(const void* w, void* tiled, int N, int K, void* stream);
 int holon_argmax(const float* logits, int32_t* out, int rows, int vocab, void* stream);
+// last_token[slots[r]] = tokens[r] for r < rows (slots are distinct; last_token has n_slots entries).
+int holon_store_tokens(int32_t* last_token, const int32_t* slots, const int32_t* tokens, int rows, int n_slots,
+                       void* stream);
 int holon_sample(const float* logits, int32_t* out, int rows, int vocab, const float* temperature,
                  const int32_t* top_k, const float* top_p, const float* min_p, const int64_t* seeds,
                  const int64_t* positions, void* stream);

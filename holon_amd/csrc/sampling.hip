@@ -60,6 +60,23 @@ extern "C" int holon_argmax(const float* logits, int32_t* out, int rows, int voc
   return 0;
 }
 
+// last_token[slots[r]] = tokens[r]: the drawn tokens kept on the device, by slot, for the rows of the next step that
+// are scheduled before these tokens reach the host.
+__global__ void store_tokens_kernel(int32_t* __restrict__ last_token, const int32_t* __restrict__ slots,
+                                    const int32_t* __restrict__ tokens, int rows, int n_slots) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r < rows && slots[r] >= 0 && slots[r] < n_slots) last_token[slots[r]] = tokens[r];
+}
+
+extern "C" int holon_store_tokens(int32_t* last_token, const int32_t* slots, const int32_t* tokens, int rows,
+                                  int n_slots, void* stream) {
+  HOLON_CHECK(rows >= 0 && n_slots > 0, "store_tokens: bad sizes");
+  if (rows == 0) return 0;
+  store_tokens_kernel<<<(rows + 255) / 256, 256, 0, (hipStream_t)stream>>>(last_token, slots, tokens, rows, n_slots);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
 // lowbias32, and the uniform of (seed, position): 24 bits, in (0, 1).
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {
   x ^= x >> 16; x *= 0x7FEB352Du; x ^= x >> 15; x *= 0x846CA68Bu; x ^= x >> 16;

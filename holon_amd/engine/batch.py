@@ -19,6 +19,8 @@ class StepRow:
     start: int
     tokens: list[int]
     want: list[int] = dataclasses.field(default_factory=list)
+    on_device: bool = False                      # its one token is the one the previous step drew for this slot and
+                                                 # left on the device (`tokens` then holds a placeholder)
 
 
 @dataclasses.dataclass
@@ -48,6 +50,8 @@ class Step:
     h_slots: np.ndarray                          # host copies, for parts that plan on the host
     h_starts: np.ndarray
     h_counts: np.ndarray
+    token_take: tuple[torch.Tensor, torch.Tensor] | None = None   # (take_slot [T], last_token [S+1]): tokens that the
+                                                 # previous step drew and left on the device replace token_ids there
 
     @property
     def query_start(self) -> torch.Tensor:

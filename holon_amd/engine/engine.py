@@ -37,6 +37,17 @@ CACHED_PREFIX_TOKENS = 1 << 22      # with a prefix cache the pools grow to this
 PROMPT_LOGPROB_PORTION = 256        # core/holon/core/executor.py:645-666 takes the prompt's logits in pieces as small
 
 
+@dataclasses.dataclass
+class _Launched:
+    """A step on the device: its rows, and where its results will be on the host once `done` has passed."""
+
+    rows: list
+    sync: bool = False                          # it read the host while it was launched: commit it at once
+    tokens: torch.Tensor | None = None          # [sampled rows] int32
+    logprobs: list[torch.Tensor] | None = None
+    done: "torch.cuda.Event | None" = None
+
+
 class Engine:
     def __init__(self, cfg: EngineConfig, kernels=None, *, random_config: dict | None = None, seed: int = 0) -> None:
         self.cfg = cfg
@@ -72,6 +83,10 @@ class Engine:
         self._live: dict[str, list[Seq]] = {}
         self._siblings: dict[Seq, list[Seq]] = {}         # n > 1: waiting until the first sequence's prompt is cached
         self._prompt_lp: dict[Seq, Logprobs] = {}         # sequences still gathering prompt log-probabilities
+        self._inflight: _Launched | None = None           # the step that runs while the next one is scheduled
+        self._token_bufs = [torch.empty(cfg.max_seqs, dtype=torch.int32, pin_memory=device.type == "cuda")
+                            for _ in range(2)]
+        self._turn = 0
         self.steps = 0
 
     def _on_admit(self, seq: Seq) -> None:
@@ -181,19 +196,12 @@ class Engine:
         return rid
 
     def has_work(self) -> bool:
-        return bool(self.sched.waiting or self.sched.running)
+        return bool(self.sched.waiting or self.sched.running or self._inflight is not None)
 
     def idle_for(self) -> float | None:
         """How long a serving loop may wait for new requests before its next `step`: 0 while a request can run, None
         (as long as it likes) when there is no work."""
         return 0.0 if self.has_work() else None
-
-    def drain(self) -> list[TokenDelta]:
-        """Nothing runs on the device after this returns. Every step is committed before `step` returns, so there is
-        never one in flight."""
-        if self.device.type == "cuda":
-            torch.cuda.synchronize(self.device)
-        return []
 
     def abort(self, rid: str, reason: str = "abort") -> list[TokenDelta]:
         """Finish every sequence of request `rid` now: one delta each, siblings that never started included."""
@@ -207,6 +215,8 @@ class Engine:
             self.sched.finish(seq, reason)
             self._prompt_lp.pop(seq, None)
             deltas.append(TokenDelta(rid, [], reason, index=seq.index))
+        if not (self.sched.waiting or self.sched.running):      # only dropped rows are in flight: nothing to wait for later
+            deltas += self.drain()
         return deltas
 
     def stats(self) -> dict[str, int]:
@@ -217,11 +227,14 @@ class Engine:
                 "prefix_tokens_saved": self.cache.tokens_saved,
                 "cached_pages": len(self.cache.prefix.entries) if self.cache.prefix is not None else 0}
 
-    def flush_prefix(self) -> None:
-        """Drop the cached prompt blocks (core/holon/core/engine.py:418-420)."""
+    def flush_prefix(self) -> list[TokenDelta]:
+        """Drop the cached prompt blocks (core/holon/core/engine.py:418-420); the step in flight is committed first."""
+        deltas = self.drain()
         self.cache.flush_prefix()
+        return deltas
 
     def close(self) -> None:
+        self.drain()
         self._live.clear()
 
     def generate(self, prompts: list[list[int]], params: SamplingParams | None = None) -> list[list[int]]:
@@ -237,16 +250,34 @@ class Engine:
                     out[d.rid].extend(d.token_ids)
                     if d.finish_reason:
                         pending.discard(d.rid)
+        if not (self.sched.waiting or self.sched.running):      # rows of requests that finished meanwhile: dropped
+            self.drain()
         return [out[r] for r in rids]
 
     # -- one step -------------------------------------------------------------------------------------------------
     @torch.no_grad()
     def step(self) -> list[TokenDelta]:
+        """Schedule and launch one step, then commit the one before it while this one runs (`overlap`), or this one at
+        once. The deltas are those of the step committed. core/holon/core/engine.py:494-524."""
+        deltas: list[TokenDelta] = []
         rows = self.sched.schedule()
+        if rows is None and self._inflight is not None:      # what is in flight may bring tokens or finish requests
+            deltas += self.drain()
+            rows = self.sched.schedule()
         if rows is None:
             if self.has_work():
                 raise RuntimeError("the scheduler made no progress with requests pending")
-            return []
+            return deltas
+        launched = self._launch(rows)
+        deltas += self.drain()
+        if self.cfg.overlap and not launched.sync:
+            self._inflight = launched
+        else:
+            deltas += self._commit(launched)
+        return deltas
+
+    def _launch(self, rows: list) -> "_Launched":
+        """Run the rows and draw their tokens, all on the device; nothing here waits for it."""
         step_rows, owed, places, at = [], [], [], 0
         for seq, n, m in rows:
             want = list(range(*self._prompt_places(seq, n))) if seq in self._prompt_lp else []
@@ -258,38 +289,85 @@ class Engine:
                 places.append(at)
                 want.append(n - 1)
                 at += 1
-            step_rows.append(StepRow(seq.slot, seq.num_computed, seq.tokens[seq.num_computed: seq.num_computed + n],
-                                     want))
+            if seq.pending:                          # its token is the one the step in flight draws: still on the device
+                step_rows.append(StepRow(seq.slot, seq.num_computed, [0], want, on_device=True))
+            else:
+                step_rows.append(StepRow(seq.slot, seq.num_computed,
+                                         seq.tokens[seq.num_computed: seq.num_computed + n], want))
         logits = self.runner.run(step_rows)
         self.steps += 1
-        for seq, lo, count, targets in owed:
+        out = _Launched(rows=rows, sync=bool(owed))
+        for seq, lo, count, targets in owed:         # (these read the host: such a step is committed at once)
             self._gather_prompt_logprobs(seq, logits[lo: lo + count], targets)
         if owed and places:
             logits = logits.index_select(0, torch.tensor(places, device=logits.device))
         sampled = [(seq, n) for seq, n, m in rows if m]
-        tokens: list[int] = []
         if sampled:
             slots = np.array([seq.slot for seq, _ in sampled], dtype=np.int64)
             positions = np.array([seq.num_computed + n for seq, n in sampled], dtype=np.int64)
             drawn = self.sampler.sample(logits, slots, positions)
+            if len(sampled) == len(rows) and not owed:
+                where = self.runner.last_slots[: len(rows)]
+            else:
+                where = torch.from_numpy(slots.astype(np.int32)).to(self.device, non_blocking=True)
+            self.kernels.store_tokens(self.runner.last_token, where, drawn)
             k = max((seq.params.logprobs if seq.params.logprobs is not None else -1) for seq, _ in sampled)
-            lps = [t.tolist() for t in self.kernels.logprobs(logits, drawn, k)] if k >= 0 else None
-            tokens = drawn.tolist()
-        deltas, at = [], 0
-        chains, page = self.cache.chain, self.cache.page_size
+            out.tokens = self._to_host(drawn)
+            if k >= 0:
+                out.logprobs = [self._to_host(t, fresh=True) for t in self.kernels.logprobs(logits, drawn, k)]
+        if self.device.type == "cuda":
+            out.done = torch.cuda.Event()
+            out.done.record()
         for seq, n, m in rows:
             seq.num_computed += n
-            chain = chains[seq.slot]                  # (the check `publish` starts with, without the call: per row, per step)
-            if chain is not None and min(seq.num_computed, len(seq.tokens)) // page > len(chain):
-                self.cache.publish(seq.slot, seq.tokens)
+            if m:
+                seq.pending += 1
+                if seq.status is not Status.RUNNING:
+                    self.sched.finished_prefill(seq)
+        return out
+
+    def _to_host(self, t: torch.Tensor, fresh: bool = False) -> torch.Tensor:
+        """A copy of `t` on its way to pinned host memory (valid once the step's event has passed). The drawn tokens
+        use two buffers in turn: at most one step is in flight while the next is launched."""
+        if self.device.type != "cuda":
+            return t
+        if fresh:
+            host = torch.empty(t.shape, dtype=t.dtype, pin_memory=True)
+        else:
+            self._turn ^= 1
+            host = self._token_bufs[self._turn][: t.shape[0]]
+        host.copy_(t, non_blocking=True)
+        return host
+
+    def drain(self) -> list[TokenDelta]:
+        """Commit the step in flight, if any: nothing runs on the device afterwards."""
+        prev, self._inflight = self._inflight, None
+        return self._commit(prev) if prev is not None else []
+
+    def _commit(self, step: "_Launched") -> list[TokenDelta]:
+        """The host's books once a step's tokens are on the host: tokens appended, requests finished, pages published,
+        deltas made. A row of a request that finished (or was aborted) after the row was launched is dropped."""
+        if step.done is not None:
+            step.done.synchronize()
+        tokens = step.tokens.tolist() if step.tokens is not None else []
+        lps = [t.tolist() for t in step.logprobs] if step.logprobs is not None else None
+        deltas, at = [], 0
+        chains, page = self.cache.chain, self.cache.page_size
+        for seq, n, m in step.rows:
+            if m:
+                at += 1
+            if seq.status is Status.FINISHED:
+                continue
+            if seq.slot >= 0:
+                chain = chains[seq.slot]              # (the check `publish` starts with, without the call: per row, per step)
+                if chain is not None and min(seq.num_computed, len(seq.tokens)) // page > len(chain):
+                    self.cache.publish(seq.slot, seq.tokens)
             if not m:
                 continue
-            token = tokens[at]
+            token = tokens[at - 1]
             want = seq.params.logprobs
-            lp = None if want is None else Logprobs([lps[0][at]], [lps[1][at][:want]], [lps[2][at][:want]])
-            at += 1
-            if seq.status is not Status.RUNNING:
-                self.sched.finished_prefill(seq)
+            lp = None if want is None else Logprobs([lps[0][at - 1]], [lps[1][at - 1][:want]], [lps[2][at - 1][:want]])
+            seq.pending -= 1
             seq.tokens.append(token)
             for sibling in reversed(self._siblings.pop(seq, [])):         # its prompt is cached now
                 self.sched.add(sibling, front=True)

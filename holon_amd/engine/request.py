@@ -25,6 +25,7 @@ class Seq:
     num_computed: int = 0                # tokens whose state is in the cache
     status: Status = Status.WAITING
     finish_reason: str | None = None
+    pending: int = 0                     # tokens drawn for it that have not reached the host yet
     index: int = 0                       # which of its request's `n` sequences
     portion_cap: int = 0                 # most prompt tokens one step runs of it (0: what the budget allows)
     share_prefix: bool = True            # False: every position is computed, whatever the cache holds

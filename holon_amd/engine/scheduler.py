@@ -12,6 +12,10 @@ goes to the front of the queue and later runs its prompt and the tokens it had g
 nothing below can make room, a running request preempts itself and a waiting one ends the step's admissions. The pool
 always holds one request of `max_model_len` tokens (checked when the engine starts), so the top-ranked request always
 fits once everything below it is preempted, and every step makes progress.
+
+A step may be scheduled while the one before it still runs (core/holon/core/sched.py:12-15, 98-104): a request whose
+last drawn token has not reached the host (`pending`) decodes from the copy of it on the device; it counts towards the
+request's length limits; a preempted request waits for it before its tokens are run again as a prompt.
 """
 from __future__ import annotations
 
@@ -56,6 +60,8 @@ class Scheduler:
     def _prefill(self, budget: int) -> list[Row]:
         rows: list[Row] = []
         for seq in list(self.waiting):
+            if seq.pending:                                     # preempted with a token on its way: not yet
+                continue
             if budget <= 0 or (seq.slot < 0 and not self._fit(seq, None)):
                 break                                           # first come first served: nobody skips ahead
             n = min(len(seq.tokens) - seq.num_computed, budget, seq.portion_cap or budget)
@@ -78,7 +84,7 @@ class Scheduler:
         return rows
 
     def at_limit(self, seq: Seq) -> bool:
-        n = len(seq.tokens)
+        n = len(seq.tokens) + seq.pending
         return n >= self.max_model_len or (seq.params.max_tokens is not None
                                            and n - seq.prompt_len >= seq.params.max_tokens)
 

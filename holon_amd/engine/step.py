@@ -44,13 +44,16 @@ class StepRunner:
         self.pinned = device.type == "cuda"
         self._stages: list[tuple[torch.Tensor, torch.cuda.Event] | None] = [None, None]
         self._turn = 0
+        # the token last drawn for each slot, for a row whose token has not reached the host when it is scheduled
+        self.last_token = torch.zeros(max_seqs + 1, dtype=torch.int32, device=device)
+        self.last_slots: torch.Tensor | None = None       # the last step's rows' slots on the device
         self.use_graphs = graphs and device.type == "cuda"
         self.graphs: dict[tuple[int, int], _Graph] = {}
         self.graph_replays = 0
 
     # -- inputs ---------------------------------------------------------------------------------------------------
-    def _arrays(self, slots: np.ndarray, starts: np.ndarray, counts: np.ndarray, tokens: np.ndarray
-                ) -> tuple[list[np.ndarray], dict]:
+    def _arrays(self, slots: np.ndarray, starts: np.ndarray, counts: np.ndarray, tokens: np.ndarray,
+                take: np.ndarray) -> tuple[list[np.ndarray], dict]:
         """The int32 arrays of a step, in a fixed order, and the host-side facts about them."""
         cache = self.cache
         total, n = int(counts.sum()), len(slots)
@@ -64,7 +67,7 @@ class StepRunner:
             decode = np.flatnonzero(counts == 1)
             chunk = np.flatnonzero(counts > 1)
         lens = starts + counts
-        arrays = [tokens, positions, token_row, slots, starts, lens, qstart, decode, chunk]
+        arrays = [tokens, positions, token_row, slots, starts, lens, qstart, decode, chunk, take]
         for g in cache.groups:
             page, off = cache.write_targets(g.gid, slots[token_row], positions)
             arrays += [page, off]
@@ -109,21 +112,22 @@ class StepRunner:
 
     def _step(self, dev: list[torch.Tensor], facts: dict, slots, starts, counts) -> Step:
         cache = self.cache
-        paged = {g.gid: PagedView(cache.page_size, g.table_dev, dev[9 + 2 * i], dev[10 + 2 * i])
+        paged = {g.gid: PagedView(cache.page_size, g.table_dev, dev[10 + 2 * i], dev[11 + 2 * i])
                  for i, g in enumerate(cache.groups)}
         attn = AttnRows(slots=dev[3], lens=dev[5], query_start=dev[6], decode_rows=dev[7], chunk_rows=dev[8],
                         n_decode=facts["n_decode"], n_chunk=facts["n_chunk"], max_decode_len=facts["max_decode_len"],
                         max_chunk_query=facts["max_chunk_query"], max_chunk_len=facts["max_chunk_len"])
         return Step(kernels=self.kernels, n_tokens=facts["total"], n_rows=facts["n_rows"], token_ids=dev[0],
                     positions=dev[1], token_row=dev[2], slots=dev[3], starts=dev[4], rows=attn, paged=paged,
-                    h_slots=slots, h_starts=starts, h_counts=counts)
+                    h_slots=slots, h_starts=starts, h_counts=counts, token_take=(dev[9], self.last_token))
 
-    def _check(self, rows: list[StepRow]) -> tuple[np.ndarray, np.ndarray, np.ndarray, np.ndarray, np.ndarray]:
+    def _check(self, rows: list[StepRow]
+               ) -> tuple[np.ndarray, np.ndarray, np.ndarray, np.ndarray, np.ndarray, np.ndarray]:
         if not rows:
             raise ValueError("a step needs at least one row")
         cache = self.cache
         computed, paged = cache.computed, bool(cache.groups)
-        slots, starts, counts, wanted, flat = [], [], [], [], []
+        slots, starts, counts, wanted, flat, take = [], [], [], [], [], []
         at = 0
         for b, r in enumerate(rows):
             n = len(r.tokens)
@@ -137,6 +141,12 @@ class StepRunner:
                 if not 0 <= w < n:
                     raise ValueError(f"row {b}: wanted place {w} is not among its {n} tokens")
                 wanted.append(at + w)
+            if r.on_device:
+                if n != 1:
+                    raise ValueError(f"row {b}: only a row of one token can take it from the device")
+                take.append(r.slot)
+            else:
+                take.extend([-1] * n) if n > 1 else take.append(-1)
             slots.append(r.slot)
             starts.append(r.start)
             counts.append(n)
@@ -150,14 +160,14 @@ class StepRunner:
         if tokens.min() < 0 or tokens.max() >= self.vocab:
             raise ValueError(f"token ids must lie in [0, {self.vocab})")
         return (np.array(slots, dtype=np.int64), np.array(starts, dtype=np.int64), np.array(counts, dtype=np.int64),
-                tokens, np.array(wanted, dtype=np.int64))
+                tokens, np.array(wanted, dtype=np.int64), np.array(take, dtype=np.int64))
 
     def prepare(self, rows: list[StepRow]) -> tuple[Step, np.ndarray]:
         """Device inputs of a step, and the flat indices of the tokens whose logits are wanted (in row order, then in
         the order of each row's `want`)."""
-        slots, starts, counts, tokens, wanted = self._check(rows)
+        slots, starts, counts, tokens, wanted, take = self._check(rows)
         self.cache.upload()
-        arrays, facts = self._arrays(slots, starts, counts, tokens)
+        arrays, facts = self._arrays(slots, starts, counts, tokens, take)
         return self._step(self._to_device(arrays), facts, slots, starts, counts), wanted
 
     # -- the step -------------------------------------------------------------------------------------------------
@@ -179,6 +189,7 @@ class StepRunner:
             logits = self._run_graphed(rows)
         else:
             step, wanted = self.prepare(rows)
+            self.last_slots = step.slots
             logits = self._forward(step, wanted)
         for r in rows:
             self.cache.advance(r.slot, r.start + len(r.tokens))
@@ -187,7 +198,7 @@ class StepRunner:
 
     # -- graphs ---------------------------------------------------------------------------------------------------
     def _run_graphed(self, rows: list[StepRow]) -> torch.Tensor:
-        slots, starts, counts, tokens, _ = self._check(rows)
+        slots, starts, counts, tokens, _, take = self._check(rows)
         n = len(rows)
         bucket = next(b for b in BUCKETS if b >= n)
         longest = int((starts + counts).max())
@@ -198,8 +209,9 @@ class StepRunner:
             starts = np.concatenate((starts, np.zeros(pad, dtype=np.int64)))
             counts = np.concatenate((counts, np.ones(pad, dtype=np.int64)))
             tokens = np.concatenate((tokens, np.zeros(pad, dtype=np.int64)))
+            take = np.concatenate((take, np.full(pad, -1, dtype=np.int64)))
         self.cache.upload()
-        arrays, facts = self._arrays(slots, starts, counts, tokens)
+        arrays, facts = self._arrays(slots, starts, counts, tokens, take)
         facts["max_decode_len"] = len_bucket       # launch shapes are the bucket's, whatever the rows' lengths
         key = (bucket, len_bucket)
         g = self.graphs.get(key)
@@ -211,6 +223,7 @@ class StepRunner:
         else:
             self._to_device(arrays, g.arena, views=False)
         g.runs += 1
+        self.last_slots = g.step.slots[:n]
         if g.graph is None and g.runs == 1:        # the first step of a bucket: eagerly, on the fixed buffers
             return self._forward(g.step, None)[:n]
         if g.graph is None:

@@ -43,8 +43,11 @@ class AttnRows:
 class Kernels(Protocol):
     name: str
 
-    def embedding(self, ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-        """ids [T] int32, table [V, H] -> [T, H] (rows of the table)."""
+    def embedding(self, ids: torch.Tensor, table: torch.Tensor,
+                  take: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
+        """ids [T] int32, table [V, H] -> [T, H] (rows of the table). `take` = (take_slot [T] int32, last_token [S]
+        int32): token t is last_token[take_slot[t]] where take_slot[t] >= 0 (a token the previous step drew and left
+        on the device), ids[t] otherwise."""
 
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
         """x [..., dim] contiguous -> a new tensor; x is not modified."""
@@ -96,6 +99,9 @@ class Kernels(Protocol):
 
     def argmax(self, logits: torch.Tensor) -> torch.Tensor:
         """logits [R, V] float32 -> [R] int32, the first maximal index of each row."""
+
+    def store_tokens(self, last_token: torch.Tensor, slots: torch.Tensor, tokens: torch.Tensor) -> None:
+        """last_token[slots[r]] = tokens[r] (all int32, slots distinct): drawn tokens kept on the device by slot."""
 
     def logprobs(self, logits: torch.Tensor, tokens: torch.Tensor, k: int
                  ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:

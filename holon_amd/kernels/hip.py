@@ -53,7 +53,7 @@ class HipKernels:
         lib = self.lib
         lib.holon_last_error.restype = ctypes.c_char_p
         sig = {
-            "holon_embedding": [_P, _P, _P, _I, _I, _I, _I, _P],
+            "holon_embedding": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
             "holon_rmsnorm": [_P, _P, _P, _P, _L, _I, _F, _I, _P],
             "holon_silu_mul": [_P, _P, _L, _I, _I, _P],
             "holon_qk_norm_rope_write": [_P, _L, _P, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _P, _P, _P, _P, _I, _I,
@@ -71,6 +71,7 @@ class HipKernels:
             "holon_gemm_skinny_add_bf16": [_P, _P, _P, _I, _I, _I, _P],
             "holon_gemm_skinny_glu_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
             "holon_argmax": [_P, _P, _I, _I, _P],
+            "holon_store_tokens": [_P, _P, _P, _I, _I, _P],
             "holon_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
             "holon_logprobs": [_P, _P, _I, _I, _I, _P, _P, _P, _P],
         }
@@ -103,12 +104,19 @@ class HipKernels:
         return _DT[t.dtype]
 
     # -- ops ------------------------------------------------------------------------------------------------------
-    def embedding(self, ids, table):
+    def embedding(self, ids, table, take=None):
         self._check(ids, "embedding ids", torch.int32)
         self._check(table, "embedding table")
+        take_slot, last_token = take if take is not None else (None, None)
+        if take is not None:
+            self._check(take_slot, "embedding take_slot", torch.int32)
+            self._check(last_token, "embedding last_token", torch.int32)
+            if take_slot.shape != ids.shape:
+                raise KernelError(f"embedding: {tuple(take_slot.shape)} slots to take from for {tuple(ids.shape)} tokens")
         out = torch.empty((ids.shape[0], table.shape[1]), dtype=table.dtype, device=table.device)
-        self._call(self.lib.holon_embedding, ids.data_ptr(), table.data_ptr(), out.data_ptr(), ids.shape[0],
-                   table.shape[1], table.shape[0], self._dt(table, "embedding"), self._stream())
+        self._call(self.lib.holon_embedding, ids.data_ptr(), _ptr(take_slot), _ptr(last_token), table.data_ptr(),
+                   out.data_ptr(), ids.shape[0], table.shape[1], table.shape[0], self._dt(table, "embedding"),
+                   self._stream())
         return out
 
     def rmsnorm(self, x, weight, eps):
@@ -296,6 +304,14 @@ class HipKernels:
         self._call(self.lib.holon_argmax, logits.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1],
                    self._stream())
         return out
+
+    def store_tokens(self, last_token, slots, tokens):
+        for t, what in ((last_token, "last_token"), (slots, "slots"), (tokens, "tokens")):
+            self._check(t, f"store_tokens {what}", torch.int32)
+        if slots.shape != tokens.shape:
+            raise KernelError(f"store_tokens: {tuple(slots.shape)} slots for {tuple(tokens.shape)} tokens")
+        self._call(self.lib.holon_store_tokens, last_token.data_ptr(), slots.data_ptr(), tokens.data_ptr(),
+                   tokens.shape[0], last_token.shape[0], self._stream())
 
     def logprobs(self, logits, tokens, k):
         self._check(logits, "logprobs logits", torch.float32)

@@ -53,7 +53,7 @@ class Model(Part):
 
     def trunk(self, step) -> tuple[torch.Tensor, torch.Tensor | None]:
         """The residual stream after every run, as (h, delta) with h + delta the stream [T, hidden]."""
-        h, delta = self.embed(step.token_ids), None
+        h, delta = self.embed(step.token_ids, step.token_take), None
         for site in self.sites:
             h, delta = self.blocks[site.layer](h, delta, step, site)
         return h, delta

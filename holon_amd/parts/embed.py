@@ -13,8 +13,9 @@ class Embedding(Part):
         super().__init__(build)
         self.declare("weight", (vocab, hidden))
 
-    def forward(self, ids: torch.Tensor) -> torch.Tensor:
-        return self.kernels.embedding(ids, self.weight)
+    def forward(self, ids: torch.Tensor, take: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
+        """Rows of the table; `take`: where a token is still on the device, see the kernel contract."""
+        return self.kernels.embedding(ids, self.weight, take)
 
     __call__ = forward
 

@@ -42,7 +42,10 @@ def _mix32(x):
 class TorchKernels:
     name = "torch-plain"
 
-    def embedding(self, ids, table):
+    def embedding(self, ids, table, take=None):
+        if take is not None:
+            take_slot, last_token = take
+            ids = torch.where(take_slot >= 0, last_token[take_slot.clamp(min=0).long()], ids)
         return table[ids.long()]
 
     def rmsnorm(self, x, weight, eps):
@@ -119,6 +122,9 @@ class TorchKernels:
 
     def argmax(self, logits):
         return logits.argmax(-1).to(torch.int32)
+
+    def store_tokens(self, last_token, slots, tokens):
+        last_token[slots.long()] = tokens
 
     def logprobs(self, logits, tokens, k):
         lp = (logits if logits.dtype == torch.float64 else logits.float()).log_softmax(-1)

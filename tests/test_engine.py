@@ -155,7 +155,8 @@ def test_random_traffic_generates_what_the_plain_model_generates(folders, seed):
     mixed = rng.choice([0, 6])
     engine = _engine(folders["Bu"], "cpu", page_size=page, max_seqs=rng.choice([2, 3, 5]), max_model_len=max_len,
                      max_step_tokens=rng.choice([16, 24]), chunk_with_decode=mixed,
-                     cache_tokens=rng.choice([64, 96, 160]), prefix_cache=rng.random() < 0.8)
+                     cache_tokens=rng.choice([64, 96, 160]), prefix_cache=rng.random() < 0.8,
+                     overlap=rng.random() < 0.7)
     starts = [H.random_ids(40, 384, 1000 * seed + i) for i in range(2)]
     todo = []
     for i in range(10):
@@ -190,6 +191,39 @@ def test_random_traffic_generates_what_the_plain_model_generates(folders, seed):
         engine.cache.check()
     assert done == set(want) and got == want
     assert _released(engine)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_a_step_in_flight_changes_no_token(folders, device):
+    """With `overlap` a step is scheduled and launched before the one before it has been committed: a decode row
+    takes its token from the device, a request that ends on an end-of-sequence token has one more row in flight (it
+    is dropped), a preempted request waits for its token. The tokens are those of the engine that commits every step
+    at once, and the plain model's."""
+    plain = PlainQwen3(folders["Bu"])
+    prompts = [H.random_ids(n, 384, 300 + n) for n in (3, 17, 8, 25, 12)]
+    free = [plain.greedy(p, 12) for p in prompts]
+    stops = tuple({f[5] for f in free})                       # every request stops on some token another one draws too
+    params = SamplingParams(temperature=0.0, max_tokens=12, stop_token_ids=stops)
+    want = []
+    for f in free:
+        cut = min(i for i, t in enumerate(f) if t in stops)
+        want.append(f[: cut + 1])
+    assert any(len(w) < 6 for w in want) or all(len(w) == 6 for w in want)
+    shape = dict(page_size=4, max_seqs=3, max_step_tokens=10, max_model_len=40, cache_tokens=48)
+    outs = {}
+    for overlap in (True, False):
+        engine = _engine(folders["Bu"], device, overlap=overlap, **shape)
+        outs[overlap] = engine.generate(prompts, params)
+        assert outs[overlap] == want, overlap
+        assert _released(engine) and not engine.has_work()
+        stats = engine.stats()
+    lagging = _engine(folders["Bu"], device, overlap=True, **shape)
+    rid = lagging.add(prompts[1], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))
+    seen = []
+    while lagging.has_work():
+        seen.append([d.token_ids for d in lagging.step()])
+    assert seen[0] == [] and sum(len(s) for s in seen) == 4     # the first step's token comes with the second step
+    assert [t for s in seen for ts in s for t in ts] == plain.greedy(prompts[1], 4)
 
 
 @pytest.mark.parametrize("device", DEVICES)
