@@ -135,23 +135,12 @@ __device__ __forceinline__ float key_float(uint32_t k) {
 // Filters in order (the reference's): top-k keeps the k largest (ties: lower index first); top-p keeps, in descending
 // order, tokens whose preceding mass is <= top_p of the top-k mass (the largest always stays); min-p keeps q >= min_p
 // times the largest q. A token is identified for ties by (value, index), so the kept set is exact.
-__global__ void sample_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, int vocab,
-                              const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
-                              const float* __restrict__ top_p, const float* __restrict__ min_p,
-                              const int64_t* __restrict__ seeds, const int64_t* __restrict__ positions) {
-  const int r = blockIdx.x;
-  const float* row = logits + (int64_t)r * vocab;
-  const float temp = temperature[r];
-  if (temp == 0.f) {
-    const ArgMax a = block_argmax(row, vocab, 1.0f);
-    if (threadIdx.x == 0) out[r] = a.i;
-    return;
-  }
-  const float inv_temp = 1.0f / temp;
-  const ArgMax top = block_argmax(row, vocab, inv_temp);
+// The general form: any k, any kept set. Bisection on the ordered keys, one pass over the row per step, every thread
+// a contiguous segment of the row (so that ranks among equal values follow the index): exact but slow, for the rows
+// whose kept set does not fit the fast form below.
+__device__ void sample_row_general(const float* __restrict__ row, int32_t* __restrict__ out_r, int vocab, float inv_temp,
+                                   ArgMax top, int k, float p_keep, float p_min, float u) {
   const float xmax = top.v;
-  const int k = top_k[r];
-  const float p_keep = top_p[r], p_min = min_p[r];
 
   // --- top-k: the k-th largest key, and how many of the tokens equal to it are kept (the first ones by index)
   uint32_t kth_key = 0;          // keep x with key > kth_key, plus the first `ties_kept` tokens with key == kth_key
@@ -286,7 +275,7 @@ __global__ void sample_kernel(const float* __restrict__ logits, int32_t* __restr
   }
   __syncthreads();
   const float before = scan_f[threadIdx.x];
-  const float target = hashed_uniform((uint64_t)seeds[r], (uint64_t)positions[r]) * total_s;
+  const float target = u * total_s;
   __shared__ int chosen;
   if (threadIdx.x == 0) chosen = -1;
   __syncthreads();
@@ -307,7 +296,403 @@ __global__ void sample_kernel(const float* __restrict__ logits, int32_t* __restr
     atomicMax(&chosen, pick >= 0 ? pick : last);
   }
   __syncthreads();
-  if (threadIdx.x == 0) out[r] = chosen >= 0 ? chosen : top.i;
+  if (threadIdx.x == 0) *out_r = chosen >= 0 ? chosen : top.i;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The fast form. Masses are integers, Q = trunc(exp(x - max) * (2^32 - 256)): sums of them are exact in any order, so
+// every decision below is the same whatever the threads' order, and a sum over a part of the row is exact too.
+//   1. the largest value;
+//   2. (a filter is set) how many tokens lie in each of 16 bands below the largest value (within 1, 2, ... 8, 12, 16,
+//      ... 128), and for top-p without top-k the row's mass; the fewest bands that are sure to hold the kept set are
+//      collected into LDS (at most SAMPLE_CANDIDATES tokens) and sorted by (value descending, index ascending): the
+//      order in which top-k and top-p take tokens. If no such set fits, the row takes the general form;
+//   3. top-k keeps the first k of the sorted set; top-p those whose preceding mass is <= top_p * (mass of what top-k
+//      kept); both keep a prefix, so the kept set is "(value, index) at or before the last kept one": one compare;
+//   4. min-p drops q < min_p (the largest q is 1); the draw is the inverse CDF in vocabulary order over the integer
+//      masses: sums of 256 consecutive tokens, the 256 that hold the target found among those sums, one scan of them.
+#define SAMPLE_CANDIDATES 4096
+#define SAMPLE_WAVES (SAMPLE_THREADS / WAVE)
+#define SAMPLE_PER (SAMPLE_CANDIDATES / SAMPLE_THREADS)
+#define SAMPLE_BANDS 16
+#define SAMPLE_CHUNK 256
+typedef unsigned long long u64;
+
+// The band of a token d = max - x below the largest value: 0..7 for d in [0, 8) by ones, then [8, 12), [12, 16),
+// [16, 24), [24, 32), [32, 48), [48, 64), [64, 96), [96, 128); SAMPLE_BANDS beyond (or for a NaN).
+__device__ __forceinline__ int near_band(float d) {
+  if (!(d < 128.f)) return SAMPLE_BANDS;
+  const int di = (int)d;
+  if (di < 8) return di;
+  const int e = 31 - __clz(di);                 // 3 .. 6
+  return 8 + 2 * (e - 3) + ((di >> (e - 1)) & 1);
+}
+__device__ __forceinline__ float band_edge(int band) {   // tokens beyond bands 0 .. band are at least this far below
+  const float edges[SAMPLE_BANDS] = {1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 24, 32, 48, 64, 96, 128};
+  return edges[band];
+}
+
+__device__ __forceinline__ uint32_t fixed_mass(float q) { return (uint32_t)(q * 4294967040.0f); }   // q in [0, 1]
+__device__ __forceinline__ u64 order_key(float x, int i) {   // larger = taken earlier
+  return ((u64)float_key(x) << 32) | (uint32_t)(0x7fffffff - i);
+}
+
+__device__ __forceinline__ u64 shfl_u64(u64 v, int src) {
+  return ((u64)__shfl((uint32_t)(v >> 32), src, WAVE) << 32) | __shfl((uint32_t)v, src, WAVE);
+}
+__device__ __forceinline__ u64 wave_sum_u64(u64 v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) {
+    const uint32_t lo = __shfl_xor((uint32_t)v, o, WAVE), hi = __shfl_xor((uint32_t)(v >> 32), o, WAVE);
+    v += ((u64)hi << 32) | lo;
+  }
+  return v;
+}
+__device__ __forceinline__ u64 wave_scan_u64(u64 v, int lane) {   // inclusive, over the lanes in order
+#pragma unroll
+  for (int o = 1; o < WAVE; o <<= 1) {
+    const uint32_t lo = __shfl_up((uint32_t)v, o, WAVE), hi = __shfl_up((uint32_t)(v >> 32), o, WAVE);
+    if (lane >= o) v += ((u64)hi << 32) | lo;
+  }
+  return v;
+}
+__device__ u64 block_sum_u64(u64 v) {
+  __shared__ u64 part[SAMPLE_WAVES];
+  __shared__ u64 result;
+  v = wave_sum_u64(v);
+  __syncthreads();
+  if (threadIdx.x % WAVE == 0) part[threadIdx.x / WAVE] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    u64 r = 0;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) r += part[w];
+    result = r;
+  }
+  __syncthreads();
+  return result;
+}
+// The sum of `v` over the threads before this one (thread order), and the whole sum.
+__device__ u64 block_scan_u64(u64 v, u64& total) {
+  __shared__ u64 part[SAMPLE_WAVES];
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const u64 incl = wave_scan_u64(v, lane);
+  __syncthreads();
+  if (lane == WAVE - 1) part[wave] = incl;
+  __syncthreads();
+  u64 before = 0, all = 0;
+  for (int w = 0; w < SAMPLE_WAVES; ++w) {
+    if (w < wave) before += part[w];
+    all += part[w];
+  }
+  total = all;
+  return before + incl - v;
+}
+
+// f(x, i) for every token of the row, x = logit * inv_temp, in no particular order: 16-byte loads where the row allows.
+template <typename F>
+__device__ __forceinline__ void for_each_token(const float* __restrict__ row, int vocab, float inv_temp, F f) {
+  if ((vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    const float4* row4 = reinterpret_cast<const float4*>(row);
+    for (int i = threadIdx.x; i < vocab / 4; i += blockDim.x) {
+      const float4 v = row4[i];
+      f(v.x * inv_temp, 4 * i); f(v.y * inv_temp, 4 * i + 1); f(v.z * inv_temp, 4 * i + 2); f(v.w * inv_temp, 4 * i + 3);
+    }
+  } else {
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) f(row[i] * inv_temp, i);
+  }
+}
+
+// About how many tokens lie in bands 0 .. j below the largest value, for every j, into counts[] (shared): every eighth
+// stretch of the row is counted (a token's place in the vocabulary says nothing about its value), a thread counting in
+// 8-bit fields of two registers.
+__device__ void estimate_band_counts(const float* __restrict__ row, int vocab, float inv_temp, float xmax, int* counts,
+                                     int (*band_counts)[SAMPLE_BANDS]) {
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  u64 near_lo = 0, near_hi = 0;                  // bands 0..7 and 8..15
+  const int stretch = 4 * SAMPLE_THREADS;        // tokens a pass of the block covers
+  for (int base = 0; base < vocab; base += 8 * stretch) {
+    const int i0 = base + 4 * tid;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (i0 + e < vocab) {
+        const int band = near_band(xmax - row[i0 + e] * inv_temp);
+        if (band < 8) near_lo += 1ull << (8 * band); else if (band < SAMPLE_BANDS) near_hi += 1ull << (8 * (band - 8));
+      }
+    }
+  }
+  // the fields widened to 16 bits (a wave's sum fits), added over the wave, then over the waves
+  u64 wide[4];
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const uint32_t four = (uint32_t)((h < 2 ? near_lo : near_hi) >> (32 * (h & 1)));
+    wide[h] = wave_sum_u64((u64)(four & 0xff) | ((u64)((four >> 8) & 0xff) << 16) | ((u64)((four >> 16) & 0xff) << 32) |
+                           ((u64)(four >> 24) << 48));
+  }
+  __syncthreads();
+  if (lane == 0) {
+#pragma unroll
+    for (int j = 0; j < SAMPLE_BANDS; ++j) band_counts[wave][j] = (int)((wide[j / 4] >> (16 * (j % 4))) & 0xffff);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int j = 0; j < SAMPLE_BANDS; ++j) {
+      for (int w = 0; w < SAMPLE_WAVES; ++w) run += band_counts[w][j];
+      counts[j] = 8 * run;
+    }
+  }
+  __syncthreads();
+}
+
+// The tokens of bands 0 .. `bands` into cand[] as order keys, in no order; returns how many there are (the same in
+// every thread), of which only the first SAMPLE_CANDIDATES were stored.
+__device__ int collect_bands(const float* __restrict__ row, int vocab, float inv_temp, float xmax, int bands, u64* cand,
+                             int* n_cand) {
+  if (threadIdx.x == 0) *n_cand = 0;
+  __syncthreads();
+  const float edge = band_edge(bands);
+  for_each_token(row, vocab, inv_temp, [&](float x, int i) {
+    if (xmax - x < edge) {
+      const int at = atomicAdd(n_cand, 1);
+      if (at < SAMPLE_CANDIDATES) cand[at] = order_key(x, i);
+    }
+  });
+  __syncthreads();
+  const int count = *n_cand;
+  __syncthreads();
+  return count;
+}
+
+// Bitonic sort of a[0 .. n_pad) in LDS by the whole block; n_pad is a power of two.
+__device__ void bitonic_sort(u64* a, int n_pad, bool descending) {
+  for (int size = 2; size <= n_pad; size <<= 1) {
+    for (int stride = size / 2; stride > 0; stride >>= 1) {
+      for (int i = threadIdx.x; i < n_pad; i += blockDim.x) {
+        const int partner = i ^ stride;
+        if (partner > i) {
+          const u64 x = a[i], y = a[partner];
+          const bool down = ((i & size) == 0) == descending;
+          if (down ? x < y : x > y) { a[i] = y; a[partner] = x; }
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+__global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
+    const float* __restrict__ logits, int32_t* __restrict__ out, int vocab, const float* __restrict__ temperature,
+    const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
+    const int64_t* __restrict__ seeds, const int64_t* __restrict__ positions) {
+  __shared__ u64 cand[SAMPLE_CANDIDATES];      // order keys of the collected tokens, sorted; later the sums of 256 tokens
+  __shared__ int counts[SAMPLE_BANDS];
+  __shared__ int band_counts[SAMPLE_WAVES][SAMPLE_BANDS];
+  __shared__ int n_cand, n_keep_s, pick_s;
+  __shared__ u64 z_k_s;
+  const int r = blockIdx.x, tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  const float* row = logits + (int64_t)r * vocab;
+  const float temp = temperature[r];
+  if (temp == 0.f) {
+    const ArgMax a = block_argmax(row, vocab, 1.0f);
+    if (tid == 0) out[r] = a.i;
+    return;
+  }
+  const float inv_temp = 1.0f / temp;
+  const ArgMax top = block_argmax(row, vocab, inv_temp);
+  const float xmax = top.v;
+  const int k = top_k[r];
+  const float p_keep = top_p[r], p_min = min_p[r];
+  const float u = hashed_uniform((uint64_t)seeds[r], (uint64_t)positions[r]);
+  const bool k_on = k > 0 && k < vocab, p_on = p_keep < 1.0f;
+  const int chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+  if ((k_on && k > SAMPLE_CANDIDATES) || vocab > 255 * SAMPLE_THREADS) {      // (uniform over the block)
+    sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
+    return;
+  }
+
+  if (k_on || p_on) {
+    u64 z_all = 0;
+    if (p_on && !k_on) {                         // top-p without top-k: the mass of the whole row
+      u64 mass = 0;
+      for_each_token(row, vocab, inv_temp, [&](float x, int) { mass += fixed_mass(__expf(x - xmax)); });
+      z_all = block_sum_u64(mass);
+    }
+    estimate_band_counts(row, vocab, inv_temp, xmax, counts, band_counts);
+    // Which bands to collect: the fewest that should hold twice what is needed (k tokens; 256 for top-p alone). The
+    // collecting counts exactly; too many, or fewer than k, and another set of bands is tried.
+    const int need = k_on ? k : 1;
+    int bands = SAMPLE_BANDS - 1;
+    for (int j = SAMPLE_BANDS - 1; j >= 0; --j)
+      if (counts[j] >= 2 * (k_on ? k : 256) + 64) bands = j;
+    while (bands > 0 && counts[bands] > SAMPLE_CANDIDATES / 2 && counts[bands - 1] >= 2 * need) --bands;
+    int count = 0;
+    for (int attempt = 0;; ++attempt) {
+      if (attempt == 6 || bands < 0 || bands >= SAMPLE_BANDS) {
+        sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
+        return;
+      }
+      count = collect_bands(row, vocab, inv_temp, xmax, bands, cand, &n_cand);
+      if (count > SAMPLE_CANDIDATES) { --bands; continue; }
+      if (count < need && count < vocab) { ++bands; continue; }
+      int n_pad = WAVE;
+      while (n_pad < count) n_pad <<= 1;
+      for (int i = count + tid; i < n_pad; i += blockDim.x) cand[i] = 0;   // after every real key
+      __syncthreads();
+      bitonic_sort(cand, n_pad, true);
+      // masses in sorted order: a thread holds consecutive ones and the sum of everything before them
+      const int per = max(1, n_pad / SAMPLE_THREADS);     // 1, 2 or 4
+      u64 incl[SAMPLE_PER];
+      u64 run = 0;
+#pragma unroll
+      for (int e = 0; e < SAMPLE_PER; ++e) {
+        const int i = tid * per + e;
+        if (e < per && i < count) run += fixed_mass(__expf(key_float((uint32_t)(cand[i] >> 32)) - xmax));
+        incl[e] = run;
+      }
+      u64 cand_mass;
+      const u64 before = block_scan_u64(run, cand_mass);
+      const int k_eff = k_on ? min(k, count) : count;
+      if (tid == 0) n_keep_s = k_eff;
+#pragma unroll
+      for (int e = 0; e < SAMPLE_PER; ++e)
+        if (e < per && tid * per + e == k_eff - 1) z_k_s = before + incl[e];
+      __syncthreads();
+      if (p_on) {
+        const u64 z_k = k_on ? z_k_s : z_all;
+        const u64 bound = (u64)((double)p_keep * (double)z_k);
+        // the kept ones are those whose preceding mass is within the bound: a prefix, as the sums only grow
+        int mine = 0;
+#pragma unroll
+        for (int e = 0; e < SAMPLE_PER; ++e) {
+          const int i = tid * per + e;
+          if (e < per && i < k_eff) mine += (before + (e ? incl[e - 1] : 0)) <= bound;
+        }
+        const int kept = block_sum_int(mine);
+        if (tid == 0) n_keep_s = kept;
+        __syncthreads();
+      }
+      // top-p alone, and everything collected was kept: the bound may lie past it, in bands not collected
+      if (p_on && !k_on && count < vocab && n_keep_s == count) {
+        __syncthreads();
+        ++bands;
+        while (bands < SAMPLE_BANDS - 1 && counts[bands] < 4 * count) ++bands;   // a good deal more at once
+        continue;
+      }
+      break;
+    }
+    // min-p drops q < min_p: the values only fall along the sorted order, so this keeps a prefix too
+    int ok = 0;
+    for (int i = tid; i < n_keep_s; i += blockDim.x) ok += __expf(key_float((uint32_t)(cand[i] >> 32)) - xmax) >= p_min;
+    const int n_final = max(1, block_sum_int(ok));
+    // the kept tokens in vocabulary order, their masses, and the first whose running mass exceeds the target
+    int n_pad = WAVE;
+    while (n_pad < n_final) n_pad <<= 1;
+    for (int i = tid; i < n_pad; i += blockDim.x) {
+      const u64 c = cand[i];
+      cand[i] = i < n_final ? ((u64)(0x7fffffffu - (uint32_t)c) << 32) | (c >> 32) : ~0ull;   // (index, value key)
+    }
+    __syncthreads();
+    bitonic_sort(cand, n_pad, false);
+    const int per = max(1, n_pad / SAMPLE_THREADS);
+    uint32_t m[SAMPLE_PER];
+    u64 mine = 0;
+#pragma unroll
+    for (int e = 0; e < SAMPLE_PER; ++e) {
+      const int i = tid * per + e;
+      m[e] = (e < per && i < n_final) ? fixed_mass(__expf(key_float((uint32_t)cand[i]) - xmax)) : 0u;
+      mine += m[e];
+    }
+    u64 total;
+    const u64 before = block_scan_u64(mine, total);
+    const u64 target = (u64)((double)u * (double)total);
+    if (tid == 0) pick_s = -1;
+    __syncthreads();
+    if (mine > 0 && before <= target && target < before + mine) {   // (one thread)
+      u64 run = before;
+      int pick = -1;
+#pragma unroll
+      for (int e = 0; e < SAMPLE_PER; ++e) {
+        run += m[e];
+        if (pick < 0 && m[e] > 0 && run > target) pick = (int)(cand[tid * per + e] >> 32);
+      }
+      pick_s = pick;
+    }
+    __syncthreads();
+    if (tid == 0) out[r] = pick_s >= 0 ? pick_s : top.i;
+    return;
+  }
+
+  const u64 cut = 0;                            // no top-k, no top-p: every token passes them
+  // the law, and the draw in vocabulary order
+  auto law = [&](float x, int i) -> uint32_t {
+    const float q = __expf(x - xmax);
+    return (order_key(x, i) >= cut && q >= p_min) ? fixed_mass(q) : 0u;
+  };
+  u64* chunk_mass = cand;                       // [chunks]: the mass of tokens 256 c .. 256 c + 255, four to a lane
+  const bool wide = (vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+  auto lane_masses = [&](int c, uint32_t (&m)[4]) {
+    const int i0 = c * SAMPLE_CHUNK + 4 * lane;
+    float x[4];
+    if (wide && i0 + 3 < vocab) {
+      const float4 v = *reinterpret_cast<const float4*>(row + i0);
+      x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[e] = i0 + e < vocab ? row[i0 + e] : -INFINITY;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) m[e] = i0 + e < vocab ? law(x[e] * inv_temp, i0 + e) : 0u;
+  };
+  for (int c = wave; c < chunks; c += SAMPLE_WAVES) {
+    uint32_t m[4];
+    lane_masses(c, m);
+    const u64 sum = wave_sum_u64((u64)m[0] + m[1] + m[2] + m[3]);
+    if (lane == 0) chunk_mass[c] = sum;
+  }
+  if (tid == 0) pick_s = -1;
+  __syncthreads();
+  // a thread holds consecutive chunks; the one whose chunks hold the target names the chunk
+  const int cper = (chunks + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  u64 mine = 0;
+  for (int e = 0; e < cper; ++e) {
+    const int c = tid * cper + e;
+    if (c < chunks) mine += chunk_mass[c];
+  }
+  u64 total;
+  const u64 before = block_scan_u64(mine, total);
+  const u64 target = (u64)((double)u * (double)total);     // the first token whose running mass exceeds it
+  __shared__ int chunk_s;
+  __shared__ u64 chunk_before_s;
+  if (mine > 0 && before <= target && target < before + mine) {   // (one thread)
+    u64 run = before;
+    for (int e = 0; e < cper; ++e) {
+      const int c = tid * cper + e;
+      const u64 m = c < chunks ? chunk_mass[c] : 0;
+      if (run + m > target) { chunk_s = c; chunk_before_s = run; break; }
+      run += m;
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    uint32_t m[4];
+    lane_masses(chunk_s, m);
+    const u64 mine4 = (u64)m[0] + m[1] + m[2] + m[3];
+    u64 run = chunk_before_s + wave_scan_u64(mine4, lane) - mine4;   // the mass before this lane's four tokens
+    int pick = -1;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      run += m[e];
+      if (pick < 0 && run > target) pick = chunk_s * SAMPLE_CHUNK + 4 * lane + e;
+    }
+    const u64 hit = __ballot(pick >= 0);
+    if (hit) {
+      const int first = __ffsll((long long)hit) - 1;
+      pick = __shfl(pick, first, WAVE);
+      if (lane == 0) pick_s = pick;
+    }
+  }
+  __syncthreads();
+  if (tid == 0) out[r] = pick_s >= 0 ? pick_s : top.i;
 }
 
 extern "C" int holon_sample(const float* logits, int32_t* out, int rows, int vocab, const float* temperature,
@@ -322,42 +707,72 @@ extern "C" int holon_sample(const float* logits, int32_t* out, int rows, int voc
 }
 
 // Log-probabilities of the raw logits (before temperature): for each row the log-probability of `token[r]` and the
-// `k` largest log-probabilities with their ids (ties: lower id first). One block per row; k passes of argmax over
-// the row with the tokens already taken masked out.
+// `k` largest log-probabilities with their ids (ties: lower id first). One block per row: the largest value, the
+// log of the sum, then the tokens nearest the largest value collected and sorted as for sampling; if no band holds
+// k tokens within the room there is, k passes of argmax over the row instead.
 #define LOGPROB_MAX_K 32
-__global__ void logprobs_kernel(const float* __restrict__ logits, const int32_t* __restrict__ tokens, int vocab, int k,
-                                float* __restrict__ token_lp, int32_t* __restrict__ top_ids,
-                                float* __restrict__ top_lp) {
-  const int r = blockIdx.x;
+__global__ void __launch_bounds__(SAMPLE_THREADS) logprobs_kernel(
+    const float* __restrict__ logits, const int32_t* __restrict__ tokens, int vocab, int k,
+    float* __restrict__ token_lp, int32_t* __restrict__ top_ids, float* __restrict__ top_lp) {
+  __shared__ u64 cand[SAMPLE_CANDIDATES];
+  __shared__ int counts[SAMPLE_BANDS];
+  __shared__ int band_counts[SAMPLE_WAVES][SAMPLE_BANDS];
+  __shared__ int n_cand;
+  const int r = blockIdx.x, tid = threadIdx.x;
   const float* row = logits + (int64_t)r * vocab;
   const ArgMax top = block_argmax(row, vocab, 1.0f);
   float part = 0.f;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) part += expf(row[i] - top.v);
+  for_each_token(row, vocab, 1.0f, [&](float x, int) { part += expf(x - top.v); });
   const float lse = top.v + logf(block_sum(part));
-  if (threadIdx.x == 0) token_lp[r] = row[tokens[r]] - lse;
-  __shared__ int taken[LOGPROB_MAX_K];
-  __shared__ ArgMax part_best[SAMPLE_THREADS / WAVE];
+  if (tid == 0) token_lp[r] = row[tokens[r]] - lse;
+  if (k == 0) return;
+  if (vocab <= 255 * SAMPLE_THREADS) {
+    estimate_band_counts(row, vocab, 1.0f, top.v, counts, band_counts);
+    int bands = SAMPLE_BANDS - 1;
+    for (int j = SAMPLE_BANDS - 1; j >= 0; --j)
+      if (counts[j] >= 2 * k + 64) bands = j;
+    for (int attempt = 0; attempt < 6 && bands >= 0 && bands < SAMPLE_BANDS; ++attempt) {
+      const int count = collect_bands(row, vocab, 1.0f, top.v, bands, cand, &n_cand);
+      if (count > SAMPLE_CANDIDATES) { --bands; continue; }
+      if (count < k && count < vocab) { ++bands; continue; }
+      int n_pad = WAVE;
+      while (n_pad < count) n_pad <<= 1;
+      for (int i = count + tid; i < n_pad; i += blockDim.x) cand[i] = 0;
+      __syncthreads();
+      bitonic_sort(cand, n_pad, true);
+      if (tid < k) {
+        const u64 c = cand[tid];
+        top_ids[(int64_t)r * k + tid] = (int)(0x7fffffffu - (uint32_t)c);
+        top_lp[(int64_t)r * k + tid] = key_float((uint32_t)(c >> 32)) - lse;
+      }
+      return;
+    }
+  }
+  // the k largest one after the other: each pass takes the first in order after the one before
+  __shared__ ArgMax part_best[SAMPLE_WAVES];
+  __shared__ u64 last_s;
+  u64 last = ~0ull;
   for (int j = 0; j < k; ++j) {
     ArgMax best{-INFINITY, 0x7fffffff};
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-      bool skip = false;
-      for (int t = 0; t < j; ++t) skip = skip || taken[t] == i;
-      if (!skip) best = better(best, ArgMax{row[i], i});
-    }
+    for_each_token(row, vocab, 1.0f, [&](float x, int i) {
+      if (order_key(x, i) < last) best = better(best, ArgMax{x, i});
+    });
 #pragma unroll
     for (int o = WAVE / 2; o > 0; o >>= 1) {
       ArgMax other{__shfl_xor(best.v, o, WAVE), __shfl_xor(best.i, o, WAVE)};
       best = better(best, other);
     }
-    if (threadIdx.x % WAVE == 0) part_best[threadIdx.x / WAVE] = best;
+    if (tid % WAVE == 0) part_best[tid / WAVE] = best;
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (tid == 0) {
       ArgMax b = part_best[0];
-      for (int w = 1; w < (int)blockDim.x / WAVE; ++w) b = better(b, part_best[w]);
-      taken[j] = b.i;
+      for (int w = 1; w < SAMPLE_WAVES; ++w) b = better(b, part_best[w]);
       top_ids[(int64_t)r * k + j] = b.i == 0x7fffffff ? 0 : b.i;
       top_lp[(int64_t)r * k + j] = b.v - lse;
+      last_s = b.i == 0x7fffffff ? 0 : order_key(b.v, b.i);
     }
+    __syncthreads();
+    last = last_s;
     __syncthreads();
   }
 }
