@@ -1,6 +1,8 @@
 // Sampling on the device: argmax, and temperature / top-k / top-p / min-p sampling by inverse CDF in vocabulary order
 // with a counter-based uniform (a hash of seed and position: no generator state, so a request's draws do not depend on
 // batching). One block per row.
+#include <type_traits>
+
 #include "common.h"
 #include "holon_hip.h"
 
@@ -480,6 +482,73 @@ __device__ void bitonic_sort(u64* a, int n_pad, bool descending) {
   }
 }
 
+// Top-p alone over a kept set too large to collect. The range of values that holds the last kept token is halved
+// until few enough tokens lie in it: `above` is the mass of the tokens over the range (all kept: it is within the
+// bound), and more than the bound lies over the range's lower end. The tokens of the range are then collected and
+// sorted, and the kept ones among them are those whose preceding mass, `above` included, is within the bound. Returns
+// the order key of the last kept token, or 0 when the range cannot be narrowed (thousands of equal values).
+__device__ u64 top_p_cut_wide(const float* __restrict__ row, int vocab, float inv_temp, float xmax, u64 bound, u64* cand,
+                              int* n_cand) {
+  __shared__ int kept_s;
+  const int tid = threadIdx.x;
+  float x_hi = xmax, x_lo = xmax - 128.f;        // (what lies further below weighs nothing)
+  u64 above = 0;
+  for (int step = 0;; ++step) {
+    const float x_mid = 0.5f * (x_lo + x_hi);
+    if (step == 48 || !(x_mid > x_lo && x_mid < x_hi)) return 0;
+    u64 mass = 0;
+    int up = 0, down = 0;
+    for_each_token(row, vocab, inv_temp, [&](float x, int) {
+      if (x > x_mid && x <= x_hi) { mass += fixed_mass(__expf(x - xmax)); ++up; }
+      else if (x > x_lo && x <= x_mid) ++down;
+    });
+    mass = block_sum_u64(mass);
+    up = block_sum_int(up);
+    down = block_sum_int(down);
+    int inside;
+    if (above + mass <= bound) { x_hi = x_mid; above += mass; inside = down; }
+    else { x_lo = x_mid; inside = up; }
+    if (inside <= SAMPLE_CANDIDATES) break;
+  }
+  if (tid == 0) *n_cand = 0;
+  __syncthreads();
+  for_each_token(row, vocab, inv_temp, [&](float x, int i) {
+    if (x > x_lo && x <= x_hi) {
+      const int at = atomicAdd(n_cand, 1);
+      if (at < SAMPLE_CANDIDATES) cand[at] = order_key(x, i);
+    }
+  });
+  __syncthreads();
+  const int count = *n_cand;
+  int n_pad = WAVE;
+  while (n_pad < count) n_pad <<= 1;
+  for (int i = count + tid; i < n_pad; i += blockDim.x) cand[i] = 0;
+  __syncthreads();
+  bitonic_sort(cand, n_pad, true);
+  const int per = max(1, n_pad / SAMPLE_THREADS);
+  u64 incl[SAMPLE_PER];
+  u64 run = 0;
+#pragma unroll
+  for (int e = 0; e < SAMPLE_PER; ++e) {
+    const int i = tid * per + e;
+    if (e < per && i < count) run += fixed_mass(__expf(key_float((uint32_t)(cand[i] >> 32)) - xmax));
+    incl[e] = run;
+  }
+  u64 all;
+  const u64 before = above + block_scan_u64(run, all);
+  int mine = 0;
+#pragma unroll
+  for (int e = 0; e < SAMPLE_PER; ++e) {
+    const int i = tid * per + e;
+    if (e < per && i < count) mine += (before + (e ? incl[e - 1] : 0)) <= bound;
+  }
+  const int kept = block_sum_int(mine);
+  if (tid == 0) kept_s = kept;
+  __syncthreads();
+  // nothing of the range kept: the last kept token is the smallest over the range, i.e. any value over x_hi passes
+  return kept_s > 0 ? cand[kept_s - 1] : ((u64)(float_key(x_hi) + 1u) << 32);
+}
+
 __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     const float* __restrict__ logits, int32_t* __restrict__ out, int vocab, const float* __restrict__ temperature,
     const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
@@ -510,6 +579,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     return;
   }
 
+  u64 cut = 0;                                  // tokens with order_key >= cut pass top-k and top-p
   if (k_on || p_on) {
     u64 z_all = 0;
     if (p_on && !k_on) {                         // top-p without top-k: the mass of the whole row
@@ -521,6 +591,8 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     // Which bands to collect: the fewest that should hold twice what is needed (k tokens; 256 for top-p alone). The
     // collecting counts exactly; too many, or fewer than k, and another set of bands is tried.
     const int need = k_on ? k : 1;
+    u64 wide_cut = 0;                            // set when the kept set is too large to collect: drawn as below
+    int beyond_at = -1;                          // the most bands found to hold too little of the mass
     int bands = SAMPLE_BANDS - 1;
     for (int j = SAMPLE_BANDS - 1; j >= 0; --j)
       if (counts[j] >= 2 * (k_on ? k : 256) + 64) bands = j;
@@ -528,11 +600,20 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     int count = 0;
     for (int attempt = 0;; ++attempt) {
       if (attempt == 6 || bands < 0 || bands >= SAMPLE_BANDS) {
-        sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
-        return;
+        if (p_on && !k_on) wide_cut = top_p_cut_wide(row, vocab, inv_temp, xmax, (u64)((double)p_keep * (double)z_all),
+                                                     cand, &n_cand);
+        if (wide_cut == 0) {
+          sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
+          return;
+        }
+        break;
       }
       count = collect_bands(row, vocab, inv_temp, xmax, bands, cand, &n_cand);
-      if (count > SAMPLE_CANDIDATES) { --bands; continue; }
+      if (count > SAMPLE_CANDIDATES) {
+        --bands;
+        if (bands <= beyond_at) attempt = 5;      // the next fewer bands held too little: no set of bands will do
+        continue;
+      }
       if (count < need && count < vocab) { ++bands; continue; }
       int n_pad = WAVE;
       while (n_pad < count) n_pad <<= 1;
@@ -574,12 +655,14 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
       // top-p alone, and everything collected was kept: the bound may lie past it, in bands not collected
       if (p_on && !k_on && count < vocab && n_keep_s == count) {
         __syncthreads();
+        beyond_at = bands;
         ++bands;
         while (bands < SAMPLE_BANDS - 1 && counts[bands] < 4 * count) ++bands;   // a good deal more at once
         continue;
       }
       break;
     }
+    if (wide_cut == 0) {
     // min-p drops q < min_p: the values only fall along the sorted order, so this keeps a prefix too
     int ok = 0;
     for (int i = tid; i < n_keep_s; i += blockDim.x) ok += __expf(key_float((uint32_t)(cand[i] >> 32)) - xmax) >= p_min;
@@ -620,17 +703,21 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     __syncthreads();
     if (tid == 0) out[r] = pick_s >= 0 ? pick_s : top.i;
     return;
+    }
+    cut = wide_cut;
+    __syncthreads();                            // `cand` is free from here on
   }
 
-  const u64 cut = 0;                            // no top-k, no top-p: every token passes them
   // the law, and the draw in vocabulary order
-  auto law = [&](float x, int i) -> uint32_t {
+  const bool every = cut == 0 && !(p_min > 0.f);   // nothing is dropped: the law is the mass itself
+  auto law = [&](float x, int i, auto all) -> uint32_t {
     const float q = __expf(x - xmax);
-    return (order_key(x, i) >= cut && q >= p_min) ? fixed_mass(q) : 0u;
+    if constexpr (decltype(all)::value) return fixed_mass(q);
+    else return (order_key(x, i) >= cut && q >= p_min) ? fixed_mass(q) : 0u;
   };
   u64* chunk_mass = cand;                       // [chunks]: the mass of tokens 256 c .. 256 c + 255, four to a lane
   const bool wide = (vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0;
-  auto lane_masses = [&](int c, uint32_t (&m)[4]) {
+  auto lane_masses = [&](int c, uint32_t (&m)[4], auto all) {
     const int i0 = c * SAMPLE_CHUNK + 4 * lane;
     float x[4];
     if (wide && i0 + 3 < vocab) {
@@ -641,14 +728,17 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
       for (int e = 0; e < 4; ++e) x[e] = i0 + e < vocab ? row[i0 + e] : -INFINITY;
     }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) m[e] = i0 + e < vocab ? law(x[e] * inv_temp, i0 + e) : 0u;
+    for (int e = 0; e < 4; ++e) m[e] = i0 + e < vocab ? law(x[e] * inv_temp, i0 + e, all) : 0u;
   };
-  for (int c = wave; c < chunks; c += SAMPLE_WAVES) {
-    uint32_t m[4];
-    lane_masses(c, m);
-    const u64 sum = wave_sum_u64((u64)m[0] + m[1] + m[2] + m[3]);
-    if (lane == 0) chunk_mass[c] = sum;
-  }
+  auto chunk_sums = [&](auto all) {
+    for (int c = wave; c < chunks; c += SAMPLE_WAVES) {
+      uint32_t m[4];
+      lane_masses(c, m, all);
+      const u64 sum = wave_sum_u64((u64)m[0] + m[1] + m[2] + m[3]);
+      if (lane == 0) chunk_mass[c] = sum;
+    }
+  };
+  if (every) chunk_sums(std::true_type{}); else chunk_sums(std::false_type{});
   if (tid == 0) pick_s = -1;
   __syncthreads();
   // a thread holds consecutive chunks; the one whose chunks hold the target names the chunk
@@ -675,7 +765,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
   __syncthreads();
   if (wave == 0) {
     uint32_t m[4];
-    lane_masses(chunk_s, m);
+    lane_masses(chunk_s, m, std::false_type{});
     const u64 mine4 = (u64)m[0] + m[1] + m[2] + m[3];
     u64 run = chunk_before_s + wave_scan_u64(mine4, lane) - mine4;   // the mass before this lane's four tokens
     int pick = -1;
