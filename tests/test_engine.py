@@ -142,18 +142,21 @@ def test_prompts_that_start_alike_share_their_cache_and_generate_the_same(folder
     assert tight.generate(prompts[:2], params) == want[:2]
 
 
-@pytest.mark.parametrize("seed", range(6))
-def test_random_traffic_generates_what_the_plain_model_generates(folders, seed):
+@pytest.mark.parametrize("device,seed", [pytest.param("cpu", s, id=f"cpu-twin-{s}") for s in range(6)] +
+                         [pytest.param("cuda", s, marks=pytest.mark.gpu, id=f"hip-{s}") for s in range(4)])
+def test_random_traffic_generates_what_the_plain_model_generates(folders, device, seed):
     """Requests arrive while others run: prompts that share starts, pools so tight that cached pages are evicted and
     requests preempted, portions beside decode rows or not, several sequences of a prompt. Every sequence is the
-    plain model's, drawn at the plain uniforms, whatever happened to it on the way (CPU twins of the kernels)."""
+    plain model's, drawn at the plain uniforms, whatever happened to it on the way. On the GPU the steps really
+    overlap: a step is launched while the one before it still runs, and pages freed by a request that just finished
+    are written by the next."""
     import random
     rng = random.Random(seed)
     plain = PlainQwen3(folders["Bu"])
     page = rng.choice([4, 8])
     max_len = 64
     mixed = rng.choice([0, 6])
-    engine = _engine(folders["Bu"], "cpu", page_size=page, max_seqs=rng.choice([2, 3, 5]), max_model_len=max_len,
+    engine = _engine(folders["Bu"], device, page_size=page, max_seqs=rng.choice([2, 3, 5]), max_model_len=max_len,
                      max_step_tokens=rng.choice([16, 24]), chunk_with_decode=mixed,
                      cache_tokens=rng.choice([64, 96, 160]), prefix_cache=rng.random() < 0.8,
                      overlap=rng.random() < 0.7)
