@@ -21,7 +21,7 @@ import numpy as np
 import torch
 
 from ..parts.base import PagedState, SlotState
-from .pool import OutOfPages, PagePool
+from .pool import PagePool
 from .prefix import PrefixIndex
 
 
