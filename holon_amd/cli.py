@@ -21,6 +21,9 @@ import typing
 from .config import EngineConfig, SamplingParams
 
 
+AUTO_CONTEXT = 32768      # `--max-model-len auto`: the model's trained context, at most this
+
+
 def engine_flags(parser: argparse.ArgumentParser | argparse._ArgumentGroup) -> None:
     hints = typing.get_type_hints(EngineConfig)
     for f in dataclasses.fields(EngineConfig):
@@ -30,6 +33,9 @@ def engine_flags(parser: argparse.ArgumentParser | argparse._ArgumentGroup) -> N
         help_ = f.metadata["help"] + (f" (default: {f.default})" if f.default is not None else "")
         if kind is bool:
             parser.add_argument(flag, action=argparse.BooleanOptionalAction, default=f.default, help=help_)
+        elif f.name == "max_model_len":            # also `auto` (core/holon/core/cli.py:44-47, 76)
+            parser.add_argument(flag, type=lambda s: s if s == "auto" else int(s), default=f.default,
+                                help=help_ + f"; auto: the model's trained context, at most {AUTO_CONTEXT}")
         elif kind in (int, float, str):
             parser.add_argument(flag, type=kind, default=f.default, help=help_)
         else:                                         # int | None
@@ -38,7 +44,12 @@ def engine_flags(parser: argparse.ArgumentParser | argparse._ArgumentGroup) -> N
 
 def engine_config(model: str, args: argparse.Namespace) -> EngineConfig:
     names = {f.name for f in dataclasses.fields(EngineConfig)} - {"model"}
-    return EngineConfig(model=model, **{k: v for k, v in vars(args).items() if k in names})
+    settings = {k: v for k, v in vars(args).items() if k in names}
+    if settings.get("max_model_len") == "auto":
+        from .config.model import read_config_json
+        trained = read_config_json(model)[0].get("max_position_embeddings")
+        settings["max_model_len"] = min(int(trained), AUTO_CONTEXT) if trained else AUTO_CONTEXT
+    return EngineConfig(model=model, **settings)
 
 
 def _ids(text: str) -> list[int]:

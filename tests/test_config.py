@@ -110,3 +110,19 @@ def test_command_line_has_a_flag_per_engine_setting():
     assert {f.name for f in dataclasses.fields(EngineConfig)} - {"model"} <= flags
     out = subprocess.run([sys.executable, "-m", "holon_amd", "models"], capture_output=True, text=True, check=True)
     assert "Qwen3ForCausalLM" in out.stdout
+
+
+def test_command_line_makes_engine_settings_and_takes_auto_for_the_context(tmp_path):
+    """One flag a field of EngineConfig; `--max-model-len auto` is the model's trained context, at most 32,768."""
+    import argparse
+    import json
+    from holon_amd import cli
+    ap = argparse.ArgumentParser()
+    cli.engine_flags(ap)
+    (tmp_path / "config.json").write_text(json.dumps({"architectures": ["Qwen3ForCausalLM"],
+                                                       "max_position_embeddings": 40960}))
+    got = cli.engine_config(str(tmp_path), ap.parse_args(["--max-model-len", "auto", "--no-prefix-cache", "--page-size", "32"]))
+    assert (got.max_model_len, got.prefix_cache, got.page_size, got.overlap) == (32768, False, 32, True)
+    (tmp_path / "config.json").write_text(json.dumps({"architectures": ["Qwen3ForCausalLM"], "max_position_embeddings": 512}))
+    assert cli.engine_config(str(tmp_path), ap.parse_args(["--max-model-len", "auto"])).max_model_len == 512
+    assert cli.engine_config(str(tmp_path), ap.parse_args(["--max-model-len", "100"])).max_model_len == 100
