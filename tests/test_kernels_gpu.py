@@ -51,6 +51,14 @@ def test_embedding_and_silu_mul(hip, dtype):
     assert torch.equal(hip.embedding(ids, table), table[ids.long()])
     table = _randn(333, 4096, dtype=dtype, seed=5)
     assert torch.equal(hip.embedding(ids[2:], table), table[ids[2:].long()])
+    # tokens that the last step drew and left on the device: kept by slot, taken where a row says so
+    last = torch.zeros(9, dtype=torch.int32).cuda()
+    hip.store_tokens(last, torch.tensor([7, 2, 5], dtype=torch.int32).cuda(), torch.tensor([330, 11, 0], dtype=torch.int32).cuda())
+    assert last.tolist() == [0, 0, 11, 0, 0, 0, 0, 330, 0]
+    take = torch.tensor([-1, 7, -1, 2, 5], dtype=torch.int32).cuda()
+    want = table[torch.tensor([0, 330, 5, 11, 0])]
+    assert torch.equal(hip.embedding(ids, table, (take, last)), want)
+    assert torch.equal(PLAIN.embedding(ids, table, (take, last)), want)
     for t, inter in ((17, 12288), (3, 100), (1, 7)):
         gu = _randn(t, 2 * inter, dtype=dtype, seed=6, scale=3.0)
         got, want = hip.silu_mul(gu), PLAIN.silu_mul(gu.double())
