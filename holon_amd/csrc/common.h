@@ -31,6 +31,14 @@ template <> struct Elem<bf16_t> {
   static __device__ __forceinline__ float round(float v) { return bf16_to_float(float_to_bf16(v)); }
 };
 
+// silu(g) = g / (1 + exp(-g)). For float32 results the library's exp and a true division; for bfloat16 results (8 bits
+// are kept) the hardware's exp2 and reciprocal, whose error of about 2^-22 vanishes in the rounding.
+template <typename T> __device__ __forceinline__ float silu(float g);
+template <> __device__ __forceinline__ float silu<float>(float g) { return g / (1.0f + expf(-g)); }
+template <> __device__ __forceinline__ float silu<bf16_t>(float g) {
+  return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);

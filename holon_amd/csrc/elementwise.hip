@@ -193,7 +193,7 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
     const int c = (int)(i - t * inter);
     const float g = Elem<T>::load(gu[t * 2 * inter + c]);
     const float u = Elem<T>::load(gu[t * 2 * inter + inter + c]);
-    const float s = Elem<T>::round(g / (1.0f + expf(-g)));
+    const float s = Elem<T>::round(silu<T>(g));
     out[i] = Elem<T>::store(s * u);
   }
 }
@@ -216,7 +216,7 @@ __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ ou
 #pragma unroll
     for (int j = 0; j < V; ++j) {
       const float g = Elem<T>::load(ge[j]);
-      const float sg = Elem<T>::round(g / (1.0f + expf(-g)));
+      const float sg = Elem<T>::round(silu<T>(g));
       oe[j] = Elem<T>::store(sg * Elem<T>::load(ue[j]));
     }
     *reinterpret_cast<uint4*>(out + t * inter + c) = oraw;
@@ -324,65 +324,81 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
     T* __restrict__ pages, const int32_t* __restrict__ write_page, const int32_t* __restrict__ write_off,
     int page_size, int total_heads) {
   constexpr int D = LPH * 8;
-  constexpr int HPB = 256 / LPH;                     // heads a block covers
+  constexpr int HPB = 256 / LPH;                     // heads a block covers at a time
   const int t = blockIdx.x;
-  const int h = blockIdx.y * HPB + threadIdx.x / LPH;
   const int li = threadIdx.x % LPH;                  // lane within the head
-  const bool active = h < total_heads;               // (shuffles below are executed by every lane)
-  const int hh = active ? h : 0;
-  const T* src = qkv + (int64_t)t * qkv_stride + (int64_t)hh * D + li * 8;
-  float v[8];
-  if (sizeof(T) == 2) {
-    const uint4 raw = *reinterpret_cast<const uint4*>(src);
-    const T* e = reinterpret_cast<const T*>(&raw);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = Elem<T>::load(e[j]);
-  } else {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = Elem<T>::load(src[j]);
-  }
-  if (active && hh >= heads + kv_heads) {   // a value head: transposed inside the page
-    const int hk = hh - heads - kv_heads;
-    T* dst = pages + (((int64_t)write_page[t] * 2 + 1) * kv_heads + hk) * (int64_t)page_size * D + write_off[t];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) dst[(int64_t)(li * 8 + j) * page_size] = Elem<T>::store(v[j]);
-  }
-  const bool is_v = hh >= heads + kv_heads;
-  const bool is_q = hh < heads;
-  const T* weight = is_q ? q_weight : k_weight;
-  if (weight != nullptr) {
-    float ss = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
-#pragma unroll
-    for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
-    const float inv = 1.0f / sqrtf(ss / (float)D + eps);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = Elem<T>::round((v[j] * inv) * Elem<T>::load(weight[li * 8 + j]));
-  }
+  // this lane's eight cosines and sines: the same for every head of the token
+  float co[8], si[8];
   if (table != nullptr) {
-    const float* cs = table + (int64_t)positions[t] * D;
-    const int i0 = (li % (LPH / 2)) * 8;   // index of the pair within the half
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float other = __shfl_xor(v[j], LPH / 2, WAVE);
-      const float co = cs[i0 + j], si = cs[D / 2 + i0 + j];
-      v[j] = li < LPH / 2 ? v[j] * co - other * si : v[j] * co + other * si;
-    }
+    const float* cs = table + (int64_t)positions[t] * D + (li % (LPH / 2)) * 8;   // the pair's place within the half
+    const float4 c0 = *reinterpret_cast<const float4*>(cs), c1 = *reinterpret_cast<const float4*>(cs + 4);
+    const float4 s0 = *reinterpret_cast<const float4*>(cs + D / 2), s1 = *reinterpret_cast<const float4*>(cs + D / 2 + 4);
+    co[0] = c0.x; co[1] = c0.y; co[2] = c0.z; co[3] = c0.w; co[4] = c1.x; co[5] = c1.y; co[6] = c1.z; co[7] = c1.w;
+    si[0] = s0.x; si[1] = s0.y; si[2] = s0.z; si[3] = s0.w; si[4] = s1.x; si[5] = s1.y; si[6] = s1.z; si[7] = s1.w;
   }
-  if (!active || is_v) return;
-  T* dst = is_q ? q_out + ((int64_t)t * heads + hh) * D + li * 8
-                : pages + (((int64_t)write_page[t] * 2 + 0) * kv_heads + (hh - heads)) * (int64_t)page_size * D +
-                      (int64_t)write_off[t] * D + li * 8;
-  if (sizeof(T) == 2) {
-    uint4 out;
-    T* oe = reinterpret_cast<T*>(&out);
+  // a block takes HPB heads, then (with fewer blocks than that along y) the next HPB, ...
+  for (int h0 = blockIdx.y * HPB; h0 < total_heads; h0 += gridDim.y * HPB) {
+    const int h = h0 + threadIdx.x / LPH;
+    const bool active = h < total_heads;             // (shuffles below are executed by every lane)
+    const int hh = active ? h : 0;
+    const T* src = qkv + (int64_t)t * qkv_stride + (int64_t)hh * D + li * 8;
+    float v[8];
+    if (sizeof(T) == 2) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(src);
+      const T* e = reinterpret_cast<const T*>(&raw);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) oe[j] = Elem<T>::store(v[j]);
-    *reinterpret_cast<uint4*>(dst) = out;
-  } else {
+      for (int j = 0; j < 8; ++j) v[j] = Elem<T>::load(e[j]);
+    } else {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) dst[j] = Elem<T>::store(v[j]);
+      for (int j = 0; j < 8; ++j) v[j] = Elem<T>::load(src[j]);
+    }
+    const bool is_v = hh >= heads + kv_heads;
+    const bool is_q = hh < heads;
+    if (active && is_v) {   // a value head: transposed inside the page
+      const int hk = hh - heads - kv_heads;
+      T* dst = pages + (((int64_t)write_page[t] * 2 + 1) * kv_heads + hk) * (int64_t)page_size * D + write_off[t];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dst[(int64_t)(li * 8 + j) * page_size] = Elem<T>::store(v[j]);
+    }
+    const T* weight = is_q ? q_weight : k_weight;
+    if (weight != nullptr) {
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
+#pragma unroll
+      for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
+      const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+      T w[8];
+      if (sizeof(T) == 2) {
+        *reinterpret_cast<uint4*>(w) = *reinterpret_cast<const uint4*>(weight + li * 8);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = weight[li * 8 + j];
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = Elem<T>::round((v[j] * inv) * Elem<T>::load(w[j]));
+    }
+    if (table != nullptr) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float other = __shfl_xor(v[j], LPH / 2, WAVE);
+        v[j] = li < LPH / 2 ? v[j] * co[j] - other * si[j] : v[j] * co[j] + other * si[j];
+      }
+    }
+    if (!active || is_v) continue;
+    T* dst = is_q ? q_out + ((int64_t)t * heads + hh) * D + li * 8
+                  : pages + (((int64_t)write_page[t] * 2 + 0) * kv_heads + (hh - heads)) * (int64_t)page_size * D +
+                        (int64_t)write_off[t] * D + li * 8;
+    if (sizeof(T) == 2) {
+      uint4 out;
+      T* oe = reinterpret_cast<T*>(&out);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) oe[j] = Elem<T>::store(v[j]);
+      *reinterpret_cast<uint4*>(dst) = out;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dst[j] = Elem<T>::store(v[j]);
+    }
   }
 }
 
@@ -463,7 +479,8 @@ extern "C" int holon_qk_norm_rope_write(const void* qkv, int64_t qkv_stride, voi
     const bool split_v = pages != nullptr && tokens >= 256;
     const int fast_heads = split_v ? heads + kv_heads : total_heads;
     const int lph = head_dim / 8;
-    grid = dim3(tokens, (fast_heads + 256 / lph - 1) / (256 / lph));
+    // many tokens: one block a token walks all its heads, with the token's cosines and sines read once
+    grid = dim3(tokens, tokens >= 256 ? 1 : (fast_heads + 256 / lph - 1) / (256 / lph));
 #define QK_FAST(T, LPH)                                                                                            \
   qk_norm_rope_write_fast_kernel<T, LPH><<<grid, 256, 0, s>>>(                                                      \
       (const T*)qkv, qkv_stride, (T*)q_out, heads, kv_heads, (const T*)q_weight, (const T*)k_weight, eps, table,    \

@@ -272,7 +272,7 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t*
     for (int r = 0; r < 4; ++r) {
       const float gate = bf16_to_float(float_to_bf16(acc[0][t][r]));
       const float up = bf16_to_float(float_to_bf16(acc[1][t][r]));
-      const float sg = bf16_to_float(float_to_bf16(gate / (1.0f + expf(-gate))));
+      const float sg = bf16_to_float(float_to_bf16(silu<bf16_t>(gate)));
       oe[r] = float_to_bf16(sg * up);
     }
     *reinterpret_cast<ushort4*>(y + (int64_t)m * I + n0 + 4 * g) = o;

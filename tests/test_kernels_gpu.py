@@ -181,7 +181,8 @@ def test_fused_norm_rope_write_is_the_three_ops(hip, dtype, geometry):
     qw, kw = _randn(head_dim, dtype=dtype, seed=9), _randn(head_dim, dtype=dtype, seed=10)
     # few tokens at scattered places; many tokens at consecutive places (whole pages and ragged ends); many scattered
     layouts = [(45, rng.permutation(40 * page)[:45]), (200, np.arange(200) + 3 * page), (130, np.arange(130) + 5),
-               (100, rng.permutation(40 * page)[:100])]
+               (100, rng.permutation(40 * page)[:100]), (300, np.arange(300) + 2 * page + 3),
+               (260, rng.permutation(80 * page)[:260])]      # from 256 tokens on a block walks all heads of its token
     for t, where in layouts:
         units = int(where.max()) // page + 2
         qkv = _randn(t, (heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=8)
