@@ -140,6 +140,30 @@ def test_paged_attention(hip, dtype, page, geometry):
         assert H.op_budget_usage(got, want, dtype, head_dim + max(s + n for s, n in rows)) <= 1, (geometry, page, rows)
 
 
+@pytest.mark.parametrize("geometry", [(32, 8, 128), (16, 8, 64), (8, 1, 128)])
+def test_long_prompt_portions_two_tiles_a_wave(hip, geometry):
+    """Portions long enough that the LDS kernel gives a wave two tiles (from two blocks a compute unit on): one row of
+    4,500 tokens from position 0, two rows continuing earlier tokens (so the keys start before the queries), and a
+    window."""
+    heads, kv_heads, head_dim = geometry
+    bf = torch.bfloat16
+    for rows, window in (([(0, 4500)], 0), ([(300, 4200), (77, 2300)], 0), ([(1000, 4100)], 600)):
+        q, pages, table, attn = _paged_case(rows, heads, kv_heads, head_dim, 16, bf, seed=len(rows) + window)
+        scale = head_dim ** -0.5
+        want = PLAIN.paged_attention(q.double(), pages.double(), table, attn, 16, scale, window)
+        got = hip.paged_attention(q, pages, table, attn, 16, scale, window)
+        # rows that see few keys are averages of few values and much larger than rows that see thousands: each
+        # stretch of rows is held to the budget of its own size and of the keys it sees
+        at = 0
+        for start, n in rows:
+            for lo, hi in ((0, 64), (64, 512), (512, n)):
+                part = slice(at + lo, at + min(hi, n))
+                span = head_dim + (min(window, start + hi) if window else start + min(hi, n))
+                assert H.op_budget_usage(got[part], want[part], bf, span) <= 1, (geometry, rows, window, lo)
+            at += n
+        assert torch.equal(got, hip.paged_attention(q, pages, table, attn, 16, scale, window))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("window", [1, 7, 16, 100])
 def test_paged_attention_window(hip, dtype, window):
