@@ -426,6 +426,33 @@ def test_sampling_filters_at_the_full_vocabulary(hip):
     assert got[2] == int(tied.argmax()) and got[3] == int(peaked.argmax())
 
 
+def test_sampling_under_random_settings(hip):
+    """Many rows with settings drawn at random, a row each its own: vocabularies of 1,000 to 33,000, flat to sharp
+    rows, every filter alone and together, k beyond what is collected. A drawn token lies in the plain law's kept set
+    and at the hashed uniform of the plain CDF."""
+    import random
+    from tests.plain import sampling as S
+    rng = random.Random(7)
+    for vocab in (1000, 5003, 33000):
+        g = torch.Generator().manual_seed(vocab)
+        rows = 48
+        scales = [rng.choice([0.3, 1.0, 3.0, 10.0]) for _ in range(rows)]
+        logits = torch.randn(rows, vocab, generator=g) * torch.tensor(scales)[:, None]
+        temp = [rng.choice([0.3, 0.7, 1.0, 1.5]) for _ in range(rows)]
+        top_k = [rng.choice([0, 0, 1, 5, 50, 500, 3000, 5000]) for _ in range(rows)]
+        top_p = [rng.choice([1.0, 1.0, 0.99, 0.9, 0.5, 0.1]) for _ in range(rows)]
+        min_p = [rng.choice([0.0, 0.0, 0.01, 0.2]) for _ in range(rows)]
+        t = lambda v, dt: torch.tensor(v, dtype=dt).cuda()
+        got = hip.sample(logits.cuda(), t(temp, torch.float32), t(top_k, torch.int32), t(top_p, torch.float32),
+                         t(min_p, torch.float32), t([11] * rows, torch.int64), torch.arange(rows).cuda()).tolist()
+        for r in range(rows):
+            law = S.probs(logits[r], temp[r], top_k[r], top_p[r], min_p[r])
+            case = (vocab, r, scales[r], temp[r], top_k[r], top_p[r], min_p[r])
+            assert law[got[r]] > 0, case
+            cdf, u = law.cumsum(0), S.uniform(11, r)
+            assert (cdf[got[r] - 1] if got[r] else 0.0) - 2e-5 <= u < cdf[got[r]] + 2e-5, case
+
+
 def test_kernels_refuse_what_they_do_not_serve(hip):
     from holon_amd.kernels.hip import KernelError
     with pytest.raises(KernelError):
