@@ -114,7 +114,8 @@ def _paged_case(rows, heads, kv_heads, head_dim, page, dtype, seed=0, max_seqs=8
 
 
 GEOMETRIES = [(32, 8, 128), (16, 4, 256), (16, 8, 64), (6, 3, 32), (4, 1, 16), (5, 5, 48), (12, 2, 80),
-              (10, 2, 64), (40, 2, 128), (7, 7, 64), (6, 1, 128), (48, 2, 64)]   # groups of 5, 20, 1, 6 and 24 heads
+              (10, 2, 64), (40, 2, 128), (7, 7, 64), (6, 1, 128), (48, 2, 64),   # groups of 5, 20, 1, 6 and 24 heads
+              (40, 1, 128), (66, 1, 64)]                                         # and of more heads than a tile has rows
 ROWSETS = [[(0, 1), (0, 17), (5, 16), (31, 33), (0, 64), (100, 7), (16, 16)],
            [(0, 1), (15, 1), (16, 1), (99, 1), (999, 1), (4096, 1)],
            [(63, 1), (200, 2), (17, 1), (0, 130), (1, 1)]]
@@ -140,11 +141,13 @@ def test_paged_attention(hip, dtype, page, geometry):
         assert H.op_budget_usage(got, want, dtype, head_dim + max(s + n for s, n in rows)) <= 1, (geometry, page, rows)
 
 
-@pytest.mark.parametrize("geometry", [(32, 8, 128), (16, 8, 64), (8, 1, 128)])
+@pytest.mark.parametrize("geometry", [(32, 8, 128), (16, 8, 64), (8, 1, 128), (7, 7, 64), (6, 2, 64), (5, 1, 128),
+                                      (24, 1, 64), (32, 1, 128), (40, 1, 128), (66, 1, 64), (80, 2, 64)])
 def test_long_prompt_portions_two_tiles_a_wave(hip, geometry):
-    """Portions long enough that the LDS kernel gives a wave two tiles (from two blocks a compute unit on): one row of
-    4,500 tokens from position 0, two rows continuing earlier tokens (so the keys start before the queries), and a
-    window."""
+    """Portions long enough for the kernels that stage keys and values through LDS (tiles of 32 rows for groups of up
+    to 32 heads, tiles of 16 rows, one or two a wave, for larger groups): one row of 4,500 tokens from position 0, two
+    rows continuing earlier tokens (so the keys start before the queries), and a window. Groups of 1, 3, 5, 24, 32
+    (tiles that hold one position or several, whole or in part), 40 and 66 heads."""
     heads, kv_heads, head_dim = geometry
     bf = torch.bfloat16
     for rows, window in (([(0, 4500)], 0), ([(300, 4200), (77, 2300)], 0), ([(1000, 4100)], 600)):
