@@ -1,7 +1,11 @@
 // Paged causal attention, the general kernel: any element type, any page size, any head_dim that is a multiple of 8.
 // One wave per (query token, query head). Keys are visited in tiles of 64 starting at the first visible key, so the
-// order of every sum depends on the token's position alone, never on how the batch was cut. Scores, softmax and the
-// value sum are float32.
+// order of every sum depends on the token's position alone, never on how the batch was cut. Scores and softmax are
+// float32. For float32 operands the two long sums (a score over head_dim, the values over the keys) are accumulated in
+// float64, which this GPU does at the float32 rate: a float32 running sum over 256 products of a sharp query and key
+// is off by 1e-4 of the score, and that shows in the weights of the softmax.
+#include <type_traits>
+
 #include "common.h"
 #include "holon_hip.h"
 
@@ -16,6 +20,7 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, T* __restrict_
   __shared__ float q_s[4][GEN_MAX_D];
   __shared__ float p_s[4][WAVE];
   __shared__ int64_t v_s[4][WAVE];   // element offset of each tile key's value column
+  using Acc = std::conditional_t<std::is_same<T, float>::value, double, float>;
   const int w = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int t = blockIdx.x;
   const bool active = blockIdx.y * 4 + w < heads;
@@ -44,9 +49,9 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, T* __restrict_
 
   const int first = window > 0 ? max(0, pos - window + 1) : 0;
   float m = -INFINITY, l = 0.f;
-  float acc[GEN_MAX_D / WAVE];
+  Acc acc[GEN_MAX_D / WAVE];
 #pragma unroll
-  for (int i = 0; i < GEN_MAX_D / WAVE; ++i) acc[i] = 0.f;
+  for (int i = 0; i < GEN_MAX_D / WAVE; ++i) acc[i] = 0;
   constexpr int V = Elem<T>::kVec;
 
   for (int j0 = first; j0 <= pos; j0 += WAVE) {
@@ -59,14 +64,14 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, T* __restrict_
       const int off = key - (key / page_size) * page_size;
       const T* kp = pages + (((int64_t)page * 2 + 0) * kv_heads + hk) * plane + (int64_t)off * head_dim;
       voff = (((int64_t)page * 2 + 1) * kv_heads + hk) * plane + off;
-      float dot = 0.f;
+      Acc dot = 0;
       for (int d = 0; d < head_dim; d += V) {
         const uint4 raw = *reinterpret_cast<const uint4*>(kp + d);
         const T* e = reinterpret_cast<const T*>(&raw);
 #pragma unroll
-        for (int i = 0; i < V; ++i) dot += q_s[w][d + i] * Elem<T>::load(e[i]);
+        for (int i = 0; i < V; ++i) dot += (Acc)q_s[w][d + i] * (Acc)Elem<T>::load(e[i]);
       }
-      s = dot * scale;
+      s = (float)dot * scale;
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float alpha = expf(m - m_new);          // m = -inf on the first tile: alpha = 0
@@ -81,8 +86,9 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, T* __restrict_
     for (int i = 0; i < GEN_MAX_D / WAVE; ++i) {
       const int d = lane + i * WAVE;
       if (d < head_dim) {
-        float a = acc[i] * alpha;
-        for (int j = 0; j < count; ++j) a += p_s[w][j] * Elem<T>::load(pages[v_s[w][j] + (int64_t)d * page_size]);
+        Acc a = acc[i] * (Acc)alpha;
+        for (int j = 0; j < count; ++j)
+          a += (Acc)p_s[w][j] * (Acc)Elem<T>::load(pages[v_s[w][j] + (int64_t)d * page_size]);
         acc[i] = a;
       }
     }
@@ -92,7 +98,7 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, T* __restrict_
 #pragma unroll
   for (int i = 0; i < GEN_MAX_D / WAVE; ++i) {
     const int d = lane + i * WAVE;
-    if (d < head_dim) o[d] = Elem<T>::store(acc[i] / l);
+    if (d < head_dim) o[d] = Elem<T>::store((float)(acc[i] / (Acc)l));
   }
 }
 
