@@ -196,6 +196,64 @@ def test_random_traffic_generates_what_the_plain_model_generates(folders, device
     assert _released(engine)
 
 
+@pytest.mark.parametrize("device,seed", [pytest.param("cpu", s, id=f"cpu-twin-{s}") for s in range(3)] +
+                         [pytest.param("cuda", s, marks=pytest.mark.gpu, id=f"hip-{s}") for s in range(2)])
+def test_random_traffic_with_aborts(folders, device, seed):
+    """The same traffic with requests aborted at random moments (waiting, in a prompt, decoding, with a step in
+    flight): what an aborted request gave until then is the plain model's, the others never notice, and every page
+    and slot comes back."""
+    import random
+    rng = random.Random(10_000 + seed)
+    plain = PlainQwen3(folders["Bu"])
+    engine = _engine(folders["Bu"], device, page_size=rng.choice([4, 8]), max_seqs=rng.choice([2, 3, 5]), max_model_len=64,
+                     max_step_tokens=rng.choice([16, 24]), chunk_with_decode=rng.choice([0, 6]),
+                     cache_tokens=rng.choice([64, 96, 160]), prefix_cache=rng.random() < 0.8, overlap=rng.random() < 0.7)
+    starts = [H.random_ids(40, 384, 1000 * seed + i) for i in range(2)]
+    todo = {}
+    for i in range(12):
+        prompt = rng.choice(starts)[:rng.randrange(0, 30)] + H.random_ids(rng.randrange(1, 12), 384, 2000 * seed + i)
+        greedy = rng.random() < 0.4
+        todo[f"r{i}"] = (prompt, SamplingParams(temperature=0.0 if greedy else 0.9, seed=50 + i, ignore_eos=True,
+                                                max_tokens=rng.randrange(1, 14), n=1 if greedy else rng.choice([1, 1, 2]),
+                                                top_k=rng.choice([0, 0, 20])))
+    want = {}
+    for rid, (prompt, p) in todo.items():
+        for i in range(p.n):
+            want[rid, i] = plain.greedy(prompt, p.max_tokens) if p.greedy else \
+                _plain_sampled(plain, prompt, p.max_tokens, S.sequence_seed(p.seed, i), p.temperature, top_k=p.top_k)
+    got = {key: [] for key in want}
+    done, aborted, added = set(), set(), []
+    pending = list(todo)
+    for _ in range(3000):
+        while pending and rng.random() < 0.3:
+            rid = pending.pop(0)
+            engine.add(todo[rid][0], todo[rid][1], rid=rid)
+            added.append(rid)
+        if added and rng.random() < 0.08:
+            rid = rng.choice(added)
+            if rid not in aborted and not all((rid, i) in done for i in range(todo[rid][1].n)):
+                engine.abort(rid)
+                aborted.add(rid)
+        if not engine.has_work():
+            if not pending:
+                break
+            continue
+        for d in engine.step():
+            assert d.rid not in aborted, "a delta of an aborted request"
+            got[d.rid, d.index] += d.token_ids
+            if d.finish_reason:
+                assert d.finish_reason == "length" and (d.rid, d.index) not in done
+                done.add((d.rid, d.index))
+        engine.cache.check()
+    assert aborted, "the seed aborts nothing"
+    for (rid, i), tokens in got.items():
+        if rid in aborted:
+            assert tokens == want[rid, i][: len(tokens)]
+        else:
+            assert tokens == want[rid, i] and (rid, i) in done
+    assert _released(engine)
+
+
 @pytest.mark.parametrize("device", DEVICES)
 def test_a_step_in_flight_changes_no_token(folders, device):
     """With `overlap` a step is scheduled and launched before the one before it has been committed: a decode row
