@@ -3,10 +3,16 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--no-points]
     python -m holon_amd bench ...          (the same)
 
+    python bench.py --workload mixed|long [--layers L]
+
 One JSON line: decoded tokens a second at the given batch (default 8) with every request near a context of 4,096 tokens
 (a 2,048-token prompt and 2,048 generated tokens), plus the prefill of one 2,048-token prompt, the decode step's memory
 roofline, and decode at batch 1 and 64. A step is one decode step of the engine: scheduling, the model, sampling and
 the commit. The engine is one process on one GPU; for --gpus > 1 a line says so and the exit code is 2.
+
+--workload runs a whole job through the engine instead and prints its own line: `mixed` is 32 requests of 128 to 4,096
+prompt tokens at the Qwen3-32B shape, portions of 512 tokens beside decode rows, 256 greedy tokens each; `long` is 8
+prompts of 32,768 tokens at the Qwen3-4B shape, 512 tokens each at temperature 0.7.
 """
 from __future__ import annotations
 
@@ -22,6 +28,60 @@ QWEN3_8B = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 36, "hid
             "vocab_size": 151936, "rope_theta": 1e6, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
             "max_position_embeddings": 40960}
 CONTEXT, PROMPT = 4096, 2048
+QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
+QWEN3_4B = dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, tie_word_embeddings=True)
+
+
+def workload(name: str, layers: int | None, dtype: str) -> int:
+    """A whole job: every request added at once, stepped until all are finished."""
+    import random
+
+    import torch
+
+    from .config import EngineConfig, SamplingParams
+    from .engine.engine import Engine
+    rng = random.Random(0)
+    if name == "mixed":
+        shape, model = QWEN3_32B, "Qwen3-32B shape"
+        prompts = [[rng.randrange(shape["vocab_size"]) for _ in range(rng.randint(128, 4096))] for _ in range(32)]
+        params = SamplingParams(temperature=0.0, max_tokens=256, ignore_eos=True)
+        ecfg = dict(max_seqs=32, max_model_len=4096 + 256 + 16, max_step_tokens=1024, chunk_with_decode=512)
+    else:
+        shape, model = QWEN3_4B, "Qwen3-4B shape"
+        prompts = [[rng.randrange(shape["vocab_size"]) for _ in range(32768)] for _ in range(8)]
+        params = SamplingParams(temperature=0.7, seed=1, max_tokens=512, ignore_eos=True)
+        ecfg = dict(max_seqs=8, max_model_len=40960, max_step_tokens=4096)
+    cfg_json = dict(shape, num_hidden_layers=layers or shape["num_hidden_layers"])
+    engine = Engine.from_random(cfg_json, seed=0, cfg=EngineConfig(
+        model=f"random:{name}", device="cuda:0", dtype=dtype, page_size=16,
+        cache_tokens=len(prompts) * (max(map(len, prompts)) + params.max_tokens + 64), **ecfg))
+    for p in prompts:
+        engine.add(p, params)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = steps = out_at = 0
+    t_prompts = None
+    while engine.has_work():
+        out += sum(len(d.token_ids) for d in engine.step())
+        steps += 1
+        if t_prompts is None and not engine.sched.waiting and all(
+                s.num_computed >= s.prompt_len for s in engine.sched.running):
+            torch.cuda.synchronize()
+            t_prompts, out_at = time.perf_counter() - t0, out
+    torch.cuda.synchronize()
+    total = time.perf_counter() - t0
+    stats = engine.stats()
+    prompt_tokens = sum(map(len, prompts))
+    print(json.dumps({
+        "metric": f"{name} workload, {model}: tokens/s over the whole job", "value": round((prompt_tokens + out) / total, 1),
+        "unit": "tokens/s", "n_gpus": 1, "seconds": round(total, 3), "dtype": "bf16" if dtype == "bfloat16" else "fp32",
+        "data": "synthetic (random weights, uniform random token ids)",
+        "config": {"model": model, "layers": cfg_json["num_hidden_layers"], "layers_of_config": shape["num_hidden_layers"],
+                   "requests": len(prompts), "prompt_tokens": prompt_tokens, "output_tokens": out, **ecfg},
+        "until_prompts_done": {"seconds": round(t_prompts, 3), "prompt_tokens_per_s": round(prompt_tokens / t_prompts, 1)},
+        "decode_tail": {"tokens_per_s": round((out - out_at) / max(total - t_prompts, 1e-9), 1)},
+        "steps": steps, "mixed_steps": stats["mixed_steps"], "preemptions": stats["preemptions"]}), flush=True)
+    return 0
 
 
 def main(argv: list[str] | None = None) -> int:
@@ -35,10 +95,16 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--workload", choices=("decode", "mixed", "long"), default="decode")
     a = ap.parse_args(argv)
     if a.gpus != 1:
         print(f"bench.py: this engine serves on one GPU; --gpus {a.gpus} is not a configuration it has", flush=True)
         return 2
+    if a.workload != "decode":
+        from .kernels import build as kernel_build
+        if kernel_build.find_library() is None:
+            kernel_build.build()
+        return workload(a.workload, None if "--layers" not in (argv or sys.argv) else a.layers, a.dtype)
 
     import torch
 
