@@ -527,18 +527,23 @@ __global__ void __launch_bounds__(256) attn_prefill_wide_kernel(AttnArgs a) {
   constexpr int KCH = D / 8;
   constexpr int ROUNDS = D / 64;
   static_assert(D == 64 || D == 128, "the LDS kernels copy one or two chunks of each kind per thread");
-  int k_key[ROUNDS], k_col[ROUNDS], k_dst[ROUNDS], v_d[ROUNDS], v_kc[ROUNDS], v_dst[ROUNDS];
+  // What a thread copies per stage: ROUNDS 16-byte pieces of keys and of values. With D = 128 a round is one half
+  // of the stage (keys 0-15, then 16-31), so that every lane of a round reads the same page and an address is a
+  // scalar base plus a lane offset that never changes; with D = 64 the one round covers both halves.
+  constexpr bool HALVES = ROUNDS == 2;
+  int k_half[ROUNDS], k_off[ROUNDS], k_dst[ROUNDS], v_half[ROUNDS], v_off[ROUNDS], v_dst[ROUNDS];
 #pragma unroll
   for (int i = 0; i < ROUNDS; ++i) {
     const int q = tid + 256 * i;
-    k_key[i] = q / KCH;
-    k_col[i] = (q % KCH) * 8;
-    const int j = k_key[i];                                    // key j of the stage goes to row 8i' + 4h' + r
+    const int j = q / KCH, col = (q % KCH) * 8;                // key j of the stage goes to row 8i' + 4h' + r
     const int row = 8 * (2 * (j / 16) + (j % 8) / 4) + 4 * ((j % 16) / 8) + j % 4;
-    k_dst[i] = row * KP + k_col[i];
-    v_d[i] = q / 4;
-    v_kc[i] = q % 4;
-    v_dst[i] = v_d[i] * VP + v_kc[i] * 8;
+    k_half[i] = j / 16;
+    k_off[i] = (j % 16) * D + col;
+    k_dst[i] = row * KP + col;
+    const int vd = HALVES ? tid / 2 : tid / 4, vkc = HALVES ? 2 * i + tid % 2 : tid % 4;   // dim, chunk of 8 keys
+    v_half[i] = vkc / 2;
+    v_off[i] = vd * P + 8 * (vkc % 2);
+    v_dst[i] = vd * VP + vkc * 8;
   }
   // the row of this lane's column: position c / rows_per_pos of the tile, head c % rows_per_pos of the group
   const int pi = c / tm.rows_per_pos, hi = c % tm.rows_per_pos;
@@ -586,12 +591,17 @@ __global__ void __launch_bounds__(256) attn_prefill_wide_kernel(AttnArgs a) {
       const int64_t pg0 = (int64_t)__builtin_amdgcn_readfirstlane(pg_lds[i0]) * page_stride;
       const int64_t pg1 = (int64_t)__builtin_amdgcn_readfirstlane(pg_lds[i1]) * page_stride;
       const int off0 = kb % P, off1 = (kb + 16) % P;
+      const bf16_t* kh[2] = {kbase + pg0 + (int64_t)off0 * D, kbase + pg1 + (int64_t)off1 * D};   // the halves' first keys
+      const bf16_t* vh[2] = {vbase + pg0 + off0, vbase + pg1 + off1};
 #pragma unroll
       for (int i = 0; i < ROUNDS; ++i) {
-        const bool hi16 = k_key[i] >= 16;
-        r.k[i] = load8(kbase + (hi16 ? pg1 : pg0) + (int64_t)((hi16 ? off1 - 16 : off0) + k_key[i]) * D + k_col[i]);
-        const bool vhi = v_kc[i] >= 2;
-        r.v[i] = load8(vbase + (vhi ? pg1 : pg0) + (int64_t)v_d[i] * P + (vhi ? off1 : off0) + 8 * (v_kc[i] % 2));
+        if constexpr (HALVES) {
+          r.k[i] = load8(kh[i] + (uint32_t)k_off[i]);
+          r.v[i] = load8(vh[i] + (uint32_t)v_off[i]);
+        } else {
+          r.k[i] = load8((k_half[i] ? kh[1] : kh[0]) + (uint32_t)k_off[i]);
+          r.v[i] = load8((v_half[i] ? vh[1] : vh[0]) + (uint32_t)v_off[i]);
+        }
       }
     };
     auto stash = [&](int buf, const Regs& r) {
@@ -606,10 +616,17 @@ __global__ void __launch_bounds__(256) attn_prefill_wide_kernel(AttnArgs a) {
         f32x16_t sc;
 #pragma unroll
         for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+        bf16x8_t kf[D / 16];                       // all of a stage's key fragments are asked for at once
 #pragma unroll
-        for (int ds = 0; ds < D / 16; ++ds) {
-          const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(&k_lds[buf][c * KP + ds * 16 + 8 * h]);
-          sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ds], sc, 0, 0, 0);
+        for (int ds = 0; ds < D / 16; ++ds)
+          kf[ds] = *reinterpret_cast<const bf16x8_t*>(&k_lds[buf][c * KP + ds * 16 + 8 * h]);
+#pragma unroll
+        for (int ds = 0; ds < D / 16; ++ds) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds], qf[ds], sc, 0, 0, 0);
+        bf16x8_t vf[D / 32][2];                    // and its value fragments before the softmax that they wait for
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db) {
+          vf[db][0] = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(db * 32 + c) * VP + 8 * h]);
+          vf[db][1] = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(db * 32 + c) * VP + 16 + 8 * h]);
         }
         // value idx = 4i + r of this lane is key kb + 16*(i/2) + 8h + 4*(i%2) + r against query column c
         const int first = a.window > 0 ? qpos - a.window + 1 : 0;
@@ -628,7 +645,10 @@ __global__ void __launch_bounds__(256) attn_prefill_wide_kernel(AttnArgs a) {
         float mx = sv[0];
 #pragma unroll
         for (int idx = 1; idx < 16; ++idx) mx = fmaxf(mx, sv[idx]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        {                                          // the other half of the keys is in lane l ^ 32
+          const auto halves = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+          mx = fmaxf(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
+        }
         const float m_new = fmaxf(m, mx * a.scale_log2);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
         bf16x8_t pb0, pb1;
@@ -649,10 +669,8 @@ __global__ void __launch_bounds__(256) attn_prefill_wide_kernel(AttnArgs a) {
         l += psum;
 #pragma unroll
         for (int db = 0; db < D / 32; ++db) {
-          const bf16x8_t vf0 = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(db * 32 + c) * VP + 8 * h]);
-          const bf16x8_t vf1 = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(db * 32 + c) * VP + 16 + 8 * h]);
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf0, pb0, o[db], 0, 0, 0);
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf1, pb1, o[db], 0, 0, 0);
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][0], pb0, o[db], 0, 0, 0);
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][1], pb1, o[db], 0, 0, 0);
         }
       }
       stash(buf ^ 1, next);
