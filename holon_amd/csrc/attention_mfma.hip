@@ -78,8 +78,12 @@ __device__ __forceinline__ bf16x8_t softmax_block(const f32x4_t& s0, const f32x4
     }
   }
   float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-  mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+  {   // over the four lane groups: the swaps leave lane l's value beside that of lane l ^ 16, then of lane l ^ 32
+    const auto rows = __builtin_amdgcn_permlane16_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+    mx = fmaxf(__uint_as_float(rows[0]), __uint_as_float(rows[1]));
+    const auto halves = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+    mx = fmaxf(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
+  }
   const float m_new = fmaxf(m, mx * scale_log2);          // (scale > 0: the largest raw score is the largest scaled one)
   const float m_use = m_new == -INFINITY ? 0.f : m_new;   // nothing visible yet: keep everything at zero
   bf16x8_t pb;
