@@ -174,7 +174,7 @@ def main(argv: list[str] | None = None) -> int:
             pms, _ = decode(b, min(a.steps, 32), min(a.warmup, 4))
             points[f"decode_b{b}"] = round(b / (pms * 1e-3), 1)
     line = {
-        "metric": "decode tok/s at batch 8 (context 4,096), Qwen3-8B shape", "value": round(a.batch / (ms * 1e-3), 1),
+        "metric": f"decode tok/s at batch {a.batch} (context 4,096), Qwen3-8B shape", "value": round(a.batch / (ms * 1e-3), 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
         "data": "synthetic (random weights, uniform random token ids)",
