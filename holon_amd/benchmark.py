@@ -171,7 +171,7 @@ def main(argv: list[str] | None = None) -> int:
     points = {}
     if not a.no_points:
         for b in (1, 64):
-            pms, _ = decode(b, min(a.steps, 32), min(a.warmup, 4))
+            pms, _ = decode(b, a.steps, a.warmup)
             points[f"decode_b{b}"] = round(b / (pms * 1e-3), 1)
     line = {
         "metric": f"decode tok/s at batch {a.batch} (context 4,096), Qwen3-8B shape", "value": round(a.batch / (ms * 1e-3), 1),
