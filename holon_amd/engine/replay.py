@@ -19,19 +19,26 @@ class Replayer:
     def step(self, entries: list[dict], end: list[str] = ()) -> torch.Tensor | None:
         """`entries`: [{"id", "tokens", "want"}]; returns float32 logits [wanted, vocab] in the order of the entries
         and of each `want`, or None when nothing is wanted. Requests in `end` give back what they hold afterwards."""
-        rows = []
-        for e in entries:
-            rid, tokens = str(e["id"]), list(e["tokens"])
-            if rid not in self.slots:
-                slot = self.cache.admit()
-                if slot is None:
-                    raise RuntimeError(f"request {rid}: all {self.cache.max_seqs} slots are taken")
-                self.slots[rid], self.fed[rid] = slot, 0
-            slot, start = self.slots[rid], self.fed[rid]
-            if not self.cache.reserve(slot, start + len(tokens)):
-                raise RuntimeError(f"request {rid}: the cache has no pages left for {start + len(tokens)} tokens")
-            rows.append(StepRow(slot, start, tokens, list(e.get("want", []))))
-        logits = self.runner.run(rows) if rows else None
+        rows, admitted = [], []
+        try:
+            for e in entries:
+                rid, tokens = str(e["id"]), list(e["tokens"])
+                if rid not in self.slots:
+                    slot = self.cache.admit()
+                    if slot is None:
+                        raise RuntimeError(f"request {rid}: all {self.cache.max_seqs} slots are taken")
+                    self.slots[rid], self.fed[rid] = slot, 0
+                    admitted.append(rid)
+                slot, start = self.slots[rid], self.fed[rid]
+                if not self.cache.reserve(slot, start + len(tokens)):
+                    raise RuntimeError(f"request {rid}: the cache has no pages left for {start + len(tokens)} tokens")
+                rows.append(StepRow(slot, start, tokens, list(e.get("want", []))))
+            logits = self.runner.run(rows) if rows else None
+        except Exception:
+            for rid in admitted:                   # a refused step leaves no request behind that it brought
+                self.cache.release(self.slots.pop(rid))
+                del self.fed[rid]
+            raise
         for e in entries:
             self.fed[str(e["id"])] += len(e["tokens"])
         for rid in end:

@@ -177,3 +177,21 @@ def test_the_trace_run_program(folders, tmp_path, dtype):
             got.update(zip(expect, rows))
     assert len(got) == sum(map(len, requests.values())) - len(dropped)
     _check(folder, dtype, requests, got, f"trace_run {dtype}")
+
+
+def test_a_refused_step_leaves_nothing_behind(folders):
+    """Steps that the step function refuses (no tokens, a wanted place beyond the tokens, a token outside the
+    vocabulary, a request longer than the model length, a request twice in a step) raise, and a request that such a
+    step brought holds neither a slot nor a page afterwards."""
+    rep = _replayer(folders["A"], "A", "cpu", "float32", cache_tokens=128, max_model_len=128)
+    assert rep.step([{"id": "a", "tokens": [1, 2, 3], "want": []}]) is None          # nothing wanted: no logits
+    free = [g.pool.free for g in rep.cache.groups]
+    for bad in ([{"id": "c", "tokens": [], "want": []}], [{"id": "c", "tokens": [1, 2], "want": [2]}],
+                [{"id": "c", "tokens": [999], "want": [0]}], [{"id": "c", "tokens": [1] * 200, "want": [0]}],
+                [{"id": "c", "tokens": [1, 2], "want": [0]}, {"id": "c", "tokens": [3], "want": [0]}]):
+        with pytest.raises((ValueError, RuntimeError)):
+            rep.step(bad)
+        assert set(rep.slots) == {"a"} and [g.pool.free for g in rep.cache.groups] == free
+        rep.cache.check()
+    assert rep.step([{"id": "a", "tokens": [4], "want": [0]}], end=["a"]).shape == (1, 256)
+    assert all(g.pool.free == g.pool.usable for g in rep.cache.groups) and rep.cache.free_slots == rep.cache.max_seqs
