@@ -888,12 +888,11 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
   return 0;
 }
 
-extern "C" int holon_attention_decode_bf16(const void* q, void* out, const void* pages, const int32_t* table,
-                                           int table_stride, const int32_t* slots, const int32_t* lens,
-                                           const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
-                                           int heads, int kv_heads, int head_dim, int page_size, float scale,
-                                           int window, float* part_o, float* part_ml, int splits, int keys_per_split,
-                                           void* stream) {
+// The decode launch both entry points share: the split kernel, then the ordered merge.
+static int decode_launch(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
+                         const int32_t* slots, const int32_t* lens, const int32_t* query_start, const int32_t* row_ids,
+                         int n_rows, int max_len, int heads, int kv_heads, int head_dim, int page_size, float scale,
+                         int window, float* part_o, float* part_ml, int splits, int keys_per_split, void* stream) {
   HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
@@ -926,4 +925,14 @@ extern "C" int holon_attention_decode_bf16(const void* q, void* out, const void*
     attn_merge_kernel<256><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits);
   HOLON_LAUNCH_OK();
   return 0;
+}
+
+extern "C" int holon_attention_decode_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                           int table_stride, const int32_t* slots, const int32_t* lens,
+                                           const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
+                                           int heads, int kv_heads, int head_dim, int page_size, float scale,
+                                           int window, float* part_o, float* part_ml, int splits, int keys_per_split,
+                                           void* stream) {
+  return decode_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len, heads,
+                       kv_heads, head_dim, page_size, scale, window, part_o, part_ml, splits, keys_per_split, stream);
 }
