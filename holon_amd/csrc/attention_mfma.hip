@@ -16,6 +16,8 @@
 //   O^T = V^T P^T: A = 16 dims x 32 keys straight from a value page (values are stored transposed inside a page, so the
 //     8 keys a lane needs are one 16-byte load), B = P^T from the registers above, rounded to bfloat16.
 // Softmax is online, float32, in base 2 with log2(e) folded into the scale.
+#include <mutex>
+
 #include "common.h"
 #include "holon_hip.h"
 
@@ -935,4 +937,64 @@ extern "C" int holon_attention_decode_bf16(const void* q, void* out, const void*
                                            void* stream) {
   return decode_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len, heads,
                        kv_heads, head_dim, page_size, scale, window, part_o, part_ml, splits, keys_per_split, stream);
+}
+
+// ---- decode attention for callers that cannot allocate ------------------------------------------------------------
+// The split partials live in a file-scope device array instead of a workspace the caller brings. Each GPU holds its own
+// copy of the array at its own address, which is looked up once per device; host code uses that address and never the
+// array's name. Nothing in it has to start at zero: the merge reads only partials that the split kernel of the same
+// call wrote (an empty split writes a weight of zero, and its values are then dropped unread). Every call on a GPU
+// shares that GPU's array, so two calls that overlap on one GPU (two streams, two threads) race on it.
+static __device__ __align__(256) float scratch[HOLON_DECODE_SCRATCH_BYTES / sizeof(float)];
+
+static constexpr int kMaxDevices = 64;
+static float* g_scratch[kMaxDevices];          // per device: where that device's copy of `scratch` lies
+static std::mutex g_scratch_lock;
+
+// The current device's copy of the array, looked up at the first call on that device.
+static int decode_scratch(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  HOLON_CHECK(e == hipSuccess, "attention decode (static): hipGetDevice: %s", hipGetErrorString(e));
+  HOLON_CHECK(dev >= 0 && dev < kMaxDevices, "attention decode (static): device %d beyond the %d this library tracks",
+              dev, kMaxDevices);
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (g_scratch[dev] == nullptr) {
+    void* found = nullptr;
+    e = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    HOLON_CHECK(e == hipSuccess && found != nullptr, "attention decode (static): hipGetSymbolAddress: %s",
+                hipGetErrorString(e));
+    g_scratch[dev] = (float*)found;
+  }
+  *ptr = g_scratch[dev];
+  return 0;
+}
+
+extern "C" int holon_decode_scratch_init(void) {
+  float* ptr = nullptr;
+  return decode_scratch(&ptr);
+}
+
+extern "C" int64_t holon_decode_scratch_bytes(void) { return HOLON_DECODE_SCRATCH_BYTES; }
+
+extern "C" int holon_attention_decode_bf16_static(const void* q, void* out, const void* pages, const int32_t* table,
+                                                  int table_stride, const int32_t* slots, const int32_t* lens,
+                                                  const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                                  int max_len, int heads, int kv_heads, int head_dim, int page_size,
+                                                  float scale, int window, int splits, int keys_per_split,
+                                                  void* stream) {
+  HOLON_CHECK(n_rows >= 0 && heads > 0 && splits > 0 && head_dim > 0, "attention decode (static): bad sizes");
+  // part_o [n_rows, heads, splits, head_dim] then part_ml [n_rows, heads, splits, 2], the second on a 256-byte edge
+  const int64_t cells = (int64_t)n_rows * heads * splits;
+  const int64_t o_floats = (cells * head_dim + 63) / 64 * 64;
+  const int64_t need = (o_floats + cells * 2) * (int64_t)sizeof(float);
+  HOLON_CHECK(need <= HOLON_DECODE_SCRATCH_BYTES,
+              "attention decode (static): %d rows x %d heads x %d splits of head_dim %d need %lld bytes of partials; the "
+              "built-in buffer holds %lld (use holon_attention_decode_bf16 with a workspace of your own)",
+              n_rows, heads, splits, head_dim, (long long)need, (long long)HOLON_DECODE_SCRATCH_BYTES);
+  float* base = nullptr;
+  if (decode_scratch(&base) != 0) return -1;
+  return decode_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len, heads,
+                       kv_heads, head_dim, page_size, scale, window, base, base + o_floats, splits, keys_per_split,
+                       stream);
 }

@@ -46,6 +46,22 @@ int holon_attention_decode_bf16(const void* q, void* out, const void* pages, con
                                 const int32_t* row_ids, int n_rows, int max_len, int heads, int kv_heads, int head_dim,
                                 int page_size, float scale, int window, float* part_o, float* part_ml, int splits,
                                 int keys_per_split, void* stream);
+// The same decode attention for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+// loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. The split partials that
+// holon_attention_decode_bf16 takes as a workspace live in a device array inside the library instead, of
+// HOLON_DECODE_SCRATCH_BYTES on every GPU the library runs on, held until the process ends; no call allocates or frees.
+// n_rows * heads * splits * (head_dim + 2) floats (the first part rounded up to 256 bytes) must fit, or the call is
+// refused. All calls on one GPU share that GPU's array: calls that overlap on one GPU (other streams, other threads)
+// race; calls in one stream's order do not. holon_decode_scratch_init() looks the array's address up for the current
+// device ahead of time (the entry point does it at its first call on a device otherwise).
+#define HOLON_DECODE_SCRATCH_BYTES (16 << 20)
+int holon_decode_scratch_init(void);
+int64_t holon_decode_scratch_bytes(void);
+int holon_attention_decode_bf16_static(const void* q, void* out, const void* pages, const int32_t* table,
+                                       int table_stride, const int32_t* slots, const int32_t* lens,
+                                       const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
+                                       int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
+                                       int splits, int keys_per_split, void* stream);
 // y[M, N] = x[M, K] w[N, K]^T for M <= 64 rows, bfloat16 in, float32 accumulation; out_f32 picks the output type;
 // tiled says that `w` is holon_tile_weight_bf16's copy ([N/16, K/32, 64, 8]: lane-major 16-byte pieces).
 int holon_gemm_skinny_supported(int M, int N, int K);
