@@ -28,7 +28,7 @@ def rope_angles(positions: torch.Tensor, head_dim: int, theta: float) -> tuple[t
     """cos and sin of position * theta^(-2i/D), i < D/2, all float32.
     std/holon_std/ops/reference.py:24-26."""
     inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
-    angles = positions.to(torch.float32)[:, None] * inv_freq[None, :]
+    angles = positions.to(torch.float32)[:, None] * inv_freq.to(positions.device)[None, :]
     return angles.cos(), angles.sin()
 
 
@@ -51,7 +51,7 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: 
     k32 = k.float().repeat_interleave(group, dim=1)
     v32 = v.float().repeat_interleave(group, dim=1)
     scores = torch.einsum("qhd,khd->hqk", q.float(), k32) / d ** 0.5
-    pos = torch.arange(t)
+    pos = torch.arange(t, device=q.device)
     hidden = pos[None, :] > pos[:, None]
     if window:
         hidden = hidden | (pos[:, None] - pos[None, :] >= window)
@@ -117,8 +117,9 @@ def logits_of(ids: list[int], w: dict[str, torch.Tensor], cfg: dict) -> torch.Te
     """Float32 logits [T, V] of every token of one sequence.
     core/holon/core/build.py:296-307 (embed, blocks, final norm, head); std/holon_std/ops/units.py:345-348 (head reads
     the embedding when tied; logits are float32)."""
-    h = w["model.embed_tokens.weight"][torch.tensor(ids, dtype=torch.long)]
-    positions = torch.arange(len(ids))
+    table = w["model.embed_tokens.weight"]
+    h = table[torch.tensor(ids, dtype=torch.long, device=table.device)]
+    positions = torch.arange(len(ids), device=table.device)
     for i in range(cfg["num_hidden_layers"]):
         h = block(h, positions, w, i, cfg)
     h = rms_norm(h, w["model.norm.weight"], cfg["rms_norm_eps"])
@@ -126,22 +127,24 @@ def logits_of(ids: list[int], w: dict[str, torch.Tensor], cfg: dict) -> torch.Te
     return linear(h, head).float()
 
 
-def read_folder(folder: str | pathlib.Path, dtype: torch.dtype = torch.float32) -> tuple[dict, dict[str, torch.Tensor]]:
-    """config.json as a dict, and every tensor of model.safetensors by its stored name, cast to `dtype`."""
+def read_folder(folder: str | pathlib.Path, dtype: torch.dtype = torch.float32, device: str = "cpu"
+                ) -> tuple[dict, dict[str, torch.Tensor]]:
+    """config.json as a dict, and every tensor of model.safetensors by its stored name, cast to `dtype`. `device`:
+    where the same plain functions run (a test of a wide model may put them on the GPU to be done in seconds)."""
     folder = pathlib.Path(folder)
     cfg = json.loads((folder / "config.json").read_text())
     weights = {}
     with safe_open(str(folder / "model.safetensors"), "pt", device="cpu") as f:
         for name in f.keys():
-            weights[name] = f.get_tensor(name).to(dtype)
+            weights[name] = f.get_tensor(name).to(dtype).to(device)
     return cfg, weights
 
 
 class PlainQwen3:
     """The plain model of one folder: `logits(ids)` for a whole sequence, `greedy(ids, n)` by recomputing it."""
 
-    def __init__(self, folder: str | pathlib.Path, dtype: torch.dtype = torch.float32) -> None:
-        self.cfg, self.weights = read_folder(folder, dtype)
+    def __init__(self, folder: str | pathlib.Path, dtype: torch.dtype = torch.float32, device: str = "cpu") -> None:
+        self.cfg, self.weights = read_folder(folder, dtype, device)
 
     @torch.no_grad()
     def logits(self, ids: list[int]) -> torch.Tensor:

@@ -141,6 +141,31 @@ def test_paged_attention(hip, dtype, page, geometry):
         assert H.op_budget_usage(got, want, dtype, head_dim + max(s + n for s, n in rows)) <= 1, (geometry, page, rows)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geometry", [(32, 8, 128), (8, 2, 64)])
+def test_sixty_four_decode_rows(hip, dtype, geometry):
+    """A decode step of 64 rows of unequal lengths (one key to 4,096, on and off page edges), with the launch shaped
+    for a longer row than any has (as a graph's length bucket shapes it), and again with 11 of the rows empty rows on
+    a table row of one page (as a graph's padding rows are)."""
+    heads, kv_heads, head_dim = geometry
+    rng = np.random.default_rng(5)
+    longest = 4095 if head_dim == 64 else 1030
+    rows = [(int(n), 1) for n in rng.integers(0, longest, 60)] + [(0, 1), (15, 1), (16, 1), (longest, 1)]
+    q, pages, table, attn = _paged_case(rows, heads, kv_heads, head_dim, 16, dtype, seed=9, max_seqs=64)
+    scale = head_dim ** -0.5
+    want = PLAIN.paged_attention(q.double(), pages.double(), table, attn, 16, scale, 0)
+    got = hip.paged_attention(q, pages, table, attn, 16, scale, 0)
+    assert H.op_budget_usage(got, want, dtype, head_dim + longest) <= 1
+    attn.max_decode_len = 1 << (longest).bit_length()                   # the bucket's length, not the rows'
+    assert H.op_budget_usage(hip.paged_attention(q, pages, table, attn, 16, scale, 0), want, dtype,
+                             head_dim + longest) <= 1
+    lens = attn.lens.clone()
+    lens[53:] = 0                                                       # rows that hold nothing give zeros
+    attn.lens = lens
+    got = hip.paged_attention(q, pages, table, attn, 16, scale, 0)
+    assert not got[53:].any() and H.op_budget_usage(got[:53], want[:53], dtype, head_dim + longest) <= 1
+
+
 @pytest.mark.parametrize("geometry", [(32, 8, 128), (16, 8, 64), (8, 1, 128), (7, 7, 64), (6, 2, 64), (5, 1, 128),
                                       (24, 1, 64), (32, 1, 128), (40, 1, 128), (66, 1, 64), (80, 2, 64)])
 def test_long_prompt_portions_two_tiles_a_wave(hip, geometry):

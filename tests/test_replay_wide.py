@@ -26,8 +26,14 @@ def folder(tmp_path_factory):
 
 
 @functools.lru_cache(maxsize=None)
+def _plain(folder: str, dtype: str) -> PlainQwen3:
+    """The plain model's own functions, run on the GPU: at these widths the CPU needs minutes for them."""
+    return PlainQwen3(folder, getattr(torch, dtype), device="cuda")
+
+
+@functools.lru_cache(maxsize=None)
 def _plain_logits(folder: str, dtype: str, ids: tuple[int, ...]) -> torch.Tensor:
-    return PlainQwen3(folder, getattr(torch, dtype)).logits(list(ids))
+    return _plain(folder, dtype).logits(list(ids)).cpu()
 
 
 def _requests():
@@ -67,6 +73,105 @@ def test_wide_layers_every_way_of_cutting(folder, dtype):
     _check(folder, dtype, requests, got, f"wide {dtype} mixed")
     rep.cache.check()
     assert all(g.pool.free == g.pool.usable for g in rep.cache.groups)
+
+
+def _wide_batch_requests() -> dict[str, tuple[list[int], int]]:
+    """64 requests as (token ids, prompt length): the rest of each is decoded one token a step, all together. The
+    decode counts make the batch shrink 64 -> 45 -> 30 -> 20 -> 12 -> 7 (padded to 48, 32, 24, 16, 8); request `long` goes from 2,042 to 2,062 tokens
+    (the longest row crosses 2,048 while 64 rows decode) and leaves after 20 steps; request `mid` goes from 990 to
+    1,050, so that the longest row crosses 1,024 while 8 rows decode. Prompt lengths sit on and around page edges."""
+    decodes = [60] * 6 + [8] * 19 + [14] * 15 + [20] * 9 + [26] * 8 + [32] * 5
+    prompts = [1, 2, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 100, 127, 128, 129, 255, 256, 257, 300]
+    out = {}
+    for i, d in enumerate(decodes):         # the first slots go to short requests that stay to the end: what a padding
+        p = prompts[(7 * i) % len(prompts)]  # row wrongly wrote there would be one of their few keys
+        out[f"s{i}"] = (H.random_ids(p + d, WIDE["vocab_size"], 1000 + i), p)
+    out["long"] = (H.random_ids(2042 + 20, WIDE["vocab_size"], 900), 2042)
+    out["mid"] = (H.random_ids(990 + 60, WIDE["vocab_size"], 901), 990)
+    assert len(out) == 64
+    return out
+
+
+def _wide_batch_trace(requests: dict[str, tuple[list[int], int]], budget: int) -> H.Trace:
+    """Prompts first, several to a step under `budget` tokens, their last logits wanted; then every live request's
+    next token in one step, every row's logits wanted, until all are done."""
+    t = H.Trace()
+    entries, used = [], 0
+    for rid, (ids, p) in requests.items():
+        if used + p > budget:
+            t.add(entries)
+            entries, used = [], 0
+        entries.append((rid, 0, ids[:p], [p - 1]))
+        used += p
+    t.add(entries)
+    at = {rid: p for rid, (_, p) in requests.items()}
+    while at:
+        entries = [(rid, pos, [requests[rid][0][pos]], [0]) for rid, pos in at.items()]
+        end = [rid for rid, pos in at.items() if pos + 1 == len(requests[rid][0])]
+        t.add(entries, end)
+        at = {rid: pos + 1 for rid, pos in at.items() if rid not in end}
+    return t
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sixty_four_rows_decode_together_from_graphs(folder, dtype):
+    """Decode steps of 64 rows shrinking to 7, replayed from graphs of every batch bucket on the way (all but the
+    first with padding rows) and of three length buckets (1,024, 2,048, 4,096): the vendor product for more
+    than 16 rows, the decode attention with 64 rows, the few-row kernels below. Every row's logits in every step
+    against the plain model."""
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    requests = _wide_batch_requests()
+    trace = _wide_batch_trace(requests, 2304)
+    loaded = load_model(folder, device="cuda", dtype=dtype, page_size=16, max_seqs=64, max_model_len=2304,
+                        max_step_tokens=2304, cache_tokens=H.peak_live_tokens(trace), graphs=True)
+    rep = Replayer(loaded)
+    got = H.run_trace(rep, trace)
+    assert len(got) == 64 + sum(len(ids) - p for ids, p in requests.values())
+    keys = set(loaded.runner.graphs)
+    assert {(64, 2048), (64, 4096), (48, 4096), (32, 4096), (24, 1024), (16, 1024), (8, 1024), (8, 2048)} <= keys, keys
+    assert loaded.runner.graph_replays >= 40
+    _check(folder, dtype, {rid: ids for rid, (ids, _) in requests.items()}, got, f"wide {dtype} 64 rows")
+    rep.cache.check()
+    assert all(g.pool.free == g.pool.usable for g in rep.cache.groups)
+
+
+def _greedy_follows_the_plain_model(plain, prompt, got, margin=0.05) -> None:
+    """Every generated token is the plain model's most likely one given the tokens before it, wherever the plain
+    model's two best logits are further apart than bfloat16 rounding reaches."""
+    ids = list(prompt)
+    for token in got:
+        logits = plain.logits(ids)[-1].float()
+        top = logits.topk(2).values
+        if float(top[0] - top[1]) > margin * float(logits.std()):
+            assert token == int(logits.argmax()), (len(ids), token)
+        ids.append(token)
+
+
+def test_engine_at_the_wide_sizes_with_everything_on(folder):
+    """The whole engine in bfloat16 at the measured layer sizes (matrix-core attention, the few-row products over
+    tiled weights, the residual add and the gated form inside them). One step in flight changes no launch, so it must
+    change no token, greedy or seeded. Graph replay shapes the decode attention for its length bucket (other splits
+    of the keys, other roundings) and shared prefixes cut the prompts elsewhere, and 20 requests make steps of more
+    than 16 rows: there the greedy tokens are held to the plain model's own greedy decoding in bfloat16."""
+    from holon_amd.config import EngineConfig, SamplingParams
+    from holon_amd.engine.engine import Engine
+    start = H.random_ids(40, WIDE["vocab_size"], 300)
+    prompts = [start[: 8 + 4 * (i % 9)] + H.random_ids(3 + 5 * i, WIDE["vocab_size"], 301 + i) for i in range(20)]
+    shape = dict(model=str(folder), device="cuda", dtype="bfloat16", page_size=16, max_seqs=24, max_model_len=256,
+                 max_step_tokens=256, cache_tokens=24 * 256)
+    bare = Engine(EngineConfig(overlap=False, graphs=False, prefix_cache=False, **shape))
+    ahead = Engine(EngineConfig(overlap=True, graphs=False, prefix_cache=False, **shape))
+    for params in (SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True),
+                   SamplingParams(temperature=0.8, top_k=40, top_p=0.95, seed=5, max_tokens=24, ignore_eos=True)):
+        assert ahead.generate(prompts, params) == bare.generate(prompts, params)
+    full = Engine(EngineConfig(overlap=True, graphs=True, prefix_cache=True, **shape))
+    plain = _plain(str(folder), "bfloat16")
+    params = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
+    for _ in range(2):                                           # the second time the prompts come from the cache
+        for prompt, got in zip(prompts, full.generate(prompts, params)):
+            _greedy_follows_the_plain_model(plain, prompt, got)
+    assert full.cache.tokens_saved > 0 and full.stats()["graphs"] >= 1 and full.runner.graph_replays > 10
 
 
 def test_long_context_attention_kernels():
