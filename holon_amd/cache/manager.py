@@ -1,10 +1,12 @@
 """The cache manager: slots, paged groups with block tables, and fixed-size per-request state.
 
 A request is given a *slot* when it is admitted: its row in every block table and in every fixed-size state tensor.
-State that grows lives in pages. Runs of the model whose mixers declare equal `PagedState`s form a *group*: one page
-pool, one block table, one storage tensor `[sites, pages, page_size * elems]` — page id p means row p of every site of
-the group. Groups with different needs (all tokens, a window of them) have pools of their own; a windowed group gives
-pages back as soon as the window has passed them, a finished request gives back everything.
+State that grows lives in pages. Paged states of equal page geometry (values per token, window, dtype), whichever runs
+declare them and however many one run declares, form a *group*: one page pool, one block table, one storage tensor
+`[members, pages, page_size * elems]` with a member for every (run, state name) of the group. Page id p means row p
+of every member. Groups with different needs (all tokens, a window of them, another width) have pools and tables of
+their own; a windowed group gives pages back as soon as the window has passed them, a finished request gives back
+everything.
 
 With a prefix index (`enable_prefix`) full pages of tokens are shared between requests that start alike: `adopt` gives
 a new request the cached pages of its longest known prefix, `publish` hands the pages a request has filled to the
@@ -21,6 +23,7 @@ import numpy as np
 import torch
 
 from ..parts.base import PagedState, SlotState
+from ..model import SitePages
 from .pool import PagePool
 from .prefix import PrefixIndex
 
@@ -29,9 +32,10 @@ from .prefix import PrefixIndex
 class PagedGroup:
     gid: int
     decl: PagedState                              # with name ignored: elems, window, dtype decide the group
-    sites: list[int]
+    sites: list[int]                              # the runs with a state in this group (a run once)
+    members: list[tuple[int, str]]                # (run, state name) of every row of `storage`
     pool: PagePool
-    storage: torch.Tensor                         # [len(sites), num_pages, page_size * elems]
+    storage: torch.Tensor                         # [len(members), num_pages, page_size * elems]
     table: np.ndarray                             # [max_seqs + 1, max_pages] int32, null page where nothing is held
     table_dev: torch.Tensor
     first: list[int]                              # per slot: first page index still held
@@ -61,34 +65,40 @@ class CacheManager:
         num_pages = -(-tokens // page_size) + 1
         if tokens < 1:
             raise ValueError("the cache needs room for at least one token")
-        keyed: dict[tuple, list[int]] = {}
+        keyed: dict[tuple, list[tuple[int, str]]] = {}
         for site, site_decls in zip(sites, decls, strict=True):
+            names = [d.name for d in site_decls]
+            if len(set(names)) != len(names):
+                raise ValueError(f"run {site.run} declares two states of one name: {names}")
             for d in site_decls:
                 if isinstance(d, PagedState):
-                    if site.group is not None:
-                        raise NotImplementedError("one paged state per run")
                     key = (d.elems, d.window, d.dtype or dtype)
-                    keyed.setdefault(key, []).append(site.run)
-                    site.group = -1
+                    keyed.setdefault(key, []).append((site.run, d.name))
                 elif isinstance(d, SlotState):
                     t = torch.zeros((max_seqs + 1, *d.shape), dtype=d.dtype or dtype, device=device)
                     site.slot_state[d.name] = t
                     self.slot_states.append((site.run, d, t))
                 else:
                     raise TypeError(f"run {site.run}: unknown state declaration {d!r}")
-        for gid, ((elems, window, gdtype), runs) in enumerate(keyed.items()):
+        for gid, ((elems, window, gdtype), members) in enumerate(keyed.items()):
             pool = PagePool(num_pages)
-            storage = torch.zeros((len(runs), num_pages, page_size * elems), dtype=gdtype, device=device)
+            storage = torch.zeros((len(members), num_pages, page_size * elems), dtype=gdtype, device=device)
             table = np.full((max_seqs + 1, self.max_pages), pool.null, dtype=np.int32)
-            group = PagedGroup(gid, PagedState("", elems, window, gdtype), runs, pool, storage, table,
+            runs = sorted({run for run, _ in members})
+            group = PagedGroup(gid, PagedState("", elems, window, gdtype), runs, members, pool, storage, table,
                                torch.from_numpy(table.copy()).to(device), [0] * (max_seqs + 1), [0] * (max_seqs + 1))
             self.groups.append(group)
-            for at, run in enumerate(runs):
-                sites[run].group, sites[run].pages = gid, storage[at]
+            for at, (run, name) in enumerate(members):
+                sites[run].paged[name] = SitePages(gid, storage[at])
+        for site, site_decls in zip(sites, decls):                # `group`, `pages`: the first paged state declared
+            first = next((d.name for d in site_decls if isinstance(d, PagedState)), None)
+            if first is not None:
+                site.group, site.pages = site.paged[first].group, site.paged[first].pages
         for site in sites:                                        # runs that read another run's cache
             if site.owner is not None:
                 owner = sites[site.owner]
-                site.group, site.pages, site.slot_state = owner.group, owner.pages, owner.slot_state
+                site.group, site.pages, site.paged, site.slot_state = owner.group, owner.pages, owner.paged, \
+                    owner.slot_state
 
     # -- slots ----------------------------------------------------------------------------------------------------
     @property
@@ -261,6 +271,21 @@ class CacheManager:
             if want - have > g.pool.free + freed:
                 return False
         return True
+
+    def victims_needed(self, slot: int, total: int, order: list[int]) -> int | None:
+        """How many of the requests in `order` (slots, the first to give way first) must give back what they hold
+        before `slot` can keep `total` tokens: the shortest start of `order` that makes room. None when not even all
+        of them would."""
+        if not self.could_fit(slot, total, order):
+            return None
+        lo, hi = 0, len(order)                    # room grows with every request that gives way
+        while lo < hi:
+            mid = (lo + hi) // 2
+            if self.could_fit(slot, total, order[:mid]):
+                hi = mid
+            else:
+                lo = mid + 1
+        return lo
 
     def fits_alone(self, total: int) -> bool:
         """Whether an empty cache holds one request of `total` tokens."""

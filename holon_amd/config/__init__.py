@@ -1,5 +1,6 @@
-"""Configuration: the model's (from config.json) and the engine's. Importing this package imports no torch."""
+"""Configuration: the engine's, and what every architecture's own configuration shares. Importing this package
+imports no torch."""
 from .engine import DTYPES, EngineConfig, SamplingParams
-from .model import ConfigError, Qwen3Config, read_config_json
+from .model import ConfigError, read_config_json
 
-__all__ = ["DTYPES", "EngineConfig", "SamplingParams", "ConfigError", "Qwen3Config", "read_config_json"]
+__all__ = ["DTYPES", "EngineConfig", "SamplingParams", "ConfigError", "read_config_json"]

@@ -77,8 +77,12 @@ class Engine:
                 print("holon_amd: this model keeps state that pages do not hold whole; prompts share nothing",
                       file=sys.stderr)
         self.sampler = Sampler(self.kernels, cfg.max_seqs, device)
+        budget = min(cfg.max_step_tokens, cfg.chunk_with_decode or cfg.max_step_tokens)
+        if self.model.cut(0, budget) < 1:
+            raise ValueError(f"no prompt portion of {budget} tokens (max_step_tokens, chunk_with_decode) ends where this "
+                             "model's parts allow a portion to end; raise them")
         self.sched = Scheduler(self.cache, cfg.max_step_tokens, cfg.max_model_len, cfg.chunk_with_decode,
-                               on_admit=self._on_admit)
+                               on_admit=self._on_admit, cut=self.model.cut)
         self._ids = itertools.count()
         self._live: dict[str, list[Seq]] = {}
         self._siblings: dict[Seq, list[Seq]] = {}         # n > 1: waiting until the first sequence's prompt is cached
@@ -166,37 +170,47 @@ class Engine:
         return int(peak * 1.1) + (64 << 20)           # the allocator's rounding and fragmentation
 
     # -- requests -------------------------------------------------------------------------------------------------
+    def _check_prompt(self, token_ids: list[int]) -> None:
+        room = self.cfg.max_model_len - len(token_ids)
+        if not token_ids or room < 1:
+            raise ValueError(f"a prompt has 1 to {self.cfg.max_model_len - 1} tokens (max_model_len "
+                             f"{self.cfg.max_model_len} less one to generate); this one has {len(token_ids)}")
+        bad = [t for t in token_ids if not 0 <= t < self.spec.vocab]
+        if bad:
+            raise ValueError(f"token id {bad[0]} is outside the vocabulary of {self.spec.vocab}")
+
     def add(self, token_ids: list[int], params: SamplingParams | None = None, rid: str | None = None) -> str:
-        p = params or SamplingParams()
-        p.check()
-        if not token_ids:
-            raise ValueError("empty prompt")
-        if len(token_ids) >= self.cfg.max_model_len:
-            raise ValueError(f"prompt of {len(token_ids)} tokens leaves no room under max_model_len "
-                             f"{self.cfg.max_model_len}")
-        if min(token_ids) < 0 or max(token_ids) >= self.spec.vocab:
-            raise ValueError(f"token ids must lie in [0, {self.spec.vocab})")
-        rid = rid if rid is not None else str(next(self._ids))
+        """Queue a prompt; returns the request's id. `params.n` sequences are drawn for it, each with a seed of its
+        own derived from the request's (core/holon/core/engine.py:332-376): what a sequence draws depends on its
+        seed and positions alone. With shared prefixes only the first sequence is queued now; the others follow when
+        its prompt is in the cache, and start from there."""
+        params = params if params is not None else SamplingParams()
+        params.check()
+        self._check_prompt(token_ids)
+        if rid is None:
+            rid = str(next(self._ids))
         if rid in self._live:
             raise ValueError(f"request id {rid!r} is already in flight")
-        base = p.seed if p.seed is not None else secrets.randbits(63)
-        for i in range(p.n):                # a concrete seed per sequence: its draws depend on nothing else
-            child = dataclasses.replace(p, seed=sequence_seed(base, i),
-                                        prompt_logprobs=p.prompt_logprobs if i == 0 else None)
-            seq = Seq(rid=rid, tokens=list(token_ids), params=child, index=i)
-            self._live.setdefault(rid, []).append(seq)
-            if child.prompt_logprobs is not None:         # every position computed, in portions whose logits stay small
-                seq.share_prefix, seq.portion_cap = False, PROMPT_LOGPROB_PORTION
-                self._prompt_lp[seq] = Logprobs([], [], [])
-            if i == 0 or self.cache.prefix is None:
+        seed = secrets.randbits(63) if params.seed is None else params.seed
+        seqs = [Seq(rid=rid, tokens=list(token_ids), index=i,
+                    params=dataclasses.replace(params, seed=sequence_seed(seed, i),
+                                               prompt_logprobs=params.prompt_logprobs if i == 0 else None))
+                for i in range(params.n)]
+        self._live[rid] = seqs
+        head = seqs[0]
+        if head.params.prompt_logprobs is not None:      # every position computed, in portions whose logits stay small
+            head.share_prefix, head.portion_cap = False, PROMPT_LOGPROB_PORTION
+            self._prompt_lp[head] = Logprobs([], [], [])
+        self.sched.add(head)
+        if self.cache.prefix is not None and len(seqs) > 1:
+            self._siblings[head] = seqs[1:]
+        else:
+            for seq in seqs[1:]:
                 self.sched.add(seq)
-                first = seq
-            else:                                         # siblings start from the first sequence's cached prompt
-                self._siblings.setdefault(first, []).append(seq)
         return rid
 
     def has_work(self) -> bool:
-        return bool(self.sched.waiting or self.sched.running or self._inflight is not None)
+        return len(self.sched) > 0 or self._inflight is not None
 
     def idle_for(self) -> float | None:
         """How long a serving loop may wait for new requests before its next `step`: 0 while a request can run, None
@@ -204,23 +218,25 @@ class Engine:
         return 0.0 if self.has_work() else None
 
     def abort(self, rid: str, reason: str = "abort") -> list[TokenDelta]:
-        """Finish every sequence of request `rid` now: one delta each, siblings that never started included."""
-        deltas = []
-        for seq in self._live.pop(rid, []):
-            for sibling in self._siblings.pop(seq, []):
-                sibling.status = Status.FINISHED
-                deltas.append(TokenDelta(rid, [], reason, index=sibling.index))
+        """End request `rid` now. One closing delta for each of its sequences that had not finished, whether it ran,
+        waited in line or had not been queued yet."""
+        seqs = self._live.pop(rid, [])
+        held_back = [s for seq in seqs for s in self._siblings.pop(seq, [])]
+        closing = []
+        for seq in seqs:
             if seq.status is Status.FINISHED:
                 continue
-            self.sched.finish(seq, reason)
+            if seq in held_back:
+                seq.status, seq.finish_reason = Status.FINISHED, reason
+            else:
+                self.sched.retire(seq, reason)
             self._prompt_lp.pop(seq, None)
-            deltas.append(TokenDelta(rid, [], reason, index=seq.index))
-        if not (self.sched.waiting or self.sched.running):      # only dropped rows are in flight: nothing to wait for later
-            deltas += self.drain()
-        return deltas
+            closing.append(TokenDelta(rid, [], reason, index=seq.index))
+        closing.sort(key=lambda d: d.index)
+        return closing + self._settle()
 
     def stats(self) -> dict[str, int]:
-        return {"waiting": len(self.sched.waiting), "running": len(self.sched.running),
+        return {"waiting": len(self.sched) - self.sched.n_running, "running": self.sched.n_running,
                 "preemptions": self.sched.preemptions, "mixed_steps": self.sched.mixed_steps, "steps": self.steps,
                 "free_pages": min((g.pool.free for g in self.cache.groups), default=0),
                 "graphs": len(getattr(self.runner, "graphs", {})),
@@ -238,21 +254,24 @@ class Engine:
         self._live.clear()
 
     def generate(self, prompts: list[list[int]], params: SamplingParams | None = None) -> list[list[int]]:
-        """Token ids generated for each prompt (one sequence per prompt)."""
+        """Run the prompts to their end; the generated token ids of each, in the prompts' order."""
         if params is not None and params.n != 1:
             raise ValueError("generate() returns one sequence per prompt; step() streams n > 1")
-        rids = [self.add(p, params) for p in prompts]
-        out: dict[str, list[int]] = {r: [] for r in rids}
-        pending = set(rids)
-        while pending:
-            for d in self.step():
-                if d.rid in out:
-                    out[d.rid].extend(d.token_ids)
-                    if d.finish_reason:
-                        pending.discard(d.rid)
-        if not (self.sched.waiting or self.sched.running):      # rows of requests that finished meanwhile: dropped
-            self.drain()
-        return [out[r] for r in rids]
+        streams: dict[str, list[int]] = {self.add(p, params): [] for p in prompts}
+        unfinished = len(streams)
+        while unfinished:
+            for delta in self.step():
+                stream = streams.get(delta.rid)
+                if stream is not None:
+                    stream.extend(delta.token_ids)
+                    unfinished -= delta.finish_reason is not None
+        self._settle()
+        return list(streams.values())
+
+    def _settle(self) -> list[TokenDelta]:
+        """When the line is empty, what is still in flight are rows of requests that have ended since: commit them now
+        (they are dropped), so that nothing is left to wait for."""
+        return self.drain() if not len(self.sched) else []
 
     # -- one step -------------------------------------------------------------------------------------------------
     @torch.no_grad()
@@ -323,7 +342,7 @@ class Engine:
             if m:
                 seq.pending += 1
                 if seq.status is not Status.RUNNING:
-                    self.sched.finished_prefill(seq)
+                    self.sched.prompt_done(seq)
         return out
 
     def _to_host(self, t: torch.Tensor, fresh: bool = False) -> torch.Tensor:
@@ -365,26 +384,36 @@ class Engine:
             if not m:
                 continue
             token = tokens[at - 1]
-            want = seq.params.logprobs
-            lp = None if want is None else Logprobs([lps[0][at - 1]], [lps[1][at - 1][:want]], [lps[2][at - 1][:want]])
             seq.pending -= 1
             seq.tokens.append(token)
-            for sibling in reversed(self._siblings.pop(seq, [])):         # its prompt is cached now
-                self.sched.add(sibling, front=True)
-            reason = self._finish_reason(seq, token)
-            if reason:
-                self.sched.finish(seq, reason)
-                live = self._live.get(seq.rid, [])
-                if seq in live:
-                    live.remove(seq)
-                if not live:
-                    self._live.pop(seq.rid, None)
-            first = not seq.reported
-            seq.reported = True
-            deltas.append(TokenDelta(seq.rid, [token], reason, lp, seq.index,
-                                     self._prompt_lp.pop(seq, None) if first else None,
-                                     seq.cached_tokens if first else None))
+            self._release_siblings(seq)
+            reason = seq.verdict(token, self.eos, self.cfg.max_model_len)
+            if reason is not None:
+                self._close(seq, reason)
+            delta = TokenDelta(seq.rid, [token], reason, index=seq.index)
+            if seq.params.logprobs is not None:
+                k, row = seq.params.logprobs, at - 1
+                delta.logprobs = Logprobs([lps[0][row]], [lps[1][row][:k]], [lps[2][row][:k]])
+            if not seq.reported:                       # the first delta also carries what belongs to the prompt
+                seq.reported = True
+                delta.prompt_logprobs = self._prompt_lp.pop(seq, None)
+                delta.cached_tokens = seq.cached_tokens
+            deltas.append(delta)
         return deltas
+
+    def _release_siblings(self, seq: Seq) -> None:
+        """The first sequence of a request has drawn a token, so its prompt is in the cache: the request's other
+        sequences join the head of the line, in their order."""
+        for sibling in reversed(self._siblings.pop(seq, ())):
+            self.sched.add(sibling, front=True)
+
+    def _close(self, seq: Seq, reason: str) -> None:
+        self.sched.retire(seq, reason)
+        rest = [s for s in self._live.get(seq.rid, ()) if s is not seq]
+        if rest:
+            self._live[seq.rid] = rest
+        else:
+            self._live.pop(seq.rid, None)
 
     def _prompt_places(self, seq: Seq, n: int) -> tuple[int, int]:
         """The places among the next `n` tokens of `seq` whose logits predict a prompt token not yet recorded (a
@@ -400,12 +429,3 @@ class Engine:
         acc.token += lp
         acc.top_ids += [row[:k] for row in ids]
         acc.top += [row[:k] for row in top]
-
-    def _finish_reason(self, seq: Seq, token: int) -> str | None:
-        p = seq.params
-        if (token in self.eos and not p.ignore_eos) or token in p.stop_token_ids:
-            return "stop"
-        generated = len(seq.tokens) - seq.prompt_len
-        if (p.max_tokens is not None and generated >= p.max_tokens) or len(seq.tokens) >= self.cfg.max_model_len:
-            return "length"
-        return None

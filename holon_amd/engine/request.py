@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import dataclasses
 import enum
+from collections.abc import Collection
 
 from ..config.engine import SamplingParams
 
@@ -35,6 +36,33 @@ class Seq:
     def __post_init__(self) -> None:
         if not self.prompt_len:
             self.prompt_len = len(self.tokens)
+
+    @property
+    def admitted(self) -> bool:
+        return self.slot >= 0
+
+    @property
+    def uncomputed(self) -> int:
+        """Tokens it has that the cache does not hold yet."""
+        return len(self.tokens) - self.num_computed
+
+    def length_left(self, max_model_len: int, in_flight: bool = True) -> int:
+        """How many more tokens it may be given before a length limit ends it. `in_flight` counts the tokens drawn for
+        it that are still on their way to the host: a request at its limit with tokens in flight is not scheduled
+        again (core/holon/core/sched.py:163-170)."""
+        have = len(self.tokens) + (self.pending if in_flight else 0)
+        left = max_model_len - have
+        if self.params.max_tokens is not None:
+            left = min(left, self.params.max_tokens - (have - self.prompt_len))
+        return max(left, 0)
+
+    def verdict(self, token: int, eos: Collection[int], max_model_len: int) -> str | None:
+        """Whether `token`, just appended, ends the sequence: "stop" for an end-of-sequence token (unless ignored) or
+        one of the request's stop tokens, "length" at `max_tokens` or `max_model_len`. The finishing token is part
+        of the output (core/holon/core/engine.py:702-709)."""
+        if token in self.params.stop_token_ids or (token in eos and not self.params.ignore_eos):
+            return "stop"
+        return "length" if self.length_left(max_model_len, in_flight=False) == 0 else None
 
 
 @dataclasses.dataclass

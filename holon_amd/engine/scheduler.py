@@ -1,133 +1,186 @@
-"""Scheduling: which requests run in the next step and how many tokens each. core/holon/core/sched.py:65-217.
+"""Scheduling: which requests run in the next step and how many tokens each. Policy as in the reference
+(core/holon/core/sched.py:65-217); the structure is this engine's own.
 
-First come, first served. Requests are ranked running (oldest first), then waiting (queue order; a preempted request
-re-enters at the front). Without mixing (`chunk_with_decode` 0) a step is either prompt portions — of as many waiting
-requests as the token budget `max_step_tokens` holds, a long prompt cut where the budget ends — or one decoded token
-for every running request; waiting requests go first. With mixing (`chunk_with_decode` C > 0) a step carries every
-running request's decode token and then prompt portions of up to C tokens.
+One line of requests in rank order. The first `n_running` of it decode (oldest first); the rest wait for their prompt,
+or for what is left of it, in arrival order. A request that ends its prompt moves to the end of the decoding part; a
+preempted one moves to the head of the waiting part. Rank decides who gives way when pages run out.
 
-When pages run out: a request that cannot get the pages it needs takes them from the requests ranked below it, the
-lowest first, as long as releasing those can make room (preemption by recompute: the victim gives back everything,
-goes to the front of the queue and later runs its prompt and the tokens it had generated again as one prompt). When
-nothing below can make room, a running request preempts itself and a waiting one ends the step's admissions. The pool
-always holds one request of `max_model_len` tokens (checked when the engine starts), so the top-ranked request always
-fits once everything below it is preempted, and every step makes progress.
+Without mixing (`chunk_with_decode` 0) a step is either prompt portions, of as many waiting requests as the token
+budget `max_step_tokens` holds (a long prompt is cut where the budget ends), or one decoded token for every running
+request; prompts go first. With mixing (`chunk_with_decode` C > 0) a step carries every running request's token and
+then prompt portions of up to C tokens in all.
+
+A portion may also be cut short by the model: a mixer whose state is kept on a grid of positions says through `cut`
+where a portion that does not end the prompt may end (core/holon/core/sched.py:149-151).
+
+When pages run out, a request takes them from the requests ranked below it, the lowest first, as many as the cache
+manager says are needed; they give back everything, wait at the head of the line and later run their prompt and the
+tokens they had generated again as one prompt (preemption by recompute). If not even all of them would make room,
+nobody is preempted: a running request then gives way itself, a waiting one ends the step's admissions (first come,
+first served: nobody behind it skips ahead). The pool always holds one request of `max_model_len` tokens (the engine
+checks that at start), so the first in line always fits once the others have given way, and every step makes
+progress.
 
 A step may be scheduled while the one before it still runs (core/holon/core/sched.py:12-15, 98-104): a request whose
-last drawn token has not reached the host (`pending`) decodes from the copy of it on the device; it counts towards the
-request's length limits; a preempted request waits for it before its tokens are run again as a prompt.
+last drawn token has not reached the host (`pending`) decodes from the copy of it on the device; that token counts
+towards its length limits; a preempted request waits for it before its tokens are run again as a prompt.
 """
 from __future__ import annotations
 
-import collections
+from collections.abc import Callable
+from typing import NamedTuple
 
 from ..cache.manager import CacheManager
 from .request import Seq, Status
 
-Row = tuple[Seq, int, int]               # (request, tokens to run, 1 if the last of them is sampled)
+
+class Portion(NamedTuple):
+    """One row of a step: `count` next tokens of `seq`; `samples`: the last of them ends what the request has, so a
+    token is drawn after it."""
+
+    seq: Seq
+    count: int
+    samples: bool
 
 
 class Scheduler:
     def __init__(self, cache: CacheManager, max_step_tokens: int, max_model_len: int, chunk_with_decode: int = 0,
-                 on_admit=None) -> None:
+                 on_admit: Callable[[Seq], None] | None = None,
+                 cut: Callable[[int, int], int] | None = None) -> None:
         self.cache, self.max_step_tokens, self.max_model_len = cache, max_step_tokens, max_model_len
         self.chunk_with_decode = chunk_with_decode
         self.on_admit = on_admit
-        self.waiting: collections.deque[Seq] = collections.deque()
-        self.running: list[Seq] = []
+        self.cut = cut                     # (tokens computed, tokens offered) -> tokens a portion may take (0: none now)
+        self.line: list[Seq] = []
+        self.n_running = 0
         self.preemptions = 0
         self.mixed_steps = 0
 
-    def add(self, seq: Seq, front: bool = False) -> None:
-        seq.status = Status.WAITING
-        (self.waiting.appendleft if front else self.waiting.append)(seq)
+    # -- the line -------------------------------------------------------------------------------------------------
+    @property
+    def running(self) -> list[Seq]:
+        return self.line[: self.n_running]
 
-    def schedule(self) -> list[Row] | None:
-        """The next step's rows: decode rows first, then prompt portions. None when nothing can run."""
-        cap = self.chunk_with_decode
-        if not cap:
-            rows = self._prefill(self.max_step_tokens) or self._decode()
+    @property
+    def waiting(self) -> list[Seq]:
+        return self.line[self.n_running:]
+
+    def __len__(self) -> int:
+        return len(self.line)
+
+    def add(self, seq: Seq, front: bool = False) -> None:
+        """A new request joins the waiting part: at its end, or at its head (`front`)."""
+        seq.status = Status.WAITING
+        self.line.insert(self.n_running if front else len(self.line), seq)
+
+    def prompt_done(self, seq: Seq) -> None:
+        """Its prompt is in the cache and its first token drawn: it decodes from now on, ranked behind those that
+        already do."""
+        self.line.remove(seq)
+        self.line.insert(self.n_running, seq)
+        self.n_running += 1
+        seq.status = Status.RUNNING
+
+    def retire(self, seq: Seq, reason: str) -> None:
+        """The request leaves the line for good and gives back what it holds."""
+        at = self.line.index(seq)
+        del self.line[at]
+        self.n_running -= at < self.n_running
+        if seq.admitted:
+            self.cache.release(seq.slot)
+            seq.slot = -1
+        seq.status, seq.finish_reason = Status.FINISHED, reason
+
+    def _evict(self, seq: Seq) -> None:
+        """Preemption by recompute: everything it holds goes back; a decoding request returns to the head of the
+        waiting part, a waiting one (part of its prompt computed) keeps its place."""
+        self.cache.release(seq.slot)
+        seq.slot, seq.num_computed = -1, 0
+        self.preemptions += 1
+        at = self.line.index(seq)
+        if at < self.n_running:
+            del self.line[at]
+            self.n_running -= 1
+            self.line.insert(self.n_running, seq)
+            seq.status = Status.PREEMPTED
+
+    # -- one step -------------------------------------------------------------------------------------------------
+    def schedule(self) -> list[Portion] | None:
+        """The next step's rows, decode rows before prompt portions; None when nothing can run."""
+        rows: list[Portion] = []
+        if self.chunk_with_decode:
+            self._decode_rows(rows)
+            n_decode = len(rows)
+            left = self.max_step_tokens - n_decode
+            self._prompt_rows(rows, min(self.chunk_with_decode, left) if n_decode else left)
+            self.mixed_steps += 0 < n_decode < len(rows)
         else:
-            decode = self._decode()
-            if decode:
-                chunks = self._prefill(min(cap, self.max_step_tokens - len(decode)))
-                self.mixed_steps += bool(chunks)
-                rows = decode + chunks
-            else:
-                rows = self._prefill(self.max_step_tokens)
+            self._prompt_rows(rows, self.max_step_tokens)
+            if not rows:
+                self._decode_rows(rows)
         return rows or None
 
-    def _prefill(self, budget: int) -> list[Row]:
-        rows: list[Row] = []
-        for seq in list(self.waiting):
-            if seq.pending:                                     # preempted with a token on its way: not yet
-                continue
-            if budget <= 0 or (seq.slot < 0 and not self._fit(seq, None)):
-                break                                           # first come first served: nobody skips ahead
-            n = min(len(seq.tokens) - seq.num_computed, budget, seq.portion_cap or budget)
-            if not self._fit(seq, seq.num_computed + n):
-                break
-            rows.append((seq, n, int(seq.num_computed + n == len(seq.tokens))))
-            budget -= n
-        return rows
-
-    def _decode(self) -> list[Row]:
-        rows: list[Row] = []
-        for seq in list(self.running):
-            if seq.status is not Status.RUNNING or self.at_limit(seq):   # preempted by a row above it
-                continue
-            total = seq.num_computed + 1
-            if total <= self.cache.capacity(seq.slot) or self._fit(seq, total):
-                rows.append((seq, 1, 1))
+    def _decode_rows(self, rows: list[Portion]) -> None:
+        at = 0
+        while at < self.n_running:                # the part shrinks when a request gives way
+            seq = self.line[at]
+            if seq.length_left(self.max_model_len) == 0:          # its last token is on its way
+                at += 1
+            elif self._room(seq, seq.num_computed + 1):
+                rows.append(Portion(seq, 1, True))
+                at += 1
             else:
-                self._preempt(seq)
-        return rows
+                self._evict(seq)                  # nothing below it can make room: it gives way itself
 
-    def at_limit(self, seq: Seq) -> bool:
-        n = len(seq.tokens) + seq.pending
-        return n >= self.max_model_len or (seq.params.max_tokens is not None
-                                           and n - seq.prompt_len >= seq.params.max_tokens)
+    def _prompt_rows(self, rows: list[Portion], budget: int) -> None:
+        for seq in self.waiting:                  # a copy: those that give way below keep their places
+            if seq.pending:                       # preempted with a token still on its way: not yet
+                continue
+            if budget <= 0 or not (seq.admitted or self._seat(seq)):
+                return
+            count = min(seq.uncomputed, budget, seq.portion_cap or budget)      # after admission: a cached start counts
+            if self.cut is not None and count < seq.uncomputed:
+                count = self.cut(seq.num_computed, count)
+            if count <= 0 or not self._room(seq, seq.num_computed + count):
+                return
+            rows.append(Portion(seq, count, count == seq.uncomputed))
+            budget -= count
 
-    def _admit(self, seq: Seq) -> bool:
+    # -- room -----------------------------------------------------------------------------------------------------
+    def _below(self, seq: Seq) -> list[Seq]:
+        """The admitted requests ranked below `seq`, the lowest first."""
+        at = self.line.index(seq)
+        return [s for s in reversed(self.line[at + 1:]) if s.admitted]
+
+    def _seat(self, seq: Seq) -> bool:
+        """A slot for a waiting request (and the cached start of its tokens, which is then not run again)."""
         slot = self.cache.admit()
         if slot is None:
-            return False
+            below = self._below(seq)
+            if not below:
+                return False
+            self._evict(below[0])
+            slot = self.cache.admit()
         seq.slot = slot
-        if seq.share_prefix:                       # the cached start of its tokens is not run again
+        if seq.share_prefix:
             seq.num_computed = self.cache.adopt(slot, seq.tokens)
         if self.on_admit is not None:
             self.on_admit(seq)
         return True
 
-    def _fit(self, seq: Seq, total: int | None) -> bool:
-        """Admit `seq` (total None) or reserve pages for its first `total` tokens, preempting requests ranked below it,
-        the lowest first, while releasing them can make room."""
-        while not (self._admit(seq) if total is None else self.cache.reserve(seq.slot, total)):
-            ranked = self.running + list(self.waiting)
-            below = [s for s in ranked[ranked.index(seq) + 1:] if s.slot >= 0]
-            if not below or not self.cache.could_fit(seq.slot if seq.slot >= 0 else None, total or 0,
-                                                     [s.slot for s in below]):
+    def _room(self, seq: Seq, total: int) -> bool:
+        """Pages for the first `total` tokens of `seq`, taken from requests below it if need be."""
+        if total <= self.cache.capacity(seq.slot) or self.cache.reserve(seq.slot, total):
+            return True
+        below = self._below(seq)
+        need = self.cache.victims_needed(seq.slot, total, [s.slot for s in below])
+        if need is None:
+            return False
+        for victim in below[:need]:
+            self._evict(victim)
+        spare = below[need:]
+        while not self.cache.reserve(seq.slot, total):            # the count was of pages as they stood: hold to it
+            if not spare:
                 return False
-            self._preempt(below[-1])
+            self._evict(spare.pop(0))
         return True
-
-    def _preempt(self, seq: Seq) -> None:
-        self.cache.release(seq.slot)
-        seq.slot, seq.num_computed = -1, 0
-        self.preemptions += 1
-        if seq.status is Status.RUNNING:
-            self.running.remove(seq)
-            self.waiting.appendleft(seq)
-            seq.status = Status.PREEMPTED
-
-    def finished_prefill(self, seq: Seq) -> None:
-        self.waiting.remove(seq)
-        seq.status = Status.RUNNING
-        self.running.append(seq)
-
-    def finish(self, seq: Seq, reason: str) -> None:
-        (self.running if seq.status is Status.RUNNING else self.waiting).remove(seq)
-        if seq.slot >= 0:
-            self.cache.release(seq.slot)
-            seq.slot = -1
-        seq.status, seq.finish_reason = Status.FINISHED, reason

@@ -12,6 +12,7 @@ first step of a bucket runs eagerly on those buffers, the second captures, later
 from __future__ import annotations
 
 import dataclasses
+import sys
 
 import numpy as np
 import torch
@@ -47,7 +48,12 @@ class StepRunner:
         # the token last drawn for each slot, for a row whose token has not reached the host when it is scheduled
         self.last_token = torch.zeros(max_seqs + 1, dtype=torch.int32, device=device)
         self.last_slots: torch.Tensor | None = None       # the last step's rows' slots on the device
-        self.use_graphs = graphs and device.type == "cuda"
+        # a captured step is replayed without any part's Python code: only over parts that say they allow it
+        self.not_graph_safe = sorted({type(p).__name__ for p in model.walk() if not p.graph_safe})
+        self.use_graphs = graphs and device.type == "cuda" and not self.not_graph_safe
+        if graphs and device.type == "cuda" and self.not_graph_safe:
+            print(f"holon_amd: steps run eagerly, not from graphs: {', '.join(self.not_graph_safe)} "
+                  "do not declare graph_safe", file=sys.stderr)
         self.graphs: dict[tuple[int, int], _Graph] = {}
         self.graph_replays = 0
 

@@ -92,6 +92,10 @@ class Kernels(Protocol):
         projection qkv [T, (Hq + 2 Hkv) D]: q and k heads are normed and rounded, rotated and rounded; k and v go to
         the cache; returns q' [T, Hq, D], a new tensor. Same roundings as the three ops one after the other."""
 
+    def check_attention(self, head_dim: int, page_size: int, dtype: torch.dtype) -> None:
+        """Raise, with a message that names the limit, when no attention kernel serves this head size, page size and
+        dtype. Mixers call it when they are built, so that a model is refused before it takes a request."""
+
     def paged_attention(self, q: torch.Tensor, pages: torch.Tensor, table: torch.Tensor, rows: AttnRows,
                         page_size: int, scale: float, window: int) -> torch.Tensor:
         """softmax(q k^T * scale) v per row over its cached tokens, causal; with window W > 0 a query at position p

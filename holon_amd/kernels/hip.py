@@ -257,6 +257,13 @@ class HipKernels:
                    pages.shape[0] if pages is not None else 0, self._dt(qkv, "qkv"), self._stream())
         return q
 
+    def check_attention(self, head_dim, page_size, dtype):
+        if dtype not in _DT:
+            raise KernelError(f"attention: dtype {dtype} is not served (float32 and bfloat16 are)")
+        if head_dim % 8 or not 8 <= head_dim <= 512 or page_size < 1:
+            raise KernelError(f"attention: head_dim {head_dim} is not served (multiples of 8 up to 512, any page size "
+                              f">= 1; got page size {page_size})")
+
     def paged_attention(self, q, pages, table, rows: AttnRows, page_size, scale, window):
         self._check(q, "attention q")
         self._check(pages, "attention pages", q.dtype)

@@ -11,9 +11,19 @@ from .spec import ModelSpec
 
 
 @dataclasses.dataclass
+class SitePages:
+    """One paged state of one run: the group whose block table addresses it, and its storage."""
+
+    group: int
+    pages: torch.Tensor                           # [num_pages, P * elems]
+
+
+@dataclasses.dataclass
 class Site:
     """One entry of the run order as the cache sees it: which layer runs, which cache it uses and whether it writes
-    it. The cache manager fills `group`, `pages` and `slot_state` when it allocates."""
+    it. The cache manager fills `paged` and `slot_state` when it allocates: one entry for every state the run's mixer
+    declares, by the declaration's name. `group` and `pages` are those of the first paged state declared (all there
+    is for a mixer that keeps one)."""
 
     run: int
     layer: int
@@ -21,14 +31,17 @@ class Site:
     owner: int | None = None                      # the run whose cache this one reads (None: its own)
     group: int | None = None                      # paged group id
     pages: torch.Tensor | None = None             # this site's page storage [num_pages, P * elems]
+    paged: dict[str, SitePages] = dataclasses.field(default_factory=dict)
     slot_state: dict[str, torch.Tensor] = dataclasses.field(default_factory=dict)   # name -> [S+1, *shape]
 
     def detach(self) -> None:
         """Forget the storage a cache manager gave (before another one is made for the same model)."""
-        self.group, self.pages, self.slot_state = None, None, {}
+        self.group, self.pages, self.paged, self.slot_state = None, None, {}, {}
 
 
 class Model(Part):
+    graph_safe = True
+
     def __init__(self, spec: ModelSpec, build: Build) -> None:
         super().__init__(build)
         self.spec = spec
@@ -50,6 +63,13 @@ class Model(Part):
             mixer = getattr(self.blocks[site.layer], "mixer", None)
             out.append(list(mixer.state()) if mixer is not None and site.writes else [])
         return out
+
+    def cut(self, start: int, count: int) -> int:
+        """Where a prompt portion of `count` tokens from position `start` may end, by every part's own `cut`."""
+        for part in self.walk():
+            if part is not self and count > 0:
+                count = min(count, max(0, part.cut(start, count)))
+        return count
 
     def trunk(self, step) -> tuple[torch.Tensor, torch.Tensor | None]:
         """The residual stream after every run, as (h, delta) with h + delta the stream [T, hidden]."""

@@ -70,6 +70,10 @@ class Part:
     """Base of all parts. Subclasses call `declare` for tensors and `attach` for sub-parts in `__init__`."""
 
     adds_residual = False     # its forward accepts `residual=h`: it may add its result into h and return None
+    graph_safe = False        # True: a captured step may be replayed over it. Its forward then reads nothing on the
+                              # host that changes from step to step (no `step.h_*`, no `.item()`, no shapes that depend
+                              # on values) and launches the same kernels on the same buffers whatever the rows are.
+                              # A model with one part that does not say so runs every step eagerly.
 
     def __init__(self, build: Build) -> None:
         self.build = build
@@ -109,6 +113,12 @@ class Part:
     def state(self) -> list[PagedState | SlotState]:
         """What this part keeps between steps (mixers)."""
         return []
+
+    def cut(self, start: int, count: int) -> int:
+        """How many of the next `count` tokens, the first at position `start`, a prompt portion that does not end the
+        prompt may take (0: none, offer more). A mixer whose state is only right on a grid of positions ends portions
+        there; the scheduler asks every part of the model and takes the smallest answer. Default: all of them."""
+        return count
 
     def nbytes(self) -> int:
         total = 0

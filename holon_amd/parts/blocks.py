@@ -14,6 +14,8 @@ class PreNorm(Part):
     its sum (the block's last add into the next reader's norm: `delta` is a term not yet added to `h`); all adds are
     in the activation dtype."""
 
+    graph_safe = True
+
     def __init__(self, build: Build, *, layer: int, hidden: int, mixer: PartRef, ffn: PartRef, norm: PartRef) -> None:
         super().__init__(build)
         self.attach("input_norm", build.make(norm, dim=hidden))

@@ -9,6 +9,8 @@ from .base import Build, Part
 
 @register_part("embed", "table")
 class Embedding(Part):
+    graph_safe = True
+
     def __init__(self, build: Build, *, vocab: int, hidden: int) -> None:
         super().__init__(build)
         self.declare("weight", (vocab, hidden))
@@ -23,6 +25,8 @@ class Embedding(Part):
 @register_part("head", "linear")
 class LMHead(Part):
     """Logits in float32. A tied head owns no tensor: it reads the embedding's."""
+
+    graph_safe = True
 
     def __init__(self, build: Build, *, vocab: int, hidden: int, tied: bool, embed: Embedding) -> None:
         super().__init__(build)

@@ -12,6 +12,8 @@ from .linear import Linear
 class SwiGLU(Part):
     """down(silu(gate(x)) * up(x)); gate and up are merged into one product after loading (gate rows first)."""
 
+    graph_safe = True
+
     def __init__(self, build: Build, *, inter: int, hidden: int, layer: int) -> None:
         super().__init__(build)
         self.inter, self.hidden = inter, hidden

@@ -8,6 +8,8 @@ from .base import Build, Part
 
 
 class Linear(Part):
+    graph_safe = True
+
     def __init__(self, build: Build, *, inp: int, out: int) -> None:
         super().__init__(build)
         self.inp, self.out = inp, out

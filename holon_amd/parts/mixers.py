@@ -18,12 +18,16 @@ class GQA(Part):
 
     A run that reads another run's cache (`site.writes` false) projects and encodes queries only."""
 
+    graph_safe = True
+
     def __init__(self, build: Build, *, heads: int, kv_heads: int, head_dim: int, hidden: int, layer: int,
                  qk_norm: PartRef | None = None, position: PartRef | None = None, window: int = 0,
                  scale: float | None = None) -> None:
         super().__init__(build)
         if heads % kv_heads:
             raise ValueError(f"gqa: {heads} heads are not a multiple of {kv_heads} kv heads")
+        if build.kernels is not None:             # a size no attention kernel serves is refused now, not at the first step
+            build.kernels.check_attention(head_dim, build.page_size, build.dtype)
         self.heads, self.kv_heads, self.head_dim, self.hidden, self.layer = heads, kv_heads, head_dim, hidden, layer
         self.window = int(window)
         self.scale = float(scale) if scale is not None else head_dim ** -0.5
@@ -35,7 +39,9 @@ class GQA(Part):
         if qk_norm is not None:
             self.attach("q_norm", build.make(qk_norm, dim=head_dim))
             self.attach("k_norm", build.make(qk_norm, dim=head_dim))
-        self.position = build.make(position, head_dim=head_dim) if position is not None else None
+        self.position = None
+        if position is not None:
+            self.attach("position", build.make(position, head_dim=head_dim))
         self.qkv: Linear | None = None
         self._fused: dict | None = None
 

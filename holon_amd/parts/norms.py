@@ -11,6 +11,8 @@ from .base import Build, Part
 class RMSNorm(Part):
     """y = x * rsqrt(mean(x^2) + eps) * weight over the last `dim` values, float32 inside, rounded once."""
 
+    graph_safe = True
+
     def __init__(self, build: Build, *, eps: float, dim: int) -> None:
         super().__init__(build)
         self.eps, self.dim = float(eps), dim

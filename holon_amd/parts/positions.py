@@ -22,6 +22,8 @@ class Rope(Part):
     """Rotary embedding, half-split ("neox") pairing: dims (i, i + rotary_dim/2) rotate by position * theta_i; dims
     beyond `rotary_dim` pass through."""
 
+    graph_safe = True
+
     def __init__(self, build: Build, *, theta: float, head_dim: int, rotary_dim: int | None = None) -> None:
         super().__init__(build)
         self.theta, self.head_dim = float(theta), head_dim
@@ -43,6 +45,8 @@ class Rope(Part):
 @register_part("position", "none")
 class NoPosition(Part):
     """No position encoding (order enters through the causal mask alone)."""
+
+    graph_safe = True
 
     def __init__(self, build: Build, *, head_dim: int) -> None:
         super().__init__(build)

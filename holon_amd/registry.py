@@ -34,6 +34,10 @@ def register_architecture(name: str, config: Any, recipe: Callable[[Any], ModelS
     _ARCHITECTURES[name] = Architecture(name, config, recipe)
 
 
+def unregister_architecture(name: str) -> None:
+    _ARCHITECTURES.pop(name, None)
+
+
 def architecture(name: str) -> Architecture:
     _load_builtin()
     if name not in _ARCHITECTURES:

@@ -58,17 +58,27 @@ class Run:
 @dataclasses.dataclass(frozen=True)
 class WeightRule:
     """A checkpoint tensor name pattern and the parameter path it fills: `{i}` matches digits, any other `{name}` one
-    or more characters, the whole name must match (core/holon/core/build.py:317-337)."""
+    or more characters, the whole name must match (core/holon/core/build.py:317-337).
+
+    `stack` names a capture of digits that is no part of the target: the tensor then fills slice number `stack` of
+    the target parameter's first dimension, so that one tensor per expert fills a parameter `[experts, ...]`
+    (core/holon/core/build.py:351-369): `WeightRule("layers.{i}.mlp.experts.{e}.up.weight", "layers.{i}.ffn.up", "e")`."""
 
     pattern: str
     target: str
+    stack: str | None = None
+
+    def __post_init__(self) -> None:
+        if self.stack is not None and ("{" + self.stack + "}" not in self.pattern or "{" + self.stack + "}" in self.target):
+            raise ValueError(f"rule {self.pattern!r}: the stacking capture {{{self.stack}}} must be in the pattern and "
+                             "not in the target")
 
     def compile(self) -> re.Pattern[str]:
         parts = re.split(r"(\{\w+\})", self.pattern)
         out = []
         for p in parts:
             if p.startswith("{") and p.endswith("}"):
-                out.append(f"(?P<{p[1:-1]}>" + (r"\d+" if p == "{i}" else ".+") + ")")
+                out.append(f"(?P<{p[1:-1]}>" + (r"\d+" if p in ("{i}", "{" + str(self.stack) + "}") else ".+") + ")")
             else:
                 out.append(re.escape(p))
         return re.compile("".join(out) + r"\Z")

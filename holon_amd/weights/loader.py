@@ -37,23 +37,46 @@ class WeightError(ValueError):
         super().__init__("\n".join(lines))
 
 
-def map_name(rules: tuple[WeightRule, ...], name: str, compiled: list[re.Pattern] | None = None) -> str | None:
-    """The parameter path of checkpoint tensor `name`, or None when no rule matches."""
+def locate(rules: tuple[WeightRule, ...], name: str, compiled: list[re.Pattern] | None = None
+           ) -> tuple[str, int | None] | None:
+    """Where checkpoint tensor `name` goes: (parameter path, slice of its first dimension or None for the whole
+    parameter); None when no rule matches."""
     for rule, pattern in zip(rules, compiled or [r.compile() for r in rules]):
         m = pattern.match(name)
         if m:
-            return rule.target.format(**m.groupdict())
+            groups = m.groupdict()
+            index = int(groups.pop(rule.stack)) if rule.stack is not None else None
+            return rule.target.format(**groups), index
     return None
 
 
-def unmap_name(rules: tuple[WeightRule, ...], path: str) -> str | None:
-    """The checkpoint name that maps to parameter path `path` (the rules run backwards)."""
+def map_name(rules: tuple[WeightRule, ...], name: str, compiled: list[re.Pattern] | None = None) -> str | None:
+    """The parameter path of checkpoint tensor `name`, or None when no rule matches."""
+    found = locate(rules, name, compiled)
+    return found[0] if found is not None else None
+
+
+def checkpoint_names(rules: tuple[WeightRule, ...], path: str, shape: tuple[int, ...]) -> list[tuple[str, int | None]]:
+    """The checkpoint tensors that fill parameter `path` of `shape`, as (name, slice or None): the rules run
+    backwards. One name for a whole parameter, one per slice for a stacked one; empty when no rule names it."""
     for rule in rules:
-        m = WeightRule(rule.target, rule.pattern).compile().match(path)
-        if m:
-            name = rule.pattern.format(**m.groupdict())
-            if map_name(rules, name) == path:
-                return name
+        m = WeightRule(rule.target, "").compile().match(path)
+        if not m:
+            continue
+        slices = [None] if rule.stack is None else list(range(shape[0]))
+        names = [(rule.pattern.format(**m.groupdict(), **({rule.stack: e} if e is not None else {})), e) for e in slices]
+        if all(locate(rules, name) == (path, e) for name, e in names):
+            return names
+    return []
+
+
+def unmap_name(rules: tuple[WeightRule, ...], path: str) -> str | None:
+    """The checkpoint name that maps to the whole of parameter `path`, if one rule gives one."""
+    for rule in rules:
+        if rule.stack is None:
+            names = checkpoint_names((rule,), path, ())
+            if names and map_name(rules, names[0][0]) == path:
+                return names[0][0]
     return None
 
 
@@ -72,7 +95,7 @@ def load_weights(model: Part, spec: ModelSpec, folder: str | pathlib.Path, devic
                  dtype: torch.dtype) -> None:
     params = {path: (owner, attr, decl) for path, owner, attr, decl in model.named_params()}
     compiled = [r.compile() for r in spec.rules]
-    where: dict[str, tuple[pathlib.Path, str]] = {}          # parameter path -> (file, tensor name)
+    where: dict[tuple[str, int | None], tuple[pathlib.Path, str]] = {}      # (parameter path, slice) -> (file, name)
     seen: dict[str, pathlib.Path] = {}
     missing, unexpected, wrong, other = [], [], [], []
     files = tensor_files(folder)
@@ -85,31 +108,51 @@ def load_weights(model: Part, spec: ModelSpec, folder: str | pathlib.Path, devic
                 seen[name] = file
                 if any(name.startswith(p) for p in spec.skip):
                     continue
-                path = map_name(spec.rules, name, compiled)
-                if path is None or path not in params:
+                found = locate(spec.rules, name, compiled)
+                if found is None or found[0] not in params:
                     unexpected.append(name)
                     continue
-                if path in where:
-                    other.append(f"tensors {where[path][1]} and {name} both fill {path}")
+                path, index = found
+                want = params[path][2].shape
+                if index is not None:             # one slice of a stacked parameter
+                    if not want or index >= want[0]:
+                        unexpected.append(name)
+                        continue
+                    want = want[1:]
+                if found in where:
+                    other.append(f"tensors {where[found][1]} and {name} both fill {path}")
                     continue
-                got, want = tuple(f.get_slice(name).get_shape()), params[path][2].shape
+                got = tuple(f.get_slice(name).get_shape())
                 if got != want:
                     wrong.append((name, got, want))
-                where[path] = (file, name)
-    for path in params:
-        if path not in where:
-            missing.append(unmap_name(spec.rules, path) or path)
+                where[found] = (file, name)
+    stacked = {path for path, index in where if index is not None}
+    for path, (_, _, decl) in params.items():
+        if path in stacked:
+            if (path, None) in where:
+                other.append(f"{where[(path, None)][1]} fills {path} whole and other tensors fill slices of it")
+            names = dict((e, n) for n, e in checkpoint_names(spec.rules, path, decl.shape))
+            missing += [names.get(e, f"{path}[{e}]") for e in range(decl.shape[0]) if (path, e) not in where]
+        elif (path, None) not in where:
+            names = checkpoint_names(spec.rules, path, decl.shape)
+            missing += [n for n, _ in names] or [path]
     if missing or unexpected or wrong or other:
         raise WeightError(sorted(missing), sorted(unexpected), sorted(wrong), other)
-    by_file: dict[pathlib.Path, list[str]] = {}
-    for path, (file, _) in where.items():
-        by_file.setdefault(file, []).append(path)
+    by_file: dict[pathlib.Path, list[tuple[str, int | None]]] = {}
+    for key, (file, _) in where.items():
+        by_file.setdefault(file, []).append(key)
+    for path in stacked:
+        owner, attr, decl = params[path]
+        setattr(owner, attr, torch.empty(decl.shape, dtype=param_dtype(decl, dtype), device=device))
     for file in files:
         with safe_open(str(file), "pt", device="cpu") as f:
-            for path in by_file.get(file, []):
+            for path, index in by_file.get(file, []):
                 owner, attr, decl = params[path]
-                tensor = f.get_tensor(where[path][1])
-                setattr(owner, attr, tensor.to(device=device, dtype=param_dtype(decl, dtype)).contiguous())
+                tensor = f.get_tensor(where[(path, index)][1]).to(device=device, dtype=param_dtype(decl, dtype))
+                if index is None:
+                    setattr(owner, attr, tensor.contiguous())
+                else:
+                    getattr(owner, attr)[index].copy_(tensor)
     finalize(model)
 
 

@@ -6,6 +6,7 @@ rounded to bfloat16 before they are stored, so the 32-bit and the bfloat16 model
 """
 from __future__ import annotations
 
+import dataclasses
 import hashlib
 import json
 import pathlib
@@ -16,7 +17,7 @@ from safetensors.torch import save_file
 
 from ..parts.base import INT32, Build, ParamDecl
 from ..registry import resolve
-from .loader import finalize, param_dtype, unmap_name
+from .loader import checkpoint_names, finalize, param_dtype
 
 LINEAR_STD, NORM_STD = 0.02, 0.1
 
@@ -50,10 +51,12 @@ def write_random_model(config_json: dict[str, Any], seed: int, folder: str | pat
     folder.mkdir(parents=True, exist_ok=True)
     tensors = {}
     for path, _, _, decl in model.named_params():
-        name = unmap_name(spec.rules, path)
-        if name is None:
+        names = checkpoint_names(spec.rules, path, decl.shape)
+        if not names:
             raise ValueError(f"no weight rule names parameter {path}")
-        tensors[name] = random_tensor(name, decl, seed).to(torch.int32 if decl.kind == INT32 else store_dtype)
+        for name, index in names:                 # a stacked parameter is stored as one tensor per slice
+            one = decl if index is None else dataclasses.replace(decl, shape=decl.shape[1:])
+            tensors[name] = random_tensor(name, one, seed).to(torch.int32 if decl.kind == INT32 else store_dtype)
     (folder / "config.json").write_text(json.dumps(cfg.to_dict(), indent=1) + "\n")
     save_file(tensors, str(folder / "model.safetensors"), metadata={"format": "pt", "seed": str(seed)})
     return folder
@@ -63,6 +66,11 @@ def fill_random(model, spec, seed: int, device: torch.device, dtype: torch.dtype
     """Random weights drawn on the device into a built model (no folder): for measurements at sizes whose folder would
     take minutes to write. The values differ from `write_random_model`'s (another generator), the law is the same."""
     for path, owner, attr, decl in model.named_params():
-        name = unmap_name(spec.rules, path) or path
-        setattr(owner, attr, random_tensor(name, decl, seed, device).to(param_dtype(decl, dtype)))
+        names = checkpoint_names(spec.rules, path, decl.shape) or [(path, None)]
+        if names[0][1] is None:
+            value = random_tensor(names[0][0], decl, seed, device)
+        else:
+            one = dataclasses.replace(decl, shape=decl.shape[1:])
+            value = torch.stack([random_tensor(name, one, seed, device) for name, _ in names])
+        setattr(owner, attr, value.to(param_dtype(decl, dtype)))
     finalize(model)

@@ -96,6 +96,9 @@ class TorchKernels:
             self.kv_write(k, v, pages, write_page, write_off, page_size)
         return q.contiguous()
 
+    def check_attention(self, head_dim, page_size, dtype):
+        return None
+
     def paged_attention(self, q, pages, table, rows, page_size, scale, window):
         t, hq, d = q.shape
         hkv = pages.shape[2]

@@ -309,3 +309,34 @@ def test_random_orders_keep_the_books_with_shared_prefixes(seed):
     cache.flush_prefix()
     cache.check()
     assert all(g.pool.free == g.pool.usable for g in cache.groups) and cache.free_slots == 5
+
+
+def test_a_run_may_keep_several_paged_states():
+    """Two states of one page geometry in one run share a group (one table, one page id for both); a state of another
+    width has a group, a pool and a table of its own. Reserving and releasing moves all of them together."""
+    decls = [[PagedState("k", 8), PagedState("v", 8), PagedState("gate", 1, dtype=torch.float32)],
+             [PagedState("k", 8), PagedState("v", 8)], [PagedState("gate", 1, dtype=torch.float32)]]
+    sites = [Site(run=i, layer=i) for i in range(3)]
+    cache = CacheManager(sites, decls, page_size=4, max_seqs=3, max_model_len=32, tokens=48,
+                         device=torch.device("cpu"), dtype=torch.bfloat16)
+    wide, narrow = cache.groups
+    assert wide.members == [(0, "k"), (0, "v"), (1, "k"), (1, "v")] and wide.sites == [0, 1]
+    assert narrow.members == [(0, "gate"), (2, "gate")] and narrow.storage.dtype == torch.float32
+    assert sites[0].paged["k"].group == sites[0].paged["v"].group == wide.gid and sites[0].paged["gate"].group == narrow.gid
+    assert sites[0].paged["k"].pages.data_ptr() != sites[0].paged["v"].pages.data_ptr()
+    assert sites[0].group == wide.gid and sites[0].pages.data_ptr() == sites[0].paged["k"].pages.data_ptr()
+    assert sites[2].group == narrow.gid
+    a, b = cache.admit(), cache.admit()
+    assert cache.reserve(a, 9) and cache.reserve(b, 30)
+    assert wide.count[a] == narrow.count[a] == 3 and cache.capacity(b) == 32
+    assert not cache.reserve(a, 32)                           # all or nothing, over both groups
+    assert wide.count[a] == narrow.count[a] == 3
+    cache.check()
+    cache.release(b)
+    assert cache.reserve(a, 32)
+    cache.release(a)
+    cache.check()
+    assert all(g.pool.free == g.pool.usable for g in cache.groups)
+    with pytest.raises(ValueError, match="two states of one name"):
+        CacheManager([Site(run=0, layer=0)], [[PagedState("k", 8), PagedState("k", 4)]], page_size=4, max_seqs=1,
+                     max_model_len=8, tokens=8, device=torch.device("cpu"), dtype=torch.float32)

@@ -6,7 +6,8 @@ import sys
 
 import pytest
 
-from holon_amd.config import ConfigError, EngineConfig, Qwen3Config, SamplingParams
+from holon_amd.config import ConfigError, EngineConfig, SamplingParams
+from holon_amd.models.qwen3 import Qwen3Config
 from holon_amd.registry import RegistryError, architectures, part_class, register_part, resolve, unregister_part
 from holon_amd.spec import ModelSpec, PartRef, Run, WeightRule
 from tests.helpers import CONFIG_A, CONFIG_B, CONFIG_C

@@ -416,3 +416,137 @@ def test_gqa_mixer_and_block_alone(device, dtype):
             return a + _plain_ffn(plain.rms_norm(a, wd["layers.0.post_norm.weight"], eps), wd, "layers.0.ffn.")
         _several_ops_close(stream, whole(x.double(), w64), whole(x, w), dtype, 4 * hidden, f"block {hq}/{hkv}/{d}")
         cache.release(slot)
+
+
+# -- the seams another architecture would need, each with a toy part from tests/toy_parts.py ---------------------------
+def _weights_of(model):
+    """Every parameter of a built model by path, as float32 copies on the host (after merging)."""
+    return {path: getattr(owner, name).detach().float().cpu() for path, owner, name, _ in model.named_params()}
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_with_two_paged_states_of_different_widths(device, dtype):
+    from tests.toy_parts import TwoCaches
+    register_part("mixer", "test-two-caches")(TwoCaches)
+    try:
+        hq, hkv, d, eps = 4, 1, 16, 1e-6
+        ffn = PartRef("ffn", "swiglu", inter=96)
+        spec = _spec([(PartRef("mixer", "test-two-caches"), ffn), (_gqa(hq, hkv, d), ffn),
+                      (PartRef("mixer", "test-two-caches"), ffn)])
+        model, w, cache, runner = _model(spec, device, dtype, 11, page_size=4, cache_tokens=96)
+        widths = sorted((g.decl.elems, len(g.members)) for g in cache.groups)
+        assert widths == [(1, 2), (2 * hkv * d, 1), (64, 2)]                 # three groups, three block tables
+        assert not runner.use_graphs and "TwoCaches" in runner.not_graph_safe
+        ids = H.random_ids(61, 97, 8)
+        pos = torch.arange(len(ids))
+
+        def logits(dt):
+            def mix(at, layer, x):
+                if layer == 1:
+                    return _plain_attention(x, pos, w, "layers.1.mixer.", hq, hkv, d, eps, 1e4)[0]
+                weight = 1 + x[:, :1].float() ** 2
+                mean = (weight * x.float()).cumsum(0) / weight.cumsum(0)
+                return plain.linear(mean.to(dt), w[f"layers.{layer}.mixer.proj.weight"].to(dt))
+            return _plain_model(ids, w, dt, [0, 1, 2], eps, mix)
+        want, floor = logits(torch.float32), logits(torch.bfloat16)
+        for cuts, also in (([61], ()), ([29] + [1] * 32, ()), ([3, 2, 17, 9, 30], (H.random_ids(13, 97, 9),))):
+            _check_logits(_run_cut(cache, runner, ids, cuts, also), want, floor, dtype, f"two caches, cuts {cuts[:3]}")
+        assert all(g.pool.free == g.pool.usable for g in cache.groups)
+    finally:
+        unregister_part("mixer", "test-two-caches")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_ffn_with_stacked_expert_weights(device, dtype):
+    from tests.toy_parts import StackedTopOne
+    register_part("ffn", "test-stacked-top-one")(StackedTopOne)
+    try:
+        hq, hkv, d, eps, inter, experts = 4, 1, 16, 1e-6, 40, 3
+        spec = _spec([(_gqa(hq, hkv, d), PartRef("ffn", "test-stacked-top-one", inter=inter, experts=experts)),
+                      (_gqa(hq, hkv, d), PartRef("ffn", "swiglu", inter=96))])
+        model, w, cache, runner = _model(spec, device, dtype, 12, std=0.3)
+        assert model.blocks[0].ffn.gate_up.shape == (experts, 2 * inter, 64)
+        ids = H.random_ids(40, 97, 10)
+        pos = torch.arange(len(ids))
+
+        def logits(dt):
+            h = w["embed.weight"].to(dt)[torch.tensor(ids)]
+            for layer in (0, 1):
+                p = f"layers.{layer}."
+                x = plain.rms_norm(h, w[p + "input_norm.weight"].to(dt), eps)
+                h = h + _plain_attention(x, pos, w, p + "mixer.", hq, hkv, d, eps, 1e4)[0]
+                x = plain.rms_norm(h, w[p + "post_norm.weight"].to(dt), eps)
+                if layer == 1:
+                    h = h + _plain_ffn(x, w, p + "ffn.")
+                    continue
+                choice = (x.float() @ w[p + "ffn.router.weight"].to(dt).float().T).argmax(-1)
+                rows = []
+                for t in range(len(ids)):
+                    gu, down = w[p + "ffn.gate_up"][int(choice[t])].to(dt), w[p + "ffn.down"][int(choice[t])].to(dt)
+                    rows.append(plain.swiglu(x[t: t + 1], gu[:inter], gu[inter:], down)[0])
+                h = h + torch.stack(rows)
+            return plain.linear(plain.rms_norm(h, w["norm.weight"].to(dt), eps), w["lm_head.weight"].to(dt)).float()
+        want = logits(torch.float32)
+        for cuts in ([40], [8] + [1] * 32, [7, 2, 31]):
+            got = _run_cut(cache, runner, ids, cuts)
+            if dtype == torch.float32:
+                H.assert_fp32_close(got, want, f"stacked experts, cuts {cuts[:3]}")
+            else:     # a routed token may flip expert in bfloat16: compare the bulk
+                close = ((got - want).abs().amax(-1) / want.pow(2).mean().sqrt()) < 0.1
+                assert close.float().mean() > 0.9
+    finally:
+        unregister_part("ffn", "test-stacked-top-one")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_toy_architecture_through_the_engine_with_a_portion_grid_and_graphs_asked_for(device):
+    """A toy architecture registered here (its own config.json keys, recipe and mixer) generates through the engine.
+    Its mixer keeps a running sum in the request's slot, lets prompt portions end only on a grid of 8 positions (the
+    step budget of 13 does not fall on it) and plans on the host, so although graphs are asked for every step runs
+    eagerly. Greedy tokens equal a computation written out here from the plain functions."""
+    from holon_amd.config import EngineConfig, SamplingParams
+    from holon_amd.engine.engine import Engine
+    from holon_amd.registry import register_architecture, unregister_architecture
+    from tests.toy_parts import GridRunningMean, ToyConfig, toy_recipe
+    register_part("mixer", "test-grid-mean")(GridRunningMean)
+    register_architecture("ToyGridModel", ToyConfig, toy_recipe)
+    try:
+        config = {"architectures": ["ToyGridModel"], "width": 48, "tokens": 61, "depth": 2, "grid": 8, "eps": 1e-5}
+        engine = Engine.from_random(config, 3, EngineConfig(
+            model="random:toy", device=device, dtype="float32", page_size=4, max_seqs=3, max_model_len=64,
+            max_step_tokens=13, graphs=True, overlap=True), kernels=_kernels(device))
+        assert not engine.runner.use_graphs and engine.runner.not_graph_safe == ["GridRunningMean"]
+        assert engine.cache.prefix is None and not engine.cache.groups           # nothing paged, nothing shared
+        w = _weights_of(engine.model)
+
+        def greedy(ids, n):
+            ids, out = list(ids), []
+            for _ in range(n):
+                h = w["embed.weight"][torch.tensor(ids)]
+                for layer in (0, 1):
+                    p = f"layers.{layer}."
+                    x = plain.rms_norm(h, w[p + "input_norm.weight"], 1e-5)
+                    mean = x.cumsum(0) / torch.arange(1, len(ids) + 1)[:, None]
+                    h = h + plain.linear(mean, w[p + "mixer.proj.weight"])
+                    x = plain.rms_norm(h, w[p + "post_norm.weight"], 1e-5)
+                    gu = w[p + "ffn.gate_up.weight"]
+                    h = h + plain.swiglu(x, gu[:96], gu[96:], w[p + "ffn.down_proj.weight"])
+                logits = plain.linear(plain.rms_norm(h, w["norm.weight"], 1e-5), w["embed.weight"])
+                out.append(int(logits[-1].argmax()))
+                ids.append(out[-1])
+            return out
+        prompts = [H.random_ids(n, 61, 20 + n) for n in (30, 5, 21, 9)]
+        got = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True))
+        assert got == [greedy(p, 10) for p in prompts]
+        portions = engine.model.blocks[0].mixer.portions
+        assert (0, 8) in portions and (8, 8) in portions and (24, 6) in portions     # the prompt of 30: 8, 8, 8, 6
+        assert all(start % 8 == 0 for start, n in portions if n > 1)
+        with pytest.raises(ValueError, match="no prompt portion"):               # a budget that reaches no grid position
+            Engine.from_random(config, 3, EngineConfig(model="random:toy", device=device, dtype="float32", page_size=4,
+                                                       max_seqs=3, max_model_len=64, max_step_tokens=7),
+                               kernels=_kernels(device))
+    finally:
+        unregister_part("mixer", "test-grid-mean")
+        unregister_architecture("ToyGridModel")

@@ -35,10 +35,10 @@ def _commit(sched, cache, rows):
         cache.publish(seq.slot, seq.tokens)
         if m:
             if seq.status is not Status.RUNNING:
-                sched.finished_prefill(seq)
+                sched.prompt_done(seq)
             seq.tokens.append(0)
-            if sched.at_limit(seq):
-                sched.finish(seq, "length")
+            if seq.length_left(sched.max_model_len) == 0:
+                sched.retire(seq, "length")
 
 
 def test_prompts_are_cut_under_the_token_budget_in_arrival_order():
@@ -154,3 +154,29 @@ def test_every_request_finishes_under_random_traffic(seed, mode, prefix):
         assert cache.tokens_saved > 0
         cache.flush_prefix()
     assert all(g.pool.free == g.pool.usable for g in cache.groups) and cache.free_slots == cache.max_seqs
+
+
+def test_a_part_may_say_where_a_portion_ends():
+    """`cut`: a model whose state is kept on a grid of 8 positions lets a portion that does not end the prompt end
+    only there. The budget of 13 then carries 8 tokens of a long prompt; a prompt's end is free; a budget that reaches
+    no grid position carries nothing of that prompt and nobody skips ahead of it."""
+    def cut(start, count):
+        return (start + count) // 8 * 8 - start
+    cache = CacheManager([Site(run=0, layer=0)], [[PagedState("kv", 2)]], page_size=4, max_seqs=4, max_model_len=64,
+                         tokens=128, device=torch.device("cpu"), dtype=torch.float32)
+    sched = Scheduler(cache, 13, 64, cut=cut)
+    a, b = _seq("a", 30), _seq("b", 5)
+    sched.add(a), sched.add(b)
+    seen = []
+    for _ in range(6):
+        rows = sched.schedule()
+        seen.append([(s.rid, s.num_computed, n, m) for s, n, m in rows])
+        _commit(sched, cache, rows)
+    assert seen[:4] == [[("a", 0, 8, 0), ("b", 0, 5, 1)], [("a", 8, 8, 0)], [("a", 16, 8, 0)], [("a", 24, 6, 1)]]
+    sched = Scheduler(cache, 13, 64, chunk_with_decode=5, cut=cut)      # 5 tokens beside decode rows reach no edge from 8
+    c, d = _seq("c", 4), _seq("d", 30)
+    sched.add(c)
+    _commit(sched, cache, sched.schedule())
+    sched.add(d), sched.add(_seq("e", 3))
+    rows = sched.schedule()
+    assert [(s.rid, n) for s, n, _ in rows] == [("c", 1)]      # (the engine refuses such a budget when it starts)

@@ -106,3 +106,53 @@ def test_no_cpu_path_in_the_product(tmp_path):
     folder = write_random_model(CONFIG_A, 0, tmp_path / "m")
     with pytest.raises(RuntimeError, match="no CPU path"):
         load_model(folder, device="cpu", dtype="float32")
+
+
+def test_one_tensor_per_expert_fills_a_stacked_parameter(tmp_path):
+    """A rule with `stack` sends tensor `...experts.{e}...` to slice e of a parameter [experts, ...]; a missing
+    expert, one beyond the parameter and a wrong slice shape are all listed in the one error."""
+    from holon_amd.engine.loading import build_from_spec
+    from holon_amd.registry import register_part, unregister_part
+    from holon_amd.spec import LayerSpec, ModelSpec, PartRef, in_order
+    from holon_amd.weights.loader import checkpoint_names, load_weights, locate
+    from tests.toy_parts import STACKED_RULES, StackedTopOne
+    register_part("ffn", "test-stacked-top-one")(StackedTopOne)
+    try:
+        norm = PartRef("norm", "rmsnorm", eps=1e-6)
+        mixer = PartRef("mixer", "gqa", heads=2, kv_heads=1, head_dim=8)
+        layer = LayerSpec(PartRef("block", "prenorm"), mixer, PartRef("ffn", "test-stacked-top-one", inter=12, experts=3), norm)
+        spec = ModelSpec(hidden=16, vocab=20, layers=(layer,), order=in_order(1), embed=PartRef("embed", "table"),
+                         norm=norm, head=PartRef("head", "linear", tied=True), rules=STACKED_RULES)
+        assert locate(STACKED_RULES, "model.layers.0.mlp.experts.2.down.weight") == ("layers.0.ffn.down", 2)
+        assert checkpoint_names(STACKED_RULES, "layers.0.ffn.down", (3, 16, 12)) == [
+            (f"model.layers.0.mlp.experts.{e}.down.weight", e) for e in range(3)]
+        shape = dict(device=torch.device("cpu"), dtype=torch.float32, kernels=TorchKernels(), page_size=4, max_seqs=2,
+                     max_model_len=16, max_step_tokens=16)
+        model, _ = build_from_spec(spec, **shape)
+        g = torch.Generator().manual_seed(0)
+        tensors = {}
+        for path, _, _, decl in model.named_params():
+            for name, index in checkpoint_names(STACKED_RULES, path, decl.shape):
+                tensors[name] = torch.randn(decl.shape if index is None else decl.shape[1:], generator=g)
+        assert "model.layers.0.mlp.experts.1.gate_up.weight" in tensors and len(tensors) == 9 + 6
+        folder = tmp_path / "stacked"
+        folder.mkdir()
+        save_file(tensors, str(folder / "model.safetensors"))
+        load_weights(model, spec, folder, shape["device"], shape["dtype"])
+        ffn = model.blocks[0].ffn
+        for e in range(3):
+            assert torch.equal(ffn.gate_up[e], tensors[f"model.layers.0.mlp.experts.{e}.gate_up.weight"])
+            assert torch.equal(ffn.down[e], tensors[f"model.layers.0.mlp.experts.{e}.down.weight"])
+        broken = dict(tensors)
+        del broken["model.layers.0.mlp.experts.1.down.weight"]
+        broken["model.layers.0.mlp.experts.3.down.weight"] = torch.zeros(16, 12)
+        broken["model.layers.0.mlp.experts.0.gate_up.weight"] = torch.zeros(24, 15)
+        save_file(broken, str(folder / "model.safetensors"))
+        model, _ = build_from_spec(spec, **shape)
+        with pytest.raises(WeightError) as err:
+            load_weights(model, spec, folder, shape["device"], shape["dtype"])
+        assert err.value.missing == ["model.layers.0.mlp.experts.1.down.weight"]
+        assert err.value.unexpected == ["model.layers.0.mlp.experts.3.down.weight"]
+        assert err.value.wrong_shape == [("model.layers.0.mlp.experts.0.gate_up.weight", (24, 15), (24, 16))]
+    finally:
+        unregister_part("ffn", "test-stacked-top-one")
