@@ -72,6 +72,9 @@ int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, 
 int holon_gemm_skinny_add_bf16(const void* x, const void* w_tiled, void* residual, int M, int N, int K, void* stream);
 // y[M, I] = round(silu(round(x gate^T))) * round(x up^T) with w = [gate; up] ([2I, K]), M <= 32.
 int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int I, int K, int tiled, void* stream);
+// y[M, N] = x[M, K] w[N, K]^T, all float32, true 32-bit products and sums in an order that depends on K alone: a row's
+// result is bit for bit the same whatever other rows are in the call.
+int holon_gemm_f32(const void* x, const void* w, void* y, int M, int N, int K, void* stream);
 int holon_tile_weight_bf16(const void* w, void* tiled, int N, int K, void* stream);
 int holon_argmax(const float* logits, int32_t* out, int rows, int vocab, void* stream);
 // last_token[slots[r]] = tokens[r] for r < rows (slots are distinct; last_token has n_slots entries).

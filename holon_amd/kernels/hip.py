@@ -68,6 +68,7 @@ class HipKernels:
             "holon_gemm_skinny_supported": [_I, _I, _I],
             "holon_gemm_skinny_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
             "holon_tile_weight_bf16": [_P, _P, _I, _I, _P],
+            "holon_gemm_f32": [_P, _P, _P, _I, _I, _I, _P],
             "holon_gemm_skinny_add_bf16": [_P, _P, _P, _I, _I, _I, _P],
             "holon_gemm_skinny_glu_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
             "holon_argmax": [_P, _P, _I, _I, _P],
@@ -168,7 +169,14 @@ class HipKernels:
             self._call(self.lib.holon_gemm_skinny_bf16, x.data_ptr(), source.data_ptr(), y.data_ptr(), m, n, k,
                        int(to_f32), int(tiled is not None), self._stream())
             return y
-        # the vendor library's product, float32 accumulation (no reduced-precision mode for float32 operands)
+        if x.dtype == torch.float32 and weight.dtype == torch.float32 and out_dtype in (None, torch.float32):
+            # the 32-bit path's own product: true float32, every sum in an order that K alone decides
+            self._check(x, "linear x")
+            self._check(weight, "linear weight")
+            y = torch.empty((m, n), dtype=torch.float32, device=x.device)
+            self._call(self.lib.holon_gemm_f32, x.data_ptr(), weight.data_ptr(), y.data_ptr(), m, n, k, self._stream())
+            return y
+        # the vendor library's product of bfloat16 operands, float32 accumulation
         y = torch.matmul(x, weight.t())
         return y if out_dtype in (None, y.dtype) else y.to(out_dtype)
 

@@ -298,6 +298,29 @@ def test_linear(hip, dtype, monkeypatch):
     assert H.op_budget_usage(hip.linear(x[:1].contiguous(), w), hip.linear(x, w)[:1].float(), dtype, 4096) <= 1
 
 
+def test_float32_product_is_true_32_bit_and_its_order_is_fixed(hip):
+    """The 32-bit path's own product: close to the float64 product as only true float32 arithmetic is (a
+    reduced-precision matrix mode would be a thousand times off), at odd sizes (K no multiple of 4 or 32, N and M
+    off the tile edges), and bit for bit independent of the rows beside a row and of the row's place in the batch."""
+    f32 = torch.float32
+    for m, k, n in ((1, 64, 256), (5, 30, 97), (33, 33, 65), (70, 200, 120), (64, 4096, 64), (130, 72, 1000),
+                    (3, 12288, 4096), (257, 4096, 192)):
+        x, w = _randn(m, k, dtype=f32, seed=40), _randn(n, k, dtype=f32, seed=41, scale=0.05)
+        got, want = hip.linear(x, w), x.double() @ w.double().T
+        assert got.dtype == f32 and H.op_budget_usage(got, want, f32, k) <= 1, (m, k, n)
+        rel = ((got.double() - want).abs().max() / want.abs().max()).item()
+        assert rel < 2e-6 * max(1.0, (k / 64) ** 0.5), (m, k, n, rel)            # bfloat16 or tf32 operands give 1e-3
+        rows = torch.tensor(sorted({0, m // 2, m - 1}))
+        alone = hip.linear(x[rows.cuda()].contiguous(), w)                        # other company, other places
+        assert torch.equal(alone, got[rows.cuda()]), (m, k, n)
+        if m > 1:
+            shifted = hip.linear(torch.cat((x[-1:], x)).contiguous(), w)          # every row one place further down
+            assert torch.equal(shifted[1:], got), (m, k, n)
+    x = torch.randint(-1, 2, (7, 100), generator=torch.Generator().manual_seed(42)).float().cuda()
+    w = (torch.randint(-1, 2, (50, 100), generator=torch.Generator().manual_seed(43)).float() / 8).cuda()
+    assert torch.equal(hip.linear(x, w), x @ w.T)                                 # exact arithmetic: any order, same bits
+
+
 def test_fused_gate_up_is_the_two_kernels(hip, monkeypatch):
     for m, k, inter in ((1, 4096, 12288), (8, 4096, 12288), (16, 512, 208), (3, 1024, 1024), (5, 256, 48)):
         x = _randn(m, k, dtype=torch.bfloat16, seed=30)

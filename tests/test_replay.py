@@ -145,6 +145,60 @@ def test_logits_do_not_depend_on_the_cut_in_float32(folders, device):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name", ["A", "B", "C-sharp"])
+def test_float32_logits_are_bit_for_bit_the_same_however_they_are_cut(folders, name):
+    """In 32-bit every sum of the engine is taken in an order that the position alone decides (the product's order
+    depends on K alone, attention walks a query's keys from the first, norms work by row). So the logits at a
+    position are the same bits whole, with the last tokens one by one (from graphs too), in portions of changing
+    size, and mixed with other requests in a pool so small that pages are used again."""
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    folder, requests = folders[name], _requests(name)
+    whole = H.run_trace(_replayer(folder, name, "cuda", "float32", cache_tokens=96), H.trace_whole(requests))
+
+    def same(got, what):
+        assert got.keys() <= whole.keys() and got
+        bad = [k for k in got if not torch.equal(got[k], whole[k])]
+        assert not bad, f"{name} {what}: {len(bad)} of {len(got)} positions differ in their bits, first {min(bad)}"
+    for rid in ("r1", "r3"):
+        rep = _replayer(folder, name, "cuda", "float32", cache_tokens=96)
+        same(H.run_trace(rep, H.trace_decode_tail(rid, requests[rid], 32)), f"decode tail {rid}")
+        same(H.run_trace(rep, H.trace_chunks(rid, requests[rid], [7, 2, 13, 3, 2, 30, 5])), f"portions {rid}")
+    loaded = load_model(folder, device="cuda", dtype="float32", page_size=MODELS[name][3], max_seqs=4,
+                        max_model_len=512, max_step_tokens=512, cache_tokens=96, graphs=True)
+    same(H.run_trace(Replayer(loaded), H.trace_decode_tail("r3", requests["r3"], 40)), "decode tail from graphs")
+    assert loaded.runner.graph_replays >= 30
+    for seed in (0, 1):
+        trace = H.trace_mixed(requests, seed)
+        rep = _replayer(folder, name, "cuda", "float32", cache_tokens=H.peak_live_tokens(trace, 64))
+        got = H.run_trace(rep, trace)
+        assert len(got) == sum(LENGTHS)
+        same(got, f"mixed seed {seed}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("head_dim", [64, 80])
+def test_float32_stays_within_its_budget_at_1700_tokens(tmp_path, head_dim):
+    """A sharp model (q/k norm weights times 3) over a 1,700-token prompt, whole and in portions that end off the page
+    edges: the 32-bit engine stays within the same budget of the plain 32-bit model as at 300 tokens. (Both are then
+    about 7e-5 from the same formulas in float64: the rotation angle position * frequency is a float32 product in the
+    reference's formula, 1e-4 rad off at these positions, and the engine and the plain model share it.)"""
+    cfg = dict(H.CONFIG_C, head_dim=head_dim, max_position_embeddings=2048)
+    folder = H.make_folder(tmp_path / "m", cfg, 21, qk_gain=3.0)
+    ids = H.random_ids(1700, cfg["vocab_size"], 5)
+    want = PlainQwen3(folder).logits(ids)
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    loaded = load_model(folder, device="cuda", dtype="float32", page_size=16, max_seqs=2, max_model_len=2048,
+                        max_step_tokens=2048, cache_tokens=1712)
+    rep = Replayer(loaded)
+    whole = H.run_trace(rep, H.trace_whole({"r": ids}))
+    H.assert_fp32_close(torch.stack([whole[("r", i)] for i in range(1700)]), want, f"1,700 tokens whole, head_dim {head_dim}")
+    parts = H.run_trace(rep, H.trace_chunks("r", ids, [501, 2, 333, 700, 17]))
+    assert all(torch.equal(parts[k], whole[k]) for k in whole)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_the_trace_run_program(folders, tmp_path, dtype):
     """bin/trace_run as a user runs it: steps on standard input, `done <step>` lines, logits files [wanted, vocab] as
