@@ -26,6 +26,16 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8_t*>(p); }
 
+// Values are fetched 32 keys at a time, so the last block of a row reaches past its last key: into slots of the page
+// that an earlier request may have left anything in, or into the null page. Their probabilities are zero, but zero
+// times a NaN or an infinity is a NaN in the value product: such values are replaced by zeros. `v` holds keys
+// first_key .. first_key + 7.
+__device__ __forceinline__ void zero_after(bf16x8_t& v, int first_key, int key_hi) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    if (first_key + i > key_hi) v[i] = (__bf16)0.f;
+}
+
 struct AttnArgs {
   const bf16_t* q;         // [T, Hq, D]
   bf16_t* out;             // [T, Hq, D]
@@ -150,6 +160,10 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
     bf16x8_t vf[D / 16];
 #pragma unroll
     for (int ds = 0; ds < D / 16; ++ds) vf[ds] = load8(vrowp + (int64_t)ds * 16 * P);
+    if (kb + 31 > key_hi) {
+#pragma unroll
+      for (int ds = 0; ds < D / 16; ++ds) zero_after(vf[ds], kb + 8 * g, key_hi);
+    }
     bf16x8_t nf0[D / 32], nf1[D / 32];
     const bool more = kb + 32 <= key_hi;
     if (more) load_keys(kb + 32, nf0, nf1);
@@ -438,7 +452,8 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
         }
 #pragma unroll
         for (int ds = 0; ds < D / 16; ++ds) {
-          const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(ds * 16 + c) * VP + 8 * g]);
+          bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(ds * 16 + c) * VP + 8 * g]);
+          if (kb + 31 > key_hi) zero_after(vf, kb + 8 * g, key_hi);
 #pragma unroll
           for (int t = 0; t < NT; ++t) {
             if (kb > tile_last[t]) continue;
@@ -633,6 +648,10 @@ __global__ void __launch_bounds__(256) attn_prefill_wide_kernel(AttnArgs a) {
         for (int db = 0; db < D / 32; ++db) {
           vf[db][0] = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(db * 32 + c) * VP + 8 * h]);
           vf[db][1] = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(db * 32 + c) * VP + 16 + 8 * h]);
+          if (kb + 31 > key_hi) {
+            zero_after(vf[db][0], kb + 8 * h, key_hi);
+            zero_after(vf[db][1], kb + 16 + 8 * h, key_hi);
+          }
         }
         // value idx = 4i + r of this lane is key kb + 16*(i/2) + 8h + 4*(i%2) + r against query column c
         const int first = a.window > 0 ? qpos - a.window + 1 : 0;

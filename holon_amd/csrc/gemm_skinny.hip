@@ -20,7 +20,7 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 template <int MT, int WPB, int UNROLL, typename OutT, bool TILED, bool RESID = false>
 __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                 const bf16_t* __restrict__ w, OutT* __restrict__ y,
-                                                                int M, int N, int K) {
+                                                                int M, int N, int K, int round_first) {
   __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * MT * WAVE : 1];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
@@ -91,7 +91,12 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
     if (m >= M) continue;
     OutT* yp = y + (int64_t)m * N + n0 + 4 * g;
     if constexpr (sizeof(OutT) == 4) {
-      *reinterpret_cast<f32x4_t*>(yp) = acc[t];
+      f32x4_t o = acc[t];
+      if (round_first) {        // the bfloat16 product, widened: what the vendor product of more rows gives, cast up
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = bf16_to_float(float_to_bf16(o[r]));
+      }
+      *reinterpret_cast<f32x4_t*>(yp) = o;
     } else {
       ushort4 o;
       o.x = float_to_bf16(acc[t][0]); o.y = float_to_bf16(acc[t][1]);
@@ -109,23 +114,25 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
 }
 
 template <int MT, int WPB, int UNROLL, typename OutT, bool RESID>
-static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s) {
+static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s,
+                          int round_first) {
   const dim3 grid(N / 16), block(WPB * 64);
   if constexpr (RESID)
     gemm_skinny_kernel<MT, WPB, UNROLL, OutT, true, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                                (OutT*)y, M, N, K);
+                                                                                (OutT*)y, M, N, K, round_first);
   else if (tiled)
     gemm_skinny_kernel<MT, WPB, UNROLL, OutT, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                          (OutT*)y, M, N, K);
+                                                                          (OutT*)y, M, N, K, round_first);
   else
     gemm_skinny_kernel<MT, WPB, UNROLL, OutT, false><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                           (OutT*)y, M, N, K);
+                                                                           (OutT*)y, M, N, K, round_first);
 }
 
 // How many waves share a tile, from the shapes alone (so a result never depends on M): wide outputs have tiles
 // enough to fill the GPU with few waves each and long loops; narrow ones split K 16 ways. Measured on MI355X.
 template <int MT, typename OutT, bool RESID = false>
-static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s) {
+static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s,
+                      int round_first = 0) {
   const int tiles = N / 16;
   int wpb = MT >= 3 ? 8 : 16;                  // 16 waves of 3 or 4 token tiles run out of registers
   if (tiles >= 1024) wpb = 4;
@@ -133,15 +140,15 @@ static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K
   constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
   switch (wpb) {
     case 16:
-      if constexpr (MT < 3) launch_skinny<MT, 16, U, OutT, RESID>(x, w, y, M, N, K, tiled, s);
+      if constexpr (MT < 3) launch_skinny<MT, 16, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first);
       break;
-    case 8: launch_skinny<MT, 8, U, OutT, RESID>(x, w, y, M, N, K, tiled, s); break;
+    case 8: launch_skinny<MT, 8, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first); break;
     case 4:
-      if constexpr (MT == 1) launch_skinny<MT, 4, 16, OutT, RESID>(x, w, y, M, N, K, tiled, s);
-      else launch_skinny<MT, 4, U, OutT, RESID>(x, w, y, M, N, K, tiled, s);
+      if constexpr (MT == 1) launch_skinny<MT, 4, 16, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first);
+      else launch_skinny<MT, 4, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first);
       break;
-    case 2: launch_skinny<MT, 2, U, OutT, RESID>(x, w, y, M, N, K, tiled, s); break;
-    default: launch_skinny<MT, 1, U, OutT, RESID>(x, w, y, M, N, K, tiled, s); break;
+    case 2: launch_skinny<MT, 2, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first); break;
+    default: launch_skinny<MT, 1, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first); break;
   }
   return 0;
 }
@@ -150,7 +157,8 @@ extern "C" int holon_gemm_skinny_supported(int M, int N, int K) {
   return M >= 1 && M <= 64 && N % 16 == 0 && K % 32 == 0 && K >= 32;
 }
 
-// out_f32: 1 writes float32, 0 bfloat16. tiled: 1 when `w` is in the tile layout (see holon_tile_weight_bf16).
+// out_f32: 0 writes bfloat16, 1 float32 straight from the accumulators, 2 float32 values that were rounded to bfloat16
+// first (the product in the operands' type, cast up). tiled: 1 when `w` is in the tile layout (see holon_tile_weight_bf16).
 extern "C" int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_f32,
                                       int tiled, void* stream) {
   HOLON_CHECK(holon_gemm_skinny_supported(M, N, K), "gemm (few rows): M=%d N=%d K=%d not served (M <= 64, N %% 16, K %% 32)",
@@ -158,7 +166,7 @@ extern "C" int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int
   hipStream_t s = (hipStream_t)stream;
   const int mt = (M + 15) / 16;
 #define SKINNY(MT)                                                                 \
-  if (out_f32) pick_waves<MT, float>(x, w, y, M, N, K, tiled != 0, s);              \
+  if (out_f32) pick_waves<MT, float>(x, w, y, M, N, K, tiled != 0, s, out_f32 == 2); \
   else pick_waves<MT, bf16_t>(x, w, y, M, N, K, tiled != 0, s)
   if (mt == 1) { SKINNY(1); } else if (mt == 2) { SKINNY(2); } else if (mt == 3) { SKINNY(3); } else { SKINNY(4); }
 #undef SKINNY

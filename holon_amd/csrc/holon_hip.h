@@ -62,7 +62,8 @@ int holon_attention_decode_bf16_static(const void* q, void* out, const void* pag
                                        const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
                                        int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
                                        int splits, int keys_per_split, void* stream);
-// y[M, N] = x[M, K] w[N, K]^T for M <= 64 rows, bfloat16 in, float32 accumulation; out_f32 picks the output type;
+// y[M, N] = x[M, K] w[N, K]^T for M <= 64 rows, bfloat16 in, float32 accumulation; out_f32: 0 bfloat16 out, 1 float32
+// out, 2 float32 out of values rounded to bfloat16 first;
 // tiled says that `w` is holon_tile_weight_bf16's copy ([N/16, K/32, 64, 8]: lane-major 16-byte pieces).
 int holon_gemm_skinny_supported(int M, int N, int K);
 int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_f32, int tiled,

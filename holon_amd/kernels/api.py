@@ -57,8 +57,9 @@ class Kernels(Protocol):
 
     def linear(self, x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None = None,
                tiled: torch.Tensor | None = None) -> torch.Tensor:
-        """x [T, K] @ weight [N, K].T -> [T, N], float32 accumulation, rounded to out_dtype (default: x's).
-        `tiled`: what `tile_weight(weight)` returned, if anything."""
+        """x [T, K] @ weight [N, K].T -> [T, N], float32 accumulation, rounded to x's dtype; with another `out_dtype`
+        that rounded product is then cast (the reference's `F.linear(...).float()`, std/holon_std/ops/units.py:348): one
+        rule for every number of rows. `tiled`: what `tile_weight(weight)` returned, if anything."""
 
     def tile_weight(self, weight: torch.Tensor) -> torch.Tensor | None:
         """Once per weight after loading: a copy in the layout steps of few rows stream fastest, or None."""

@@ -163,11 +163,11 @@ class HipKernels:
             raise KernelError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(weight.shape)}")
         if (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows and k >= 256
                 and x.is_contiguous() and weight.is_contiguous() and self.lib.holon_gemm_skinny_supported(m, n, k)):
-            to_f32 = out_dtype == torch.float32
+            to_f32 = out_dtype == torch.float32       # then: the bfloat16 product cast up, as for any number of rows
             y = torch.empty((m, n), dtype=torch.float32 if to_f32 else torch.bfloat16, device=x.device)
             source = tiled if tiled is not None else weight
             self._call(self.lib.holon_gemm_skinny_bf16, x.data_ptr(), source.data_ptr(), y.data_ptr(), m, n, k,
-                       int(to_f32), int(tiled is not None), self._stream())
+                       2 if to_f32 else 0, int(tiled is not None), self._stream())
             return y
         if x.dtype == torch.float32 and weight.dtype == torch.float32 and out_dtype in (None, torch.float32):
             # the 32-bit path's own product: true float32, every sum in an order that K alone decides

@@ -59,7 +59,7 @@ class TorchKernels:
         return None
 
     def linear(self, x, weight, out_dtype=None, tiled=None):
-        return (_up(x) @ _up(weight).T).to(out_dtype or x.dtype)
+        return (_up(x) @ _up(weight).T).to(x.dtype).to(out_dtype or x.dtype)      # rounded to x's dtype, then cast
 
     def linear_add(self, x, weight, tiled, residual):
         residual.copy_((_up(residual) + _up(self.linear(x, weight))).to(residual.dtype))

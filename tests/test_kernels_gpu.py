@@ -142,6 +142,31 @@ def test_paged_attention(hip, dtype, page, geometry):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geometry", [(32, 8, 128), (6, 3, 32), (8, 2, 64), (32, 1, 64)])
+def test_attention_never_touches_what_lies_beyond_a_row(hip, dtype, geometry):
+    """Every cache slot that no row of the step holds a token in (the rest of a row's last page, pages of other
+    requests, spare pages) is filled with NaN: a kernel that lets such a slot into a product, even with weight zero,
+    gives NaN. Decode rows, short portions and portions long enough for the kernels that stage through LDS."""
+    heads, kv_heads, head_dim = geometry
+    page = 16
+    for rows in ([(0, 1), (14, 1), (16, 1), (99, 1), (1000, 1)], [(0, 17), (5, 16), (31, 33), (100, 7)],
+                 [(3, 700), (0, 530)]):
+        q, pages, table, attn = _paged_case(rows, heads, kv_heads, head_dim, page, dtype, seed=len(rows))
+        held = torch.zeros(pages.shape[0], page, dtype=torch.bool)
+        for slot, (s, n) in zip(attn.slots.tolist(), rows):
+            pos = torch.arange(s + n)
+            held[table[slot, pos // page].cpu().long(), pos % page] = True
+        kp, vp = pages[:, 0].view(-1, kv_heads, page, head_dim), pages[:, 1].view(-1, kv_heads, head_dim, page)
+        free = (~held).cuda()
+        kp.masked_fill_(free[:, None, :, None], float("nan"))
+        vp.masked_fill_(free[:, None, None, :], float("nan"))
+        want = PLAIN.paged_attention(q.double(), pages.double(), table, attn, page, head_dim ** -0.5, 0)
+        got = hip.paged_attention(q, pages, table, attn, page, head_dim ** -0.5, 0)
+        assert torch.isfinite(got.float()).all(), (geometry, rows)
+        assert H.op_budget_usage(got, want, dtype, head_dim + max(s + n for s, n in rows)) <= 1
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("geometry", [(32, 8, 128), (8, 2, 64)])
 def test_sixty_four_decode_rows(hip, dtype, geometry):
     """A decode step of 64 rows of unequal lengths (one key to 4,096, on and off page edges), with the launch shaped
@@ -280,6 +305,7 @@ def test_linear(hip, dtype, monkeypatch):
         assert got.dtype == dtype and H.op_budget_usage(got, want, dtype, k) <= 1, (t, k, n)
         got32 = hip.linear(x, w, torch.float32)
         assert got32.dtype == torch.float32 and H.op_budget_usage(got32, want, dtype, k) <= 1
+        assert torch.equal(got32, got.float())         # one rule for every number of rows: the product, then the cast
         tiled = hip.tile_weight(w)
         assert (tiled is None) == (dtype != torch.bfloat16 or n % 16 != 0 or k % 32 != 0 or k < 256)
         if tiled is not None:                          # the tile layout is a permutation: the same bits come out
