@@ -292,14 +292,23 @@ class CacheManager:
         return all(-(-total // self.page_size) <= g.pool.usable for g in self.groups)
 
     # -- per-step views -------------------------------------------------------------------------------------------
-    def upload(self) -> None:
-        """Copy the block-table rows that changed to the device (core/holon/core/state.py:51-58)."""
+    def take_dirty(self) -> list[tuple[PagedGroup, np.ndarray, np.ndarray]]:
+        """The block-table rows that changed since the last call, per group: (group, row numbers [n] int32, their new
+        contents [n, max_pages] int32). The caller brings them to the device with the step's other inputs and puts
+        them into `group.table_dev` (core/holon/core/state.py:51-58, 525-532: dirty rows ride the step's upload)."""
+        out = []
         for g in self.groups:
             if g.dirty:
-                rows = sorted(g.dirty)
-                idx = torch.tensor(rows, dtype=torch.long, device=self.device)
-                g.table_dev.index_copy_(0, idx, torch.from_numpy(g.table[rows]).to(self.device))
+                rows = np.fromiter(sorted(g.dirty), dtype=np.int32, count=len(g.dirty))
+                out.append((g, rows, g.table[rows]))
                 g.dirty.clear()
+        return out
+
+    def upload(self) -> None:
+        """Copy the block-table rows that changed to the device, by themselves (for callers outside a step)."""
+        for g, rows, contents in self.take_dirty():
+            idx = torch.from_numpy(rows.astype(np.int64)).to(self.device)
+            g.table_dev.index_copy_(0, idx, torch.from_numpy(contents).to(self.device))
 
     def write_targets(self, gid: int, slots: np.ndarray, positions: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
         """(page, offset) of each token's position in its request's pages (core/holon/core/state.py:541-554)."""

@@ -81,9 +81,15 @@ int holon_argmax(const float* logits, int32_t* out, int rows, int vocab, void* s
 // last_token[slots[r]] = tokens[r] for r < rows (slots are distinct; last_token has n_slots entries).
 int holon_store_tokens(int32_t* last_token, const int32_t* slots, const int32_t* tokens, int rows, int n_slots,
                        void* stream);
+// One token per row. Without `slots`, row r's parameters are temperature[r], top_k[r], ...; with `slots` ([rows]) they
+// are tables by slot and row r reads entry slots[r]. `positions` ([rows]: the position of the token being drawn) is
+// int32 when positions_i32 is set, int64 otherwise.
 int holon_sample(const float* logits, int32_t* out, int rows, int vocab, const float* temperature,
                  const int32_t* top_k, const float* top_p, const float* min_p, const int64_t* seeds,
-                 const int64_t* positions, void* stream);
+                 const void* positions, const int32_t* slots, int positions_i32, void* stream);
+// dst[idx[r], :] = src[r, :], rows of `width` int32 values; idx outside [0, dst_rows) is skipped.
+int holon_scatter_rows(int32_t* dst, const int32_t* idx, const int32_t* src, int rows, int width, int dst_rows,
+                       void* stream);
 
 // log_softmax of the raw logits: token_lp[r] for tokens[r], and the k (<= 32) largest with their ids, [rows, k].
 int holon_logprobs(const float* logits, const int32_t* tokens, int rows, int vocab, int k, float* token_lp,

@@ -79,6 +79,24 @@ extern "C" int holon_store_tokens(int32_t* last_token, const int32_t* slots, con
   return 0;
 }
 
+// dst[idx[r], :] = src[r, :] for rows of `width` int32 values: the block-table rows that changed since the last step,
+// brought with the step's other inputs, put into the device's table.
+__global__ void scatter_rows_kernel(int32_t* __restrict__ dst, const int32_t* __restrict__ idx,
+                                    const int32_t* __restrict__ src, int width, int dst_rows) {
+  const int r = blockIdx.x, to = idx[r];
+  if (to < 0 || to >= dst_rows) return;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[(int64_t)to * width + i] = src[(int64_t)r * width + i];
+}
+
+extern "C" int holon_scatter_rows(int32_t* dst, const int32_t* idx, const int32_t* src, int rows, int width,
+                                  int dst_rows, void* stream) {
+  HOLON_CHECK(rows >= 0 && width > 0 && dst_rows > 0, "scatter_rows: bad sizes");
+  if (rows == 0) return 0;
+  scatter_rows_kernel<<<rows, 256, 0, (hipStream_t)stream>>>(dst, idx, src, width, dst_rows);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
 // lowbias32, and the uniform of (seed, position): 24 bits, in (0, 1).
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {
   x ^= x >> 16; x *= 0x7FEB352Du; x ^= x >> 15; x *= 0x846CA68Bu; x ^= x >> 16;
@@ -552,7 +570,8 @@ __device__ u64 top_p_cut_wide(const float* __restrict__ row, int vocab, float in
 __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     const float* __restrict__ logits, int32_t* __restrict__ out, int vocab, const float* __restrict__ temperature,
     const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
-    const int64_t* __restrict__ seeds, const int64_t* __restrict__ positions) {
+    const int64_t* __restrict__ seeds, const void* __restrict__ positions, const int32_t* __restrict__ slots,
+    int positions_i32) {
   __shared__ u64 cand[SAMPLE_CANDIDATES];      // order keys of the collected tokens, sorted; later the sums of 256 tokens
   __shared__ int counts[SAMPLE_BANDS];
   __shared__ int band_counts[SAMPLE_WAVES][SAMPLE_BANDS];
@@ -560,7 +579,8 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
   __shared__ u64 z_k_s;
   const int r = blockIdx.x, tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const float* row = logits + (int64_t)r * vocab;
-  const float temp = temperature[r];
+  const int pr = slots != nullptr ? slots[r] : r;     // where this row's parameters lie: by its slot, or by its place
+  const float temp = temperature[pr];
   if (temp == 0.f) {
     const ArgMax a = block_argmax(row, vocab, 1.0f);
     if (tid == 0) out[r] = a.i;
@@ -569,9 +589,10 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
   const float inv_temp = 1.0f / temp;
   const ArgMax top = block_argmax(row, vocab, inv_temp);
   const float xmax = top.v;
-  const int k = top_k[r];
-  const float p_keep = top_p[r], p_min = min_p[r];
-  const float u = hashed_uniform((uint64_t)seeds[r], (uint64_t)positions[r]);
+  const int k = top_k[pr];
+  const float p_keep = top_p[pr], p_min = min_p[pr];
+  const uint64_t position = positions_i32 ? (uint64_t)((const int32_t*)positions)[r] : (uint64_t)((const int64_t*)positions)[r];
+  const float u = hashed_uniform((uint64_t)seeds[pr], position);
   const bool k_on = k > 0 && k < vocab, p_on = p_keep < 1.0f;
   const int chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
   if ((k_on && k > SAMPLE_CANDIDATES) || vocab > 255 * SAMPLE_THREADS) {      // (uniform over the block)
@@ -787,11 +808,11 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
 
 extern "C" int holon_sample(const float* logits, int32_t* out, int rows, int vocab, const float* temperature,
                             const int32_t* top_k, const float* top_p, const float* min_p, const int64_t* seeds,
-                            const int64_t* positions, void* stream) {
+                            const void* positions, const int32_t* slots, int positions_i32, void* stream) {
   HOLON_CHECK(rows >= 0 && vocab > 0, "sample: bad sizes");
   if (rows == 0) return 0;
   sample_kernel<<<rows, SAMPLE_THREADS, 0, (hipStream_t)stream>>>(logits, out, vocab, temperature, top_k, top_p,
-                                                                  min_p, seeds, positions);
+                                                                  min_p, seeds, positions, slots, positions_i32);
   HOLON_LAUNCH_OK();
   return 0;
 }

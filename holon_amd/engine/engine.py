@@ -324,11 +324,12 @@ class Engine:
         if sampled:
             slots = np.array([seq.slot for seq, _ in sampled], dtype=np.int64)
             positions = np.array([seq.num_computed + n for seq, n in sampled], dtype=np.int64)
-            drawn = self.sampler.sample(logits, slots, positions)
-            if len(sampled) == len(rows) and not owed:
+            if len(sampled) == len(rows) and not owed:       # every row draws: slots and positions are on the device
                 where = self.runner.last_slots[: len(rows)]
+                drawn = self.sampler.sample(logits, slots, positions, (where, self.runner.last_lens[: len(rows)]))
             else:
                 where = torch.from_numpy(slots.astype(np.int32)).to(self.device, non_blocking=True)
+                drawn = self.sampler.sample(logits, slots, positions)
             self.kernels.store_tokens(self.runner.last_token, where, drawn)
             k = max((seq.params.logprobs if seq.params.logprobs is not None else -1) for seq, _ in sampled)
             out.tokens = self._to_host(drawn)

@@ -48,6 +48,7 @@ class StepRunner:
         # the token last drawn for each slot, for a row whose token has not reached the host when it is scheduled
         self.last_token = torch.zeros(max_seqs + 1, dtype=torch.int32, device=device)
         self.last_slots: torch.Tensor | None = None       # the last step's rows' slots on the device
+        self.last_lens: torch.Tensor | None = None        # and how many tokens each then holds
         # a captured step is replayed without any part's Python code: only over parts that say they allow it
         self.not_graph_safe = sorted({type(p).__name__ for p in model.walk() if not p.graph_safe})
         self.use_graphs = graphs and device.type == "cuda" and not self.not_graph_safe
@@ -77,16 +78,22 @@ class StepRunner:
         for g in cache.groups:
             page, off = cache.write_targets(g.gid, slots[token_row], positions)
             arrays += [page, off]
-        facts = dict(total=total, n_rows=len(slots), n_decode=len(decode), n_chunk=len(chunk),
+        fixed = len(arrays)
+        dirty = cache.take_dirty()                  # block-table rows that changed: they ride the same copy
+        for _, rows, contents in dirty:
+            arrays += [rows, contents]
+        facts = dict(fixed=fixed, dirty=[(g, len(rows)) for g, rows, _ in dirty],
+                     total=total, n_rows=len(slots), n_decode=len(decode), n_chunk=len(chunk),
                      max_decode_len=int(lens[decode].max()) if len(decode) else 0,
                      max_chunk_query=int(counts[chunk].max()) if len(chunk) else 0,
                      max_chunk_len=int(lens[chunk].max()) if len(chunk) else 0)
         return arrays, facts
 
-    def _to_device(self, arrays: list[np.ndarray], arena: torch.Tensor | None = None, views: bool = True
+    def _to_device(self, arrays: list[np.ndarray], arena: torch.Tensor | None = None, first: int = 0
                    ) -> list[torch.Tensor]:
-        """Several int32 arrays to the device in one copy (into `arena`, a buffer of fixed address, when given). The
-        host side is one of two pinned buffers used in turn; a buffer is written again only after its last copy ran."""
+        """Several int32 arrays to the device in one copy (into `arena`, a buffer of fixed address, when given).
+        Returns views of arrays `first` onwards. The host side is one of two pinned buffers used in turn; a buffer
+        is written again only after its last copy ran."""
         sizes = [a.size for a in arrays]
         total = sum(sizes)
         if self.pinned:
@@ -108,13 +115,17 @@ class StepRunner:
             dev.copy_(host, non_blocking=True)
         if self.pinned:
             stage[1].record()
-        if not views:                              # a graph's step already holds its views of the arena
-            return []
         out, at = [], 0
-        for n in sizes:
-            out.append(dev[at: at + n])
+        for i, n in enumerate(sizes):
+            if i >= first:
+                out.append(dev[at: at + n])
             at += n
         return out
+
+    def _table_rows(self, dev: list[torch.Tensor], facts: dict) -> None:
+        """Put the changed block-table rows, now on the device, into the tables. `dev`: views from `facts["fixed"]` on."""
+        for i, (g, n) in enumerate(facts["dirty"]):
+            self.kernels.scatter_rows(g.table_dev, dev[2 * i], dev[2 * i + 1])
 
     def _step(self, dev: list[torch.Tensor], facts: dict, slots, starts, counts) -> Step:
         cache = self.cache
@@ -172,9 +183,10 @@ class StepRunner:
         """Device inputs of a step, and the flat indices of the tokens whose logits are wanted (in row order, then in
         the order of each row's `want`)."""
         slots, starts, counts, tokens, wanted, take = self._check(rows)
-        self.cache.upload()
         arrays, facts = self._arrays(slots, starts, counts, tokens, take)
-        return self._step(self._to_device(arrays), facts, slots, starts, counts), wanted
+        dev = self._to_device(arrays)
+        self._table_rows(dev[facts["fixed"]:], facts)
+        return self._step(dev, facts, slots, starts, counts), wanted
 
     # -- the step -------------------------------------------------------------------------------------------------
     def _forward(self, step: Step, wanted: np.ndarray | None) -> torch.Tensor | None:
@@ -195,7 +207,7 @@ class StepRunner:
             logits = self._run_graphed(rows)
         else:
             step, wanted = self.prepare(rows)
-            self.last_slots = step.slots
+            self.last_slots, self.last_lens = step.slots, step.lens
             logits = self._forward(step, wanted)
         for r in rows:
             self.cache.advance(r.slot, r.start + len(r.tokens))
@@ -216,20 +228,23 @@ class StepRunner:
             counts = np.concatenate((counts, np.ones(pad, dtype=np.int64)))
             tokens = np.concatenate((tokens, np.zeros(pad, dtype=np.int64)))
             take = np.concatenate((take, np.full(pad, -1, dtype=np.int64)))
-        self.cache.upload()
         arrays, facts = self._arrays(slots, starts, counts, tokens, take)
         facts["max_decode_len"] = len_bucket       # launch shapes are the bucket's, whatever the rows' lengths
         key = (bucket, len_bucket)
         g = self.graphs.get(key)
-        if g is None:
-            size = sum(a.size for a in arrays)
+        if g is None:                              # the step's inputs at a fixed address, then room for every table row
+            size = sum(a.size for a in arrays[: facts["fixed"]])
+            size += sum(gr.table.size + gr.table.shape[0] for gr in self.cache.groups)
             arena = torch.zeros(size, dtype=torch.int32, device=self.device)
-            g = _Graph(arena=arena, step=self._step(self._to_device(arrays, arena), facts, slots, starts, counts))
+            dev = self._to_device(arrays, arena)
+            g = _Graph(arena=arena, step=self._step(dev, facts, slots, starts, counts))
             self.graphs[key] = g
         else:
-            self._to_device(arrays, g.arena, views=False)
+            dev = self._to_device(arrays, g.arena)
+            g.step.h_slots, g.step.h_starts, g.step.h_counts = slots, starts, counts
+        self._table_rows(dev[facts["fixed"]:], facts)
         g.runs += 1
-        self.last_slots = g.step.slots[:n]
+        self.last_slots, self.last_lens = g.step.slots[:n], g.step.lens[:n]
         if g.graph is None and g.runs == 1:        # the first step of a bucket: eagerly, on the fixed buffers
             return self._forward(g.step, None)[:n]
         if g.graph is None:

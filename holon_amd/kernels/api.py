@@ -114,7 +114,12 @@ class Kernels(Protocol):
         their log-probabilities [R, k]); k <= 32; ties go to the lower id."""
 
     def sample(self, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-               min_p: torch.Tensor, seeds: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
-        """One token per row [R] int32. temperature/top_p/min_p float32 [R], top_k int32 [R], seeds int64 [R],
-        positions int64 [R] (the position of the token being drawn). Rows with temperature 0 take the argmax;
-        the others draw by inverse CDF in vocabulary order with the hashed uniform of (seed, position)."""
+               min_p: torch.Tensor, seeds: torch.Tensor, positions: torch.Tensor,
+               slots: torch.Tensor | None = None) -> torch.Tensor:
+        """One token per row [R] int32. temperature/top_p/min_p float32, top_k int32, seeds int64: [R], row r's own;
+        or, with `slots` [R] int32, tables [S] of which row r reads entry slots[r]. positions [R] int32 or int64 (the
+        position of the token being drawn). Rows with temperature 0 take the argmax; the others draw by inverse CDF
+        in vocabulary order with the hashed uniform of (seed, position)."""
+
+    def scatter_rows(self, dst: torch.Tensor, idx: torch.Tensor, src: torch.Tensor) -> None:
+        """dst[idx[r]] = src[r] for int32 rows: dst [N, W], idx [n], src n * W values."""

@@ -73,7 +73,8 @@ class HipKernels:
             "holon_gemm_skinny_glu_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
             "holon_argmax": [_P, _P, _I, _I, _P],
             "holon_store_tokens": [_P, _P, _P, _I, _I, _P],
-            "holon_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
+            "holon_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P],
+            "holon_scatter_rows": [_P, _P, _P, _I, _I, _I, _P],
             "holon_logprobs": [_P, _P, _I, _I, _I, _P, _P, _P, _P],
         }
         for name, args in sig.items():
@@ -341,17 +342,35 @@ class HipKernels:
                    token_lp.data_ptr(), top_ids.data_ptr(), top_lp.data_ptr(), self._stream())
         return token_lp, top_ids, top_lp
 
-    def sample(self, logits, temperature, top_k, top_p, min_p, seeds, positions):
+    def sample(self, logits, temperature, top_k, top_p, min_p, seeds, positions, slots=None):
         self._check(logits, "sample logits", torch.float32)
         r = logits.shape[0]
+        n = r
+        if slots is not None:                      # the parameters are tables by slot
+            self._check(slots, "sample slots", torch.int32)
+            if slots.shape != (r,):
+                raise KernelError(f"sample slots: shape {tuple(slots.shape)} for {r} rows")
+            n = temperature.shape[0]
         for t, dt, what in ((temperature, torch.float32, "temperature"), (top_k, torch.int32, "top_k"),
                             (top_p, torch.float32, "top_p"), (min_p, torch.float32, "min_p"),
-                            (seeds, torch.int64, "seeds"), (positions, torch.int64, "positions")):
+                            (seeds, torch.int64, "seeds")):
             self._check(t, f"sample {what}", dt)
-            if t.shape != (r,):
-                raise KernelError(f"sample {what}: shape {tuple(t.shape)} for {r} rows")
+            if t.shape != (n,):
+                raise KernelError(f"sample {what}: shape {tuple(t.shape)}, expected ({n},)")
+        if positions.dtype not in (torch.int32, torch.int64) or positions.shape != (r,):
+            raise KernelError(f"sample positions: {positions.dtype} {tuple(positions.shape)} for {r} rows")
+        self._check(positions, "sample positions")
         out = torch.empty((r,), dtype=torch.int32, device=logits.device)
         self._call(self.lib.holon_sample, logits.data_ptr(), out.data_ptr(), r, logits.shape[1],
                    temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), min_p.data_ptr(), seeds.data_ptr(),
-                   positions.data_ptr(), self._stream())
+                   positions.data_ptr(), _ptr(slots), int(positions.dtype == torch.int32), self._stream())
         return out
+
+    def scatter_rows(self, dst, idx, src):
+        for t, what in ((dst, "dst"), (idx, "idx"), (src, "src")):
+            self._check(t, f"scatter_rows {what}", torch.int32)
+        n, width = idx.shape[0], dst.shape[1]
+        if src.numel() != n * width:
+            raise KernelError(f"scatter_rows: {src.numel()} values for {n} rows of {width}")
+        self._call(self.lib.holon_scatter_rows, dst.data_ptr(), idx.data_ptr(), src.data_ptr(), n, width, dst.shape[0],
+                   self._stream())

@@ -134,7 +134,14 @@ class TorchKernels:
         order = lp.argsort(dim=-1, descending=True, stable=True)[:, :k]
         return lp.gather(-1, tokens.long()[:, None])[:, 0], order.to(torch.int32), lp.gather(-1, order)
 
-    def sample(self, logits, temperature, top_k, top_p, min_p, seeds, positions):
+    def scatter_rows(self, dst, idx, src):
+        dst[idx.long()] = src.view(idx.shape[0], dst.shape[1])
+
+    def sample(self, logits, temperature, top_k, top_p, min_p, seeds, positions, slots=None):
+        if slots is not None:
+            at = slots.long()
+            temperature, top_k, top_p, min_p, seeds = (t[at] for t in (temperature, top_k, top_p, min_p, seeds))
+        positions = positions.long()
         m = 0xFFFFFFFF
         h = _mix32(seeds & m) ^ ((seeds >> 32) & m) ^ _mix32(positions & m)
         h = _mix32(h)
