@@ -6,8 +6,11 @@
     python bench.py --workload mixed|long [--layers L]
 
 One JSON line: decoded tokens a second at the given batch (default 8) with every request near a context of 4,096 tokens
-(a 2,048-token prompt and 2,048 generated tokens), plus the prefill of one 2,048-token prompt, the decode step's memory
-roofline, and decode at batch 1 and 64. A step is one decode step of the engine: scheduling, the model, sampling and
+(the far end of a 2,048-token prompt and 2,048 generated tokens: the requests are given prompts that leave just the
+timed steps, `config.decode_prompt_len`), plus the prefill of one 2,048-token prompt, the decode step's memory
+roofline, decode at batch 1 and 64 with their step times and roofline fractions (`points`), and the time to the first
+token of the 2,048-token prompt and the median time between two tokens of a request (`latency`, as the reference's
+driver reports them: bench/driver.py:102-134). A step is one decode step of the engine: scheduling, the model, sampling and
 the commit. The engine is one process on one GPU; for --gpus > 1 a line says so and the exit code is 2.
 
 --workload runs a whole job through the engine instead and prints its own line: `mixed` is 32 requests of 128 to 4,096
@@ -125,8 +128,9 @@ def main(argv: list[str] | None = None) -> int:
     g = torch.Generator().manual_seed(0)
     greedy = lambda n: SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True)
 
-    def decode(batch: int, steps: int, warmup: int) -> tuple[float, float]:
-        """(ms per decode step, mean context) for `batch` requests whose contexts end at CONTEXT."""
+    def decode(batch: int, steps: int, warmup: int) -> tuple[float, float, float, int]:
+        """(ms per decode step, mean context, median ms between two steps' ends, prompt length) for `batch` requests
+        whose contexts end at CONTEXT."""
         start = CONTEXT - steps - warmup - 1
         for _ in range(batch):
             engine.add(torch.randint(0, c["vocab_size"], (start,), generator=g).tolist(), greedy(steps + warmup + 1))
@@ -136,16 +140,20 @@ def main(argv: list[str] | None = None) -> int:
             engine.step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
+        ends = []
         for _ in range(steps):
-            engine.step()
+            engine.step()                      # returns when the step before has been committed: one step's time apart
+            ends.append(time.perf_counter())
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) * 1e3 / steps
+        gaps = sorted(b - a for a, b in zip(ends, ends[1:])) or [ms * 1e-3]
         while engine.has_work():
             engine.step()
-        return ms, start + 1 + warmup + steps / 2
+        return ms, start + 1 + warmup + steps / 2, gaps[len(gaps) // 2] * 1e3, start
 
-    def prefill(tokens: int) -> float:
-        best = float("inf")
+    def prefill(tokens: int) -> tuple[float, float]:
+        """(best, median) ms from adding a prompt of `tokens` to its first generated token on the host."""
+        times = []
         for _ in range(3):                     # another prompt each time: nothing of it is in the prefix cache
             ids = torch.randint(0, c["vocab_size"], (tokens,), generator=g).tolist()
             engine.add(ids, greedy(1))
@@ -154,25 +162,28 @@ def main(argv: list[str] | None = None) -> int:
             engine.step()
             engine.drain()                     # the step's one token on the host: the request is finished
             torch.cuda.synchronize()
-            best = min(best, (time.perf_counter() - t0) * 1e3)
+            times.append((time.perf_counter() - t0) * 1e3)
             assert not engine.has_work()
-        return best
+        return min(times), sorted(times)[1]
 
     h, hq, hkv, d, inter, v, layers = (c["hidden_size"], c["num_attention_heads"], c["num_key_value_heads"],
                                        c["head_dim"], c["intermediate_size"], c["vocab_size"], a.layers)
     layer_params = h * (hq + 2 * hkv) * d + hq * d * h + 3 * h * inter
     weight_bytes = (layers * (layer_params + 2 * h + 2 * d) + h + h * v) * item      # every weight a decode step reads
     kv_token_bytes = layers * 2 * hkv * d * item
-    pre_ms = prefill(PROMPT)
+    pre_ms, ttft_ms = prefill(PROMPT)
     pre_flops = layers * (2 * PROMPT * layer_params + 2 * hq * d * PROMPT * PROMPT) + 2 * h * v
-    ms, ctx = decode(a.batch, a.steps, a.warmup)
+    ms, ctx, tpot_ms, decode_prompt = decode(a.batch, a.steps, a.warmup)
     step_bytes = weight_bytes + a.batch * ctx * kv_token_bytes
     achieved = step_bytes / (ms * 1e-3) / 1e9
     points = {}
     if not a.no_points:
         for b in (1, 64):
-            pms, _ = decode(b, a.steps, a.warmup)
+            pms, pctx, _, _ = decode(b, a.steps, a.warmup)
             points[f"decode_b{b}"] = round(b / (pms * 1e-3), 1)
+            points[f"decode_b{b}_ms"] = round(pms, 4)
+            points[f"decode_b{b}_gb"] = round((weight_bytes + b * pctx * kv_token_bytes) / 1e9, 2)
+            points[f"decode_b{b}_frac"] = round((weight_bytes + b * pctx * kv_token_bytes) / (pms * 1e-3) / 1e9 / HBM_GBS, 4)
     line = {
         "metric": f"decode tok/s at batch {a.batch} (context 4,096), Qwen3-8B shape", "value": round(a.batch / (ms * 1e-3), 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
@@ -180,13 +191,16 @@ def main(argv: list[str] | None = None) -> int:
         "data": "synthetic (random weights, uniform random token ids)",
         "config": {"model": "Qwen3-8B shape", "layers": layers, "layers_of_config": QWEN3_8B["num_hidden_layers"],
                    "hidden": h, "heads": hq, "kv_heads": hkv, "head_dim": d, "intermediate": inter, "vocab": v,
-                   "tied": False, "global_batch": a.batch, "seq_len": CONTEXT, "prompt_len": PROMPT, "page_size": 16,
+                   "tied": False, "global_batch": a.batch, "seq_len": CONTEXT, "prefill_tokens": PROMPT,
+                   "decode_prompt_len": decode_prompt, "page_size": 16,
                    "parallelism": "single GPU", "graphs": not a.no_graphs, "mean_context": round(ctx, 1)},
         "prefill": {"value": round(PROMPT / (pre_ms * 1e-3), 1), "tokens": PROMPT, "ms": round(pre_ms, 3),
                     "frac": round(pre_flops / (pre_ms * 1e-3) / PEAK_FLOPS[a.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},
         "points": points,
+        "latency": {"ttft_ms_p50": round(ttft_ms, 3), "ttft_tokens": PROMPT, "tpot_ms_p50": round(tpot_ms, 4),
+                    "tpot_batch": a.batch},
     }
     if engine.stats()["prefix_tokens_saved"]:
         raise RuntimeError("the prefix cache served part of a timed prompt: the figures above would count work not done")

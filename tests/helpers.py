@@ -103,6 +103,21 @@ def assert_bf16_close(got: torch.Tensor, want32: torch.Tensor, floor16: torch.Te
         f"{what}: bfloat16 logits differ: rms {r:.3g} (floor {fr:.3g}), max {m:.3g} (floor {fm:.3g})"
 
 
+def assert_greedy_follows(plain, prompt: list[int], got: list[int], margin: float = 0.05) -> int:
+    """Every generated token is the plain model's most likely one given the tokens before it, wherever the plain
+    model's two best logits are further apart than `margin` of the logits' spread (closer than that, rounding may
+    decide). Returns how many tokens were held to the plain model's choice."""
+    ids, held = list(prompt), 0
+    for token in got:
+        logits = plain.logits(ids)[-1].float()
+        top = logits.topk(2).values
+        if float(top[0] - top[1]) > margin * float(logits.std()):
+            assert token == int(logits.argmax()), f"token {len(ids)}: {token}, the plain model says {int(logits.argmax())}"
+            held += 1
+        ids.append(token)
+    return held
+
+
 # -- traces -------------------------------------------------------------------------------------------------------
 class Trace:
     """Steps for the replayer, and for each step the (request, position) of every wanted logit row."""

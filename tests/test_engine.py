@@ -314,19 +314,15 @@ def test_rejections_and_limits(folders, device):
 
 @pytest.mark.gpu
 def test_bfloat16_generation_stays_with_the_plain_model(folders):
-    """In bfloat16 a near-tie may flip a token; every token the engine picks must be within the rounding floor of the
-    plain model's best at that place, and the first token of a clear-cut prompt is the plain one."""
-    plain32, plain16 = PlainQwen3(folders["Bu"]), PlainQwen3(folders["Bu"], torch.bfloat16)
+    """In bfloat16 rounding may decide between two tokens whose logits nearly tie, and only there: every token the
+    engine picks is the most likely one of the plain model run in bfloat16 on the same tokens, wherever that model's
+    two best logits are further apart than a twentieth of the logits' spread. Most places are that clear."""
+    plain16 = PlainQwen3(folders["Bu"], torch.bfloat16)
     prompts = [H.random_ids(n, 384, 40 + n) for n in (5, 17, 33)]
     engine = _engine(folders["Bu"], "cuda", dtype="bfloat16", page_size=16, max_seqs=3, max_model_len=64)
     out = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16, ignore_eos=True))
-    for prompt, tokens in zip(prompts, out):
-        ids = list(prompt)
-        for t in tokens:
-            want, floor = plain32.logits(ids)[-1], plain16.logits(ids)[-1]
-            margin = 2 * (floor - want).abs().max().item() + 1e-3
-            assert want[t] >= want.max() - 2 * margin
-            ids.append(t)
+    held = sum(H.assert_greedy_follows(plain16, prompt, tokens) for prompt, tokens in zip(prompts, out))
+    assert held >= 36, f"only {held} of 48 places were clear enough to hold the engine to"
 
 
 @pytest.mark.gpu

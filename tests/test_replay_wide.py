@@ -136,18 +136,6 @@ def test_sixty_four_rows_decode_together_from_graphs(folder, dtype):
     assert all(g.pool.free == g.pool.usable for g in rep.cache.groups)
 
 
-def _greedy_follows_the_plain_model(plain, prompt, got, margin=0.05) -> None:
-    """Every generated token is the plain model's most likely one given the tokens before it, wherever the plain
-    model's two best logits are further apart than bfloat16 rounding reaches."""
-    ids = list(prompt)
-    for token in got:
-        logits = plain.logits(ids)[-1].float()
-        top = logits.topk(2).values
-        if float(top[0] - top[1]) > margin * float(logits.std()):
-            assert token == int(logits.argmax()), (len(ids), token)
-        ids.append(token)
-
-
 def test_engine_at_the_wide_sizes_with_everything_on(folder):
     """The whole engine in bfloat16 at the measured layer sizes (matrix-core attention, the few-row products over
     tiled weights, the residual add and the gated form inside them). One step in flight changes no launch, so it must
@@ -170,7 +158,7 @@ def test_engine_at_the_wide_sizes_with_everything_on(folder):
     params = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
     for _ in range(2):                                           # the second time the prompts come from the cache
         for prompt, got in zip(prompts, full.generate(prompts, params)):
-            _greedy_follows_the_plain_model(plain, prompt, got)
+            H.assert_greedy_follows(plain, prompt, got)
     assert full.cache.tokens_saved > 0 and full.stats()["graphs"] >= 1 and full.runner.graph_replays > 10
 
 
