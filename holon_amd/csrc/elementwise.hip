@@ -9,7 +9,7 @@
 template <typename T>
 __global__ void embedding_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ take_slot,
                                  const int32_t* __restrict__ last_token, const T* __restrict__ table,
-                                 T* __restrict__ out, int hidden, int vocab) {
+                                 T* __restrict__ out, int hidden, int vocab, float* __restrict__ stats_out) {
   const int64_t t = blockIdx.x;
   int id = ids[t];
   if (take_slot != nullptr && take_slot[t] >= 0) id = last_token[take_slot[t]];
@@ -24,21 +24,58 @@ __global__ void embedding_kernel(const int32_t* __restrict__ ids, const int32_t*
   } else {
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
   }
+  if (stats_out != nullptr) {     // the row's sum of squares, for a norm folded into the product that reads the row
+    __shared__ float part[4];
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float v = Elem<T>::load(src[i]);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    if (threadIdx.x % WAVE == 0) part[threadIdx.x / WAVE] = ss;
+    __syncthreads();
+    if (threadIdx.x == 0) stats_out[t] = ((part[0] + part[1]) + part[2]) + part[3];
+  }
 }
 
+// stats[0][m] = sum of squares of row m (m < rows <= 16): one wave per row.
+template <typename T>
+__global__ void row_sumsq_kernel(const T* __restrict__ x, float* __restrict__ stats, int rows, int dim) {
+  const int row = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  float ss = 0.f;
+  if (row < rows)
+    for (int i = lane; i < dim; i += WAVE) {
+      const float v = Elem<T>::load(x[(int64_t)row * dim + i]);
+      ss += v * v;
+    }
+  ss = wave_sum(ss);
+  if (lane == 0) stats[row] = ss;
+}
+
+extern "C" int holon_row_sumsq(const void* x, float* stats, int rows, int dim, int dtype, void* stream) {
+  HOLON_CHECK(rows >= 0 && rows <= 16 && dim > 0, "row_sumsq: %d rows of %d (at most 16 rows)", rows, dim);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HOLON_F32) row_sumsq_kernel<float><<<1, 16 * WAVE, 0, s>>>((const float*)x, stats, rows, dim);
+  else row_sumsq_kernel<bf16_t><<<1, 16 * WAVE, 0, s>>>((const bf16_t*)x, stats, rows, dim);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+// stats_out (nullable, tokens <= 16): [16] float32, the sum of squares of every row written.
 extern "C" int holon_embedding(const int32_t* ids, const int32_t* take_slot, const int32_t* last_token,
                                const void* table, void* out, int tokens, int hidden, int vocab, int dtype,
-                               void* stream) {
+                               float* stats_out, void* stream) {
   HOLON_CHECK(tokens >= 0 && hidden > 0 && vocab > 0, "embedding: bad sizes tokens=%d hidden=%d", tokens, hidden);
   HOLON_CHECK((take_slot == nullptr) == (last_token == nullptr), "embedding: slots to take tokens from need the tokens");
+  HOLON_CHECK(stats_out == nullptr || tokens <= 16, "embedding: row sums for at most 16 tokens, not %d", tokens);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == HOLON_F32)
     embedding_kernel<float><<<tokens, 256, 0, s>>>(ids, take_slot, last_token, (const float*)table, (float*)out,
-                                                   hidden, vocab);
+                                                   hidden, vocab, stats_out);
   else
     embedding_kernel<bf16_t><<<tokens, 256, 0, s>>>(ids, take_slot, last_token, (const bf16_t*)table, (bf16_t*)out,
-                                                    hidden, vocab);
+                                                    hidden, vocab, stats_out);
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -15,13 +15,42 @@
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
+// A norm folded into the product that reads it. With RMSNorm y = x * rsqrt(mean(x^2) + eps) * g in front of a product
+// with W, the product of the un-normed rows with W * diag(g) (folded into the tiled copy once, after loading), scaled
+// per row by rsqrt(mean(x^2) + eps) in the epilogue, is the same number with one rounding moved from the normed
+// activations to the folded weights; and the norm's kernel, which moves next to nothing and costs as much as a
+// quarter of a projection, is gone. The sums of squares come as partial sums `stats` [parts, 16] (float32, row m of
+// the step in column m): the kernel that last wrote the rows leaves one partial per 16 columns it owned, and the
+// reader adds them in a fixed order (every wave a share in ascending order, the waves in wave order, the four lane
+// groups in order).
+struct RowScale {
+  const float* stats;   // nullptr: rows are used as they are
+  int parts;
+  float eps, inv_dim;
+};
+
+// This lane's share of the sum of squares of row c: parts wave * 4 + g, then every 4 * WPB-th.
+template <int WPB>
+__device__ __forceinline__ float row_scale_share(const RowScale& rs, int wave, int g, int c) {
+  float ss = 0.f;
+  for (int j = wave * 4 + g; j < rs.parts; j += 4 * WPB) ss += rs.stats[j * 16 + c];
+  return ss;
+}
+// The four lane groups' shares of row c, added in order; every lane of column c gets the same sum.
+__device__ __forceinline__ float over_lane_groups(float v, int c) {
+  const float a = __shfl(v, c, WAVE), b = __shfl(v, 16 + c, WAVE), d = __shfl(v, 32 + c, WAVE), e = __shfl(v, 48 + c, WAVE);
+  return ((a + b) + d) + e;
+}
+
 // RESID: y is the residual stream, y = round(y + round(product)) in place: the add that the next norm's kernel would
 // have done, with its roundings.
 template <int MT, int WPB, int UNROLL, typename OutT, bool TILED, bool RESID = false>
 __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                 const bf16_t* __restrict__ w, OutT* __restrict__ y,
-                                                                int M, int N, int K, int round_first) {
+                                                                int M, int N, int K, int round_first, RowScale rs,
+                                                                float* __restrict__ stats_out) {
   __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * MT * WAVE : 1];
+  __shared__ float red_ss[WPB > 1 ? (WPB - 1) * WAVE : 1];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
   const int n0 = blockIdx.x * 16;
@@ -37,6 +66,8 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
   bool have[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) have[t] = t * 16 + c < M;
+  float ss = 0.f;                                // (asked for now: it arrives while the weights stream)
+  if (MT == 1 && rs.stats != nullptr) ss = row_scale_share<WPB>(rs, wave, g, c);
 
   int s = 0;
   for (; s + UNROLL <= steps; s += UNROLL) {
@@ -78,13 +109,21 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
     if (wave > 0) {
 #pragma unroll
       for (int t = 0; t < MT; ++t) red[((wave - 1) * MT + t) * WAVE + lane] = acc[t];
+      red_ss[(wave - 1) * WAVE + lane] = ss;
     }
     __syncthreads();
     if (wave > 0) return;
-    for (int ww = 1; ww < WPB; ++ww)
+    for (int ww = 1; ww < WPB; ++ww) {
 #pragma unroll
       for (int t = 0; t < MT; ++t) acc[t] += red[((ww - 1) * MT + t) * WAVE + lane];
+      ss += red_ss[(ww - 1) * WAVE + lane];
+    }
   }
+  if (MT == 1 && rs.stats != nullptr) {          // the norm's scale of row c, on the float32 sums before they are rounded
+    const float inv = 1.0f / sqrtf(over_lane_groups(ss, c) * rs.inv_dim + rs.eps);
+    acc[0] *= inv;
+  }
+  float mine = 0.f;                              // RESID with stats_out: the squares of the residual values written
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + c;
@@ -107,32 +146,40 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
         o.y = float_to_bf16(bf16_to_float(r.y) + bf16_to_float(o.y));
         o.z = float_to_bf16(bf16_to_float(r.z) + bf16_to_float(o.z));
         o.w = float_to_bf16(bf16_to_float(r.w) + bf16_to_float(o.w));
+        const float v0 = bf16_to_float(o.x), v1 = bf16_to_float(o.y), v2 = bf16_to_float(o.z), v3 = bf16_to_float(o.w);
+        mine = ((v0 * v0 + v1 * v1) + v2 * v2) + v3 * v3;
       }
       *reinterpret_cast<ushort4*>(yp) = o;
+    }
+  }
+  if constexpr (RESID && MT == 1) {
+    if (stats_out != nullptr) {                  // this block's 16 columns of every row: one partial per row
+      const float part = over_lane_groups(mine, c);
+      if (g == 0) stats_out[(int64_t)blockIdx.x * 16 + c] = part;
     }
   }
 }
 
 template <int MT, int WPB, int UNROLL, typename OutT, bool RESID>
 static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s,
-                          int round_first) {
+                          int round_first, RowScale rs, float* stats_out) {
   const dim3 grid(N / 16), block(WPB * 64);
   if constexpr (RESID)
     gemm_skinny_kernel<MT, WPB, UNROLL, OutT, true, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                                (OutT*)y, M, N, K, round_first);
+                                                                                (OutT*)y, M, N, K, round_first, rs, stats_out);
   else if (tiled)
     gemm_skinny_kernel<MT, WPB, UNROLL, OutT, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                          (OutT*)y, M, N, K, round_first);
+                                                                          (OutT*)y, M, N, K, round_first, rs, stats_out);
   else
     gemm_skinny_kernel<MT, WPB, UNROLL, OutT, false><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                           (OutT*)y, M, N, K, round_first);
+                                                                           (OutT*)y, M, N, K, round_first, rs, stats_out);
 }
 
 // How many waves share a tile, from the shapes alone (so a result never depends on M): wide outputs have tiles
 // enough to fill the GPU with few waves each and long loops; narrow ones split K 16 ways. Measured on MI355X.
 template <int MT, typename OutT, bool RESID = false>
 static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s,
-                      int round_first = 0) {
+                      int round_first = 0, RowScale rs = RowScale{nullptr, 0, 0.f, 0.f}, float* stats_out = nullptr) {
   const int tiles = N / 16;
   int wpb = MT >= 3 ? 8 : 16;                  // 16 waves of 3 or 4 token tiles run out of registers
   if (tiles >= 1024) wpb = 4;
@@ -140,15 +187,15 @@ static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K
   constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
   switch (wpb) {
     case 16:
-      if constexpr (MT < 3) launch_skinny<MT, 16, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first);
+      if constexpr (MT < 3) launch_skinny<MT, 16, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out);
       break;
-    case 8: launch_skinny<MT, 8, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first); break;
+    case 8: launch_skinny<MT, 8, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
     case 4:
-      if constexpr (MT == 1) launch_skinny<MT, 4, 16, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first);
-      else launch_skinny<MT, 4, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first);
+      if constexpr (MT == 1) launch_skinny<MT, 4, 16, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out);
+      else launch_skinny<MT, 4, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out);
       break;
-    case 2: launch_skinny<MT, 2, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first); break;
-    default: launch_skinny<MT, 1, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first); break;
+    case 2: launch_skinny<MT, 2, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
+    default: launch_skinny<MT, 1, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
   }
   return 0;
 }
@@ -174,13 +221,31 @@ extern "C" int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int
   return 0;
 }
 
+// The same product over rows that a folded norm has yet to scale: `w_tiled` holds W * diag(g), x the un-normed rows,
+// `stats` [parts, 16] the partial sums of squares of x's rows; row m of the result is scaled by
+// rsqrt(sum(stats[:, m]) / K + eps) before it is rounded. M <= 16.
+extern "C" int holon_gemm_skinny_scaled_bf16(const void* x, const void* w_tiled, void* y, int M, int N, int K,
+                                             int out_f32, const float* stats, int parts, float eps, void* stream) {
+  HOLON_CHECK(M >= 1 && M <= 16 && holon_gemm_skinny_supported(M, N, K) && stats != nullptr && parts >= 1,
+              "gemm (few rows, folded norm): M=%d N=%d K=%d parts=%d not served (M <= 16, N %% 16, K %% 32)", M, N, K, parts);
+  const RowScale rs{stats, parts, eps, 1.0f / (float)K};
+  hipStream_t s = (hipStream_t)stream;
+  if (out_f32) pick_waves<1, float>(x, w_tiled, y, M, N, K, true, s, out_f32 == 2, rs);
+  else pick_waves<1, bf16_t>(x, w_tiled, y, M, N, K, true, s, 0, rs);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
 // residual[M, N] += x[M, K] w^T in place (the product rounded, then the sum rounded), for one tile of rows (M <= 16)
-// over tiled weights: the output projection's product and the residual add that follows it, in one kernel.
+// over tiled weights: the output projection's product and the residual add that follows it, in one kernel. With
+// `stats_out` ([N / 16, 16] float32) it also leaves, per block of 16 columns, the sums of squares of the residual
+// values it wrote: what a norm over the new rows needs.
 extern "C" int holon_gemm_skinny_add_bf16(const void* x, const void* w_tiled, void* residual, int M, int N, int K,
-                                          void* stream) {
+                                          float* stats_out, void* stream) {
   HOLON_CHECK(M >= 1 && M <= 16 && holon_gemm_skinny_supported(M, N, K),
               "gemm (few rows, added to the residual): M=%d N=%d K=%d not served (M <= 16, N %% 16, K %% 32)", M, N, K);
-  pick_waves<1, bf16_t, true>(x, w_tiled, residual, M, N, K, true, (hipStream_t)stream);
+  pick_waves<1, bf16_t, true>(x, w_tiled, residual, M, N, K, true, (hipStream_t)stream, 0,
+                              RowScale{nullptr, 0, 0.f, 0.f}, stats_out);
   HOLON_LAUNCH_OK();
   return 0;
 }
@@ -190,8 +255,10 @@ extern "C" int holon_gemm_skinny_add_bf16(const void* x, const void* w_tiled, vo
 template <int MT, int WPB, int UNROLL, bool TILED>
 __global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t* __restrict__ x,
                                                                     const bf16_t* __restrict__ w,
-                                                                    bf16_t* __restrict__ y, int M, int I, int K) {
+                                                                    bf16_t* __restrict__ y, int M, int I, int K,
+                                                                    RowScale rs) {
   __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * 2 * MT * WAVE : 1];
+  __shared__ float red_ss[WPB > 1 ? (WPB - 1) * WAVE : 1];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
   const int n0 = blockIdx.x * 16;
@@ -212,6 +279,8 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t*
     acc[0][t] = acc[1][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     have[t] = t * 16 + c < M;
   }
+  float ss = 0.f;
+  if (MT == 1 && rs.stats != nullptr) ss = row_scale_share<WPB>(rs, wave, g, c);
   int s = 0;
   for (; s + UNROLL <= steps; s += UNROLL) {
     bf16x8_t wf[2][UNROLL], xf[UNROLL][MT];
@@ -261,14 +330,22 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t*
       for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int t = 0; t < MT; ++t) red[(((wave - 1) * 2 + h) * MT + t) * WAVE + lane] = acc[h][t];
+      red_ss[(wave - 1) * WAVE + lane] = ss;
     }
     __syncthreads();
     if (wave > 0) return;
-    for (int ww = 1; ww < WPB; ++ww)
+    for (int ww = 1; ww < WPB; ++ww) {
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[h][t] += red[(((ww - 1) * 2 + h) * MT + t) * WAVE + lane];
+      ss += red_ss[(ww - 1) * WAVE + lane];
+    }
+  }
+  if (MT == 1 && rs.stats != nullptr) {
+    const float inv = 1.0f / sqrtf(over_lane_groups(ss, c) * rs.inv_dim + rs.eps);
+    acc[0][0] *= inv;
+    acc[1][0] *= inv;
   }
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -287,16 +364,21 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t*
   }
 }
 
+// `stats` (nullable, with `parts` and `eps`): x holds un-normed rows and `w` the tiled weights with the norm's weight
+// folded in; rows are scaled as in holon_gemm_skinny_scaled_bf16 (M <= 16, tiled).
 extern "C" int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int I, int K, int tiled,
-                                          void* stream) {
+                                          const float* stats, int parts, float eps, void* stream) {
   HOLON_CHECK(M >= 1 && M <= 32 && I % 16 == 0 && K % 128 == 0, "gated gemm (few rows): M=%d I=%d K=%d not served", M, I, K);
+  HOLON_CHECK(stats == nullptr || (M <= 16 && tiled && parts >= 1), "gated gemm (few rows, folded norm): M=%d tiled=%d parts=%d",
+              M, tiled, parts);
+  const RowScale rs{stats, parts, eps, 1.0f / (float)K};
   hipStream_t s = (hipStream_t)stream;
   const bool few = I / 16 < 512;   // few tile pairs: four waves share each
 #define GLU(MT, WPB, U)                                                                                              \
   if (tiled) gemm_skinny_glu_kernel<MT, WPB, U, true><<<I / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, \
-                                                                                 (bf16_t*)y, M, I, K);               \
+                                                                                 (bf16_t*)y, M, I, K, rs);           \
   else gemm_skinny_glu_kernel<MT, WPB, U, false><<<I / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,      \
-                                                                            (bf16_t*)y, M, I, K)
+                                                                            (bf16_t*)y, M, I, K, rs)
   if (M <= 16) { if (few) { GLU(1, 4, 8); } else { GLU(1, 1, 8); } }
   else { if (few) { GLU(2, 4, 4); } else { GLU(2, 1, 4); } }
 #undef GLU
@@ -305,20 +387,29 @@ extern "C" int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y,
 }
 
 // tiled[t][s][l][e] = w[16 t + l % 16][32 s + 8 (l / 16) + e]: the layout the few-row product streams.
-__global__ void tile_weight_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ tiled, int N, int K) {
+// With `scale` [K]: tiled holds round(w[n][k] * scale[k]), a norm's weight folded into the columns it multiplies.
+__global__ void tile_weight_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ tiled, int N, int K,
+                                   const bf16_t* __restrict__ scale) {
   const int64_t chunks = (int64_t)N * K / 8;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * blockDim.x) {
     const int lane = (int)(i % 64);
     const int64_t ts = i / 64;
     const int64_t step = ts % (K / 32), tile = ts / (K / 32);
-    const int64_t src = (tile * 16 + lane % 16) * K + step * 32 + 8 * (lane / 16);
-    *reinterpret_cast<uint4*>(tiled + i * 8) = *reinterpret_cast<const uint4*>(w + src);
+    const int64_t col = step * 32 + 8 * (lane / 16);
+    const int64_t src = (tile * 16 + lane % 16) * K + col;
+    uint4 v = *reinterpret_cast<const uint4*>(w + src);
+    if (scale != nullptr) {
+      bf16_t* e = reinterpret_cast<bf16_t*>(&v);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e[j] = float_to_bf16(bf16_to_float(e[j]) * bf16_to_float(scale[col + j]));
+    }
+    *reinterpret_cast<uint4*>(tiled + i * 8) = v;
   }
 }
 
-extern "C" int holon_tile_weight_bf16(const void* w, void* tiled, int N, int K, void* stream) {
+extern "C" int holon_tile_weight_bf16(const void* w, void* tiled, int N, int K, const void* scale, void* stream) {
   HOLON_CHECK(N > 0 && K > 0 && N % 16 == 0 && K % 32 == 0, "tile_weight: N=%d K=%d must be multiples of 16 and 32", N, K);
-  tile_weight_kernel<<<4096, 256, 0, (hipStream_t)stream>>>((const bf16_t*)w, (bf16_t*)tiled, N, K);
+  tile_weight_kernel<<<4096, 256, 0, (hipStream_t)stream>>>((const bf16_t*)w, (bf16_t*)tiled, N, K, (const bf16_t*)scale);
   HOLON_LAUNCH_OK();
   return 0;
 }

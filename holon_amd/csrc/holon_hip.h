@@ -12,8 +12,11 @@ int holon_abi_version(void);
 
 // out[t] = table[ids[t]]; with take_slot and last_token (both or neither), token t is last_token[take_slot[t]] where
 // take_slot[t] >= 0: a token the previous step drew and left on the device.
+// stats_out (nullable, tokens <= 16): [16] float32, the sum of squares of every row written.
 int holon_embedding(const int32_t* ids, const int32_t* take_slot, const int32_t* last_token, const void* table, void* out,
-                    int tokens, int hidden, int vocab, int dtype, void* stream);
+                    int tokens, int hidden, int vocab, int dtype, float* stats_out, void* stream);
+// stats[m] = sum of squares of row m of x [rows, dim], rows <= 16.
+int holon_row_sumsq(const void* x, float* stats, int rows, int dim, int dtype, void* stream);
 // y = rmsnorm(x) over rows of `dim`; with `residual`: residual += x (rounded), y = rmsnorm(residual).
 int holon_rmsnorm(const void* x, void* residual, const void* weight, void* y, int64_t rows, int dim, float eps,
                   int dtype, void* stream);
@@ -70,13 +73,23 @@ int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, 
                            void* stream);
 // residual[M, N] = round(residual + round(x w^T)) in place, M <= 16, tiled weights: the product and the residual add
 // that follows it in one kernel.
-int holon_gemm_skinny_add_bf16(const void* x, const void* w_tiled, void* residual, int M, int N, int K, void* stream);
+// With stats_out ([N / 16, 16] float32): per block of 16 columns, the sums of squares of the residual values written.
+int holon_gemm_skinny_add_bf16(const void* x, const void* w_tiled, void* residual, int M, int N, int K, float* stats_out,
+                               void* stream);
+// A norm folded into the product: w_tiled holds W * diag(g) (holon_tile_weight_bf16 with `scale`), x the un-normed rows,
+// stats [parts, 16] partial sums of squares of x's rows (row m in column m); row m of the result is scaled by
+// rsqrt(sum(stats[:, m]) / K + eps) before rounding. M <= 16.
+int holon_gemm_skinny_scaled_bf16(const void* x, const void* w_tiled, void* y, int M, int N, int K, int out_f32,
+                                  const float* stats, int parts, float eps, void* stream);
 // y[M, I] = round(silu(round(x gate^T))) * round(x up^T) with w = [gate; up] ([2I, K]), M <= 32.
-int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int I, int K, int tiled, void* stream);
+// stats (nullable): as in holon_gemm_skinny_scaled_bf16 (M <= 16, tiled weights with the norm's weight folded in).
+int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int I, int K, int tiled, const float* stats,
+                               int parts, float eps, void* stream);
 // y[M, N] = x[M, K] w[N, K]^T, all float32, true 32-bit products and sums in an order that depends on K alone: a row's
 // result is bit for bit the same whatever other rows are in the call.
 int holon_gemm_f32(const void* x, const void* w, void* y, int M, int N, int K, void* stream);
-int holon_tile_weight_bf16(const void* w, void* tiled, int N, int K, void* stream);
+// scale (nullable, [K] bfloat16): tiled holds round(w[n][k] * scale[k]).
+int holon_tile_weight_bf16(const void* w, void* tiled, int N, int K, const void* scale, void* stream);
 int holon_argmax(const float* logits, int32_t* out, int rows, int vocab, void* stream);
 // last_token[slots[r]] = tokens[r] for r < rows (slots are distinct; last_token has n_slots entries).
 int holon_store_tokens(int32_t* last_token, const int32_t* slots, const int32_t* tokens, int rows, int n_slots,

@@ -44,10 +44,18 @@ class Kernels(Protocol):
     name: str
 
     def embedding(self, ids: torch.Tensor, table: torch.Tensor,
-                  take: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
+                  take: tuple[torch.Tensor, torch.Tensor] | None = None, want_stats: bool = False):
         """ids [T] int32, table [V, H] -> [T, H] (rows of the table). `take` = (take_slot [T] int32, last_token [S]
         int32): token t is last_token[take_slot[t]] where take_slot[t] >= 0 (a token the previous step drew and left
-        on the device), ids[t] otherwise."""
+        on the device), ids[t] otherwise. With `want_stats` -> (rows, row statistics or None): see `row_sumsq`."""
+
+    def row_sumsq(self, x: torch.Tensor) -> torch.Tensor:
+        """Row statistics of x [M <= 16, H]: float32 [parts, 16] whose column m sums to the sum of squares of row m
+        (here parts = 1). A kernel that writes rows may leave the same thing in several parts (`linear_add`); a
+        product with a folded norm (`linear(..., row_scale=)`) adds the parts in a fixed order."""
+
+    def folds_norm(self, rows: int, weight: torch.Tensor, tiled: torch.Tensor | None) -> bool:
+        """Whether `linear(x, weight, tiled=tiled, row_scale=...)` serves `rows` rows."""
 
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
         """x [..., dim] contiguous -> a new tensor; x is not modified."""
@@ -56,22 +64,30 @@ class Kernels(Protocol):
         """residual += x in place (sum rounded to dtype), returns rmsnorm(residual) as a new tensor."""
 
     def linear(self, x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None = None,
-               tiled: torch.Tensor | None = None) -> torch.Tensor:
+               tiled: torch.Tensor | None = None, row_scale: tuple[torch.Tensor, float] | None = None) -> torch.Tensor:
         """x [T, K] @ weight [N, K].T -> [T, N], float32 accumulation, rounded to x's dtype; with another `out_dtype`
         that rounded product is then cast (the reference's `F.linear(...).float()`, std/holon_std/ops/units.py:348): one
-        rule for every number of rows. `tiled`: what `tile_weight(weight)` returned, if anything."""
+        rule for every number of rows. `tiled`: what `tile_weight(weight)` returned, if anything.
+        `row_scale` = (row statistics of x, eps): an RMSNorm folded into the product. `tiled` is then
+        `tile_weight(weight, norm_weight)`, x the un-normed rows, and row m of the float32 sums is scaled by
+        rsqrt(mean(x[m]^2) + eps) before it is rounded: norm(x) W^T with the rounding of the normed activations
+        moved to the folded weights."""
 
-    def tile_weight(self, weight: torch.Tensor) -> torch.Tensor | None:
-        """Once per weight after loading: a copy in the layout steps of few rows stream fastest, or None."""
+    def tile_weight(self, weight: torch.Tensor, scale: torch.Tensor | None = None) -> torch.Tensor | None:
+        """Once per weight after loading: a copy in the layout steps of few rows stream fastest, or None. With
+        `scale` [K] the copy holds weight * scale[None, :] (rounded): a norm's weight folded in."""
 
-    def linear_add(self, x: torch.Tensor, weight: torch.Tensor, tiled: torch.Tensor | None, residual: torch.Tensor
-                   ) -> bool:
+    def linear_add(self, x: torch.Tensor, weight: torch.Tensor, tiled: torch.Tensor | None, residual: torch.Tensor,
+                   want_stats: bool = False) -> "bool | torch.Tensor":
         """residual += linear(x, weight) in place in one kernel: the product rounded to dtype, then the sum rounded,
-        as the add of `add_rmsnorm` does. False when not fused for this shape; then nothing was done."""
+        as the add of `add_rmsnorm` does. False when not fused for this shape; then nothing was done. Otherwise
+        True, or with `want_stats` the row statistics of the residual rows as they now are, when the kernel can
+        leave them."""
 
-    def linear_silu_mul(self, x: torch.Tensor, weight: torch.Tensor, tiled: torch.Tensor | None = None
-                        ) -> torch.Tensor | None:
-        """silu_mul(linear(x, weight)) fused, with the composition's roundings; None when not fused for this shape."""
+    def linear_silu_mul(self, x: torch.Tensor, weight: torch.Tensor, tiled: torch.Tensor | None = None,
+                        row_scale: tuple[torch.Tensor, float] | None = None) -> torch.Tensor | None:
+        """silu_mul(linear(x, weight)) fused, with the composition's roundings; None when not fused for this shape.
+        `row_scale` as in `linear`."""
 
     def silu_mul(self, gate_up: torch.Tensor) -> torch.Tensor:
         """gate_up [T, 2I] (gate columns first) -> [T, I] = round(silu(gate)) * up."""

@@ -53,7 +53,8 @@ class HipKernels:
         lib = self.lib
         lib.holon_last_error.restype = ctypes.c_char_p
         sig = {
-            "holon_embedding": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+            "holon_embedding": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P],
+            "holon_row_sumsq": [_P, _P, _I, _I, _I, _P],
             "holon_rmsnorm": [_P, _P, _P, _P, _L, _I, _F, _I, _P],
             "holon_silu_mul": [_P, _P, _L, _I, _I, _P],
             "holon_qk_norm_rope_write": [_P, _L, _P, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _P, _P, _P, _P, _I, _I,
@@ -67,10 +68,11 @@ class HipKernels:
                                             _I, _I, _P],
             "holon_gemm_skinny_supported": [_I, _I, _I],
             "holon_gemm_skinny_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
-            "holon_tile_weight_bf16": [_P, _P, _I, _I, _P],
+            "holon_tile_weight_bf16": [_P, _P, _I, _I, _P, _P],
+            "holon_gemm_skinny_scaled_bf16": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _F, _P],
             "holon_gemm_f32": [_P, _P, _P, _I, _I, _I, _P],
-            "holon_gemm_skinny_add_bf16": [_P, _P, _P, _I, _I, _I, _P],
-            "holon_gemm_skinny_glu_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
+            "holon_gemm_skinny_add_bf16": [_P, _P, _P, _I, _I, _I, _P, _P],
+            "holon_gemm_skinny_glu_bf16": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _F, _P],
             "holon_argmax": [_P, _P, _I, _I, _P],
             "holon_store_tokens": [_P, _P, _P, _I, _I, _P],
             "holon_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P],
@@ -106,7 +108,7 @@ class HipKernels:
         return _DT[t.dtype]
 
     # -- ops ------------------------------------------------------------------------------------------------------
-    def embedding(self, ids, table, take=None):
+    def embedding(self, ids, table, take=None, want_stats=False):
         self._check(ids, "embedding ids", torch.int32)
         self._check(table, "embedding table")
         take_slot, last_token = take if take is not None else (None, None)
@@ -116,10 +118,23 @@ class HipKernels:
             if take_slot.shape != ids.shape:
                 raise KernelError(f"embedding: {tuple(take_slot.shape)} slots to take from for {tuple(ids.shape)} tokens")
         out = torch.empty((ids.shape[0], table.shape[1]), dtype=table.dtype, device=table.device)
+        stats = None
+        if want_stats and ids.shape[0] <= self.skinny_rows and table.dtype == torch.bfloat16:
+            stats = torch.empty((1, 16), dtype=torch.float32, device=table.device)
         self._call(self.lib.holon_embedding, ids.data_ptr(), _ptr(take_slot), _ptr(last_token), table.data_ptr(),
                    out.data_ptr(), ids.shape[0], table.shape[1], table.shape[0], self._dt(table, "embedding"),
+                   _ptr(stats), self._stream())
+        return (out, stats) if want_stats else out
+
+    def row_sumsq(self, x):
+        self._check(x, "row_sumsq x")
+        rows, dim = x.shape
+        if rows > 16:
+            raise KernelError(f"row_sumsq: {rows} rows (at most 16)")
+        stats = torch.empty((1, 16), dtype=torch.float32, device=x.device)
+        self._call(self.lib.holon_row_sumsq, x.data_ptr(), stats.data_ptr(), rows, dim, self._dt(x, "row_sumsq"),
                    self._stream())
-        return out
+        return stats
 
     def rmsnorm(self, x, weight, eps):
         self._check(x, "rmsnorm x")
@@ -146,22 +161,52 @@ class HipKernels:
 
     skinny_rows = 16          # up to this many rows the hand-written weight-streaming product runs
 
-    def tile_weight(self, weight):
+    def tile_weight(self, weight, scale=None):
         """A copy of `weight` [N, K] in the layout the few-row product streams fastest, or None when its shape or
-        dtype has no such layout (then `linear` reads the rows as they are)."""
+        dtype has no such layout (then `linear` reads the rows as they are). With `scale` [K] the copy holds
+        weight * scale (a norm's weight folded in)."""
         n, k = weight.shape
         if weight.dtype != torch.bfloat16 or not weight.is_cuda or n % 16 or k % 32 or k < 256:
             return None
         self._check(weight, "tile_weight")
+        if scale is not None:
+            self._check(scale, "tile_weight scale", torch.bfloat16)
+            if scale.shape != (k,):
+                raise KernelError(f"tile_weight: scale {tuple(scale.shape)} for K = {k}")
         tiled = torch.empty_like(weight)
-        self._call(self.lib.holon_tile_weight_bf16, weight.data_ptr(), tiled.data_ptr(), n, k, self._stream())
+        self._call(self.lib.holon_tile_weight_bf16, weight.data_ptr(), tiled.data_ptr(), n, k, _ptr(scale),
+                   self._stream())
         return tiled
 
-    def linear(self, x, weight, out_dtype=None, tiled=None):
+    def _row_scale(self, x, tiled, row_scale, what):
+        """Checks of a product over un-normed rows with the norm folded into `tiled`; returns (stats, parts, eps)."""
+        stats, eps = row_scale
+        if tiled is None or x.shape[0] > min(self.skinny_rows, 16) or x.dtype != torch.bfloat16:
+            raise KernelError(f"{what}: a folded norm needs tiled weights and at most 16 bfloat16 rows")
+        self._check(stats, f"{what} stats", torch.float32)
+        if stats.dim() != 2 or stats.shape[1] != 16:
+            raise KernelError(f"{what}: stats {tuple(stats.shape)}, expected [parts, 16]")
+        return stats, stats.shape[0], float(eps)
+
+    def folds_norm(self, rows, weight, tiled):
+        """Whether `linear(x, ..., row_scale=...)` serves `rows` rows over this weight."""
+        n, k = weight.shape
+        return bool(tiled is not None and weight.dtype == torch.bfloat16 and 1 <= rows <= min(self.skinny_rows, 16)
+                    and k >= 256 and self.lib.holon_gemm_skinny_supported(rows, n, k))
+
+    def linear(self, x, weight, out_dtype=None, tiled=None, row_scale=None):
         m, k = x.shape
         n = weight.shape[0]
         if weight.shape[1] != k:
             raise KernelError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(weight.shape)}")
+        if row_scale is not None:
+            stats, parts, eps = self._row_scale(x, tiled, row_scale, "linear")
+            self._check(x, "linear x")
+            to_f32 = out_dtype == torch.float32
+            y = torch.empty((m, n), dtype=torch.float32 if to_f32 else torch.bfloat16, device=x.device)
+            self._call(self.lib.holon_gemm_skinny_scaled_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), m, n, k,
+                       2 if to_f32 else 0, stats.data_ptr(), parts, eps, self._stream())
+            return y
         if (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows and k >= 256
                 and x.is_contiguous() and weight.is_contiguous() and self.lib.holon_gemm_skinny_supported(m, n, k)):
             to_f32 = out_dtype == torch.float32       # then: the bfloat16 product cast up, as for any number of rows
@@ -181,7 +226,9 @@ class HipKernels:
         y = torch.matmul(x, weight.t())
         return y if out_dtype in (None, y.dtype) else y.to(out_dtype)
 
-    def linear_add(self, x, weight, tiled, residual):
+    def linear_add(self, x, weight, tiled, residual, want_stats=False):
+        """-> False when not fused; otherwise True, or with `want_stats` the partial sums of squares [N / 16, 16] of
+        the residual rows as they now are."""
         (m, k), n = x.shape, weight.shape[0]
         if not (tiled is not None and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
                 and residual.dtype == torch.bfloat16 and 1 <= m <= min(self.skinny_rows, 16) and weight.shape[1] == k
@@ -190,11 +237,12 @@ class HipKernels:
             return False
         if tuple(residual.shape) != (m, n):
             raise KernelError(f"linear_add: residual {tuple(residual.shape)} for a product of {(m, n)}")
+        stats = torch.empty((n // 16, 16), dtype=torch.float32, device=x.device) if want_stats else None
         self._call(self.lib.holon_gemm_skinny_add_bf16, x.data_ptr(), tiled.data_ptr(), residual.data_ptr(), m, n, k,
-                   self._stream())
-        return True
+                   _ptr(stats), self._stream())
+        return stats if want_stats else True
 
-    def linear_silu_mul(self, x, weight, tiled=None):
+    def linear_silu_mul(self, x, weight, tiled=None, row_scale=None):
         """silu_mul(linear(x, weight)) in one kernel for steps of few rows, with the roundings of the two kernels one
         after the other (the sums over K may be split differently); None when this shape is not fused (the caller then composes the two)."""
         m, k = x.shape
@@ -204,8 +252,10 @@ class HipKernels:
             return None
         y = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
         source = tiled if tiled is not None else weight
+        stats, parts, eps = self._row_scale(x, tiled, row_scale, "linear_silu_mul") if row_scale is not None \
+            else (None, 0, 0.0)
         self._call(self.lib.holon_gemm_skinny_glu_bf16, x.data_ptr(), source.data_ptr(), y.data_ptr(), m, two_i // 2, k,
-                   int(tiled is not None), self._stream())
+                   int(tiled is not None), _ptr(stats), parts, eps, self._stream())
         return y
 
     def silu_mul(self, gate_up):

@@ -6,7 +6,7 @@ import dataclasses
 
 import torch
 
-from .parts.base import Build, PagedState, Part, SlotState
+from .parts.base import Build, PagedState, Part, SlotState, Stream
 from .spec import ModelSpec
 
 
@@ -73,10 +73,11 @@ class Model(Part):
 
     def trunk(self, step) -> tuple[torch.Tensor, torch.Tensor | None]:
         """The residual stream after every run, as (h, delta) with h + delta the stream [T, hidden]."""
-        h, delta = self.embed(step.token_ids, step.token_take), None
+        h, stats = self.embed(step.token_ids, step.token_take, want_stats=True)
+        stream = Stream(h, stats=stats)
         for site in self.sites:
-            h, delta = self.blocks[site.layer](h, delta, step, site)
-        return h, delta
+            stream = self.blocks[site.layer](stream, step, site)
+        return stream.h, stream.delta
 
     def head(self, h: torch.Tensor, delta: torch.Tensor | None) -> torch.Tensor:
         """Final norm and head on the given rows -> float32 logits [R, vocab]. The rows are consumed."""

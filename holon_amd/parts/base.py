@@ -50,6 +50,18 @@ class SlotState:
 
 
 @dataclasses.dataclass
+class Stream:
+    """The residual stream between blocks: `h` [T, hidden], updated in place; `delta`, a term not yet added to it (the
+    next norm's kernel fuses the add) or None; `stats`, what the kernel that last wrote `h` left about its rows for a
+    norm that follows (partial sums of squares, see the kernel contract) or None when nothing is known. Whoever
+    changes `h` sets `stats` anew or to None."""
+
+    h: torch.Tensor
+    delta: torch.Tensor | None = None
+    stats: torch.Tensor | None = None
+
+
+@dataclasses.dataclass
 class Build:
     """What a part may know of the engine while it is built."""
 

@@ -5,7 +5,7 @@ import torch
 
 from ..registry import register_part
 from ..spec import PartRef
-from .base import Build, Part
+from .base import Build, Part, Stream
 
 
 @register_part("block", "prenorm")
@@ -23,13 +23,35 @@ class PreNorm(Part):
         self.attach("post_norm", build.make(norm, dim=hidden))
         self.attach("ffn", build.make(ffn, layer=layer, hidden=hidden))
 
-    def forward(self, h: torch.Tensor, delta: torch.Tensor | None, step, site
-                ) -> tuple[torch.Tensor, torch.Tensor | None]:
-        """The residual stream is `h + delta` on entry and on return; `h` is updated in place. A part that can add
-        its result into `h` inside its own kernel (`adds_residual`) is given `h`; it returns None when it did."""
-        a = self.input_norm(h) if delta is None else self.input_norm.add(delta, h)[0]
-        mixed = self.mixer(a, step, site, **({"residual": h} if self.mixer.adds_residual else {}))
-        x = self.post_norm(h) if mixed is None else self.post_norm.add(mixed, h)[0]
-        return h, self.ffn(x, step, **({"residual": h} if self.ffn.adds_residual else {}))
+    def finalize(self) -> None:
+        """A mixer or feed-forward that can fold the norm in front of it into its own first product does so now (its
+        weights are loaded and merged); it is then handed the norm deferred (`Normed`) instead of its result."""
+        self._mixer_defers = bool(getattr(self.mixer, "absorb_norm", None)) and self.mixer.absorb_norm(self.input_norm)
+        self._ffn_defers = bool(getattr(self.ffn, "absorb_norm", None)) and self.ffn.absorb_norm(self.post_norm)
+
+    _mixer_defers = _ffn_defers = False
+
+    def forward(self, stream: Stream, step, site) -> Stream:
+        """The residual stream is `stream.h + stream.delta` on entry and on return; `h` is updated in place. A part
+        that can add its result into `h` inside its own kernel (`adds_residual`) is given the stream; it returns None
+        when it did (and the kernel leaves the rows' statistics in `stream.stats` for the norm that follows)."""
+        h = stream.h
+        if stream.delta is not None:
+            a = self.input_norm.add(stream.delta, h)[0]
+        elif self._mixer_defers:
+            a = self.input_norm.defer(h, stream.stats)
+        else:
+            a = self.input_norm(h)
+        stream.delta = stream.stats = None
+        mixed = self.mixer(a, step, site, **({"residual": stream} if self.mixer.adds_residual else {}))
+        if mixed is not None:
+            x = self.post_norm.add(mixed, h)[0]
+        elif self._ffn_defers:
+            x = self.post_norm.defer(h, stream.stats)
+        else:
+            x = self.post_norm(h)
+        stream.stats = None
+        stream.delta = self.ffn(x, step, **({"residual": stream} if self.ffn.adds_residual else {}))
+        return stream
 
     __call__ = forward

@@ -15,9 +15,11 @@ class Embedding(Part):
         super().__init__(build)
         self.declare("weight", (vocab, hidden))
 
-    def forward(self, ids: torch.Tensor, take: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
-        """Rows of the table; `take`: where a token is still on the device, see the kernel contract."""
-        return self.kernels.embedding(ids, self.weight, take)
+    def forward(self, ids: torch.Tensor, take: tuple[torch.Tensor, torch.Tensor] | None = None,
+                want_stats: bool = False):
+        """Rows of the table; `take`: where a token is still on the device, see the kernel contract. With
+        `want_stats`: (rows, their statistics for a norm that follows, or None)."""
+        return self.kernels.embedding(ids, self.weight, take, want_stats)
 
     __call__ = forward
 

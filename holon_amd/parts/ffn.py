@@ -4,8 +4,9 @@ from __future__ import annotations
 import torch
 
 from ..registry import register_part
-from .base import Build, Part
+from .base import Build, Part, Stream
 from .linear import Linear
+from .norms import Normed
 
 
 @register_part("ffn", "swiglu")
@@ -30,10 +31,19 @@ class SwiGLU(Part):
 
     adds_residual = True
 
-    def forward(self, x: torch.Tensor, step=None, residual: torch.Tensor | None = None) -> torch.Tensor | None:
-        y = self.kernels.linear_silu_mul(x, self.gate_up.weight, self.gate_up.tiled)   # fused for steps of few rows
+    def absorb_norm(self, norm: Part) -> bool:
+        """Fold the norm in front of this part into its first product; it then takes `Normed` input."""
+        return self.gate_up.absorb(norm)
+
+    def forward(self, x: torch.Tensor | Normed, step=None, residual: Stream | None = None) -> torch.Tensor | None:
+        gate_up, y = self.gate_up, None
+        if gate_up.folds(x):
+            y = self.kernels.linear_silu_mul(x.h, gate_up.weight, gate_up.tiled, row_scale=gate_up.row_scale(x))
+        elif gate_up.folded is None:               # fused for steps of few rows
+            x = x.value() if isinstance(x, Normed) else x
+            y = self.kernels.linear_silu_mul(x, gate_up.weight, gate_up.tiled)
         if y is None:
-            y = self.kernels.silu_mul(self.gate_up(x))
+            y = self.kernels.silu_mul(gate_up(x))
         return self.down_proj(y, residual=residual)
 
     __call__ = forward

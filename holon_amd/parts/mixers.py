@@ -6,8 +6,9 @@ import torch
 
 from ..registry import register_part
 from ..spec import PartRef
-from .base import Build, PagedState, Part
+from .base import Build, PagedState, Part, Stream
 from .linear import Linear
+from .norms import Normed
 
 
 @register_part("mixer", "gqa")
@@ -62,7 +63,11 @@ class GQA(Part):
 
     adds_residual = True
 
-    def forward(self, x: torch.Tensor, step, site, residual: torch.Tensor | None = None) -> torch.Tensor | None:
+    def absorb_norm(self, norm: Part) -> bool:
+        """Fold the norm in front of this mixer into its merged q/k/v product; it then takes `Normed` input."""
+        return self.qkv is not None and self.qkv.absorb(norm)
+
+    def forward(self, x: "torch.Tensor | Normed", step, site, residual: Stream | None = None) -> torch.Tensor | None:
         k = self.kernels
         t, hq, hkv, d = x.shape[0], self.heads, self.kv_heads, self.head_dim
         view = step.paged[site.group]

@@ -42,11 +42,21 @@ def _mix32(x):
 class TorchKernels:
     name = "torch-plain"
 
-    def embedding(self, ids, table, take=None):
+    fold_norms = False       # a test may switch the folded-norm path on: the twin then stands in for the tiled copy
+
+    def embedding(self, ids, table, take=None, want_stats=False):
         if take is not None:
             take_slot, last_token = take
             ids = torch.where(take_slot >= 0, last_token[take_slot.clamp(min=0).long()], ids)
-        return table[ids.long()]
+        rows = table[ids.long()]
+        if not want_stats:
+            return rows
+        return rows, (self.row_sumsq(rows) if self.fold_norms and rows.shape[0] <= 16 else None)
+
+    def row_sumsq(self, x):
+        stats = torch.zeros(1, 16, dtype=torch.float32, device=x.device)
+        stats[0, : x.shape[0]] = x.float().pow(2).sum(-1)
+        return stats
 
     def rmsnorm(self, x, weight, eps):
         return _rmsnorm(x, weight, eps)
@@ -55,18 +65,36 @@ class TorchKernels:
         residual.add_(x)
         return _rmsnorm(residual, weight, eps)
 
-    def tile_weight(self, weight):
-        return None
+    def tile_weight(self, weight, scale=None):
+        """No tile layout here. With `scale` (and `fold_norms`) the stand-in for a folded copy: the scaled rows."""
+        if scale is None or not self.fold_norms:
+            return None
+        return (_up(weight) * _up(scale)[None, :]).to(weight.dtype)
 
-    def linear(self, x, weight, out_dtype=None, tiled=None):
+    def folds_norm(self, rows, weight, tiled):
+        return tiled is not None and rows <= 16
+
+    @staticmethod
+    def _scaled(x, folded, row_scale):
+        stats, eps = row_scale
+        inv = torch.rsqrt(stats.sum(0)[: x.shape[0]] / x.shape[1] + eps)
+        return (_up(x) @ _up(folded).T) * inv[:, None].to(_up(x).dtype)
+
+    def linear(self, x, weight, out_dtype=None, tiled=None, row_scale=None):
+        if row_scale is not None:
+            return self._scaled(x, tiled, row_scale).to(x.dtype).to(out_dtype or x.dtype)
         return (_up(x) @ _up(weight).T).to(x.dtype).to(out_dtype or x.dtype)      # rounded to x's dtype, then cast
 
-    def linear_add(self, x, weight, tiled, residual):
+    def linear_add(self, x, weight, tiled, residual, want_stats=False):
         residual.copy_((_up(residual) + _up(self.linear(x, weight))).to(residual.dtype))
+        if want_stats and self.fold_norms and residual.shape[0] <= 16:
+            return self.row_sumsq(residual)
         return True
 
-    def linear_silu_mul(self, x, weight, tiled=None):
-        return None
+    def linear_silu_mul(self, x, weight, tiled=None, row_scale=None):
+        if row_scale is None:
+            return None
+        return self.silu_mul(self._scaled(x, tiled, row_scale).to(x.dtype))
 
     def silu_mul(self, gate_up):
         gate, up = gate_up.chunk(2, dim=-1)

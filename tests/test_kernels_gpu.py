@@ -347,6 +347,53 @@ def test_float32_product_is_true_32_bit_and_its_order_is_fixed(hip):
     assert torch.equal(hip.linear(x, w), x @ w.T)                                 # exact arithmetic: any order, same bits
 
 
+def test_norm_folded_into_the_product(hip):
+    """The norm's weight folded into the tiled copy, the rows scaled inside the product from statistics another kernel
+    left: against norm then product in float64, within the budget of the two operations; the statistics from the
+    residual add's kernel, from the embedding and from `row_sumsq` are the rows' sums of squares; the gated form too."""
+    bf = torch.bfloat16
+    for m, k, n in ((1, 4096, 6144), (8, 4096, 1024), (16, 512, 208), (5, 12288, 4096), (3, 4096, 24576)):
+        h = _randn(m, k, dtype=bf, seed=50, scale=2.0)
+        g = (1 + 0.2 * torch.randn(k, generator=torch.Generator().manual_seed(51))).to(bf).cuda()
+        w = _randn(n, k, dtype=bf, seed=52, scale=0.05)
+        eps = 1e-5
+        exact = PLAIN.rmsnorm(h.double(), g.double(), eps) @ w.double().T
+        composed = hip.linear(hip.rmsnorm(h, g, eps), w)
+        folded = hip.tile_weight(w, g)
+        assert hip.folds_norm(m, w, folded)
+        stats = hip.row_sumsq(h)
+        assert stats.shape == (1, 16)
+        assert torch.allclose(stats[0, :m], h.float().pow(2).sum(-1), rtol=1e-5)
+        got = hip.linear(h, w, None, folded, row_scale=(stats, eps))
+        assert got.dtype == bf and H.op_budget_usage(got, exact, bf, 2 * k) <= 1, (m, k, n)
+        assert H.rel_rms(got, exact) <= 1.5 * H.rel_rms(composed, exact) + 1e-4          # no worse than norm, then product
+        split = torch.zeros(7, 16, device="cuda")                                      # the same sums in seven parts
+        split[:, :m] = (h.float().pow(2).sum(-1) / 7)[None, :]
+        assert H.op_budget_usage(hip.linear(h, w, None, folded, row_scale=(split, eps)), exact, bf, 2 * k) <= 1
+        got32 = hip.linear(h, w, torch.float32, folded, row_scale=(stats, eps))
+        assert torch.equal(got32, got.float())
+        if n % 32 == 0 and k % 128 == 0:                                               # the gated form
+            want = PLAIN.silu_mul((PLAIN.rmsnorm(h.double(), g.double(), eps) @ w.double().T))
+            glu = hip.linear_silu_mul(h, w, folded, row_scale=(stats, eps))
+            assert glu.shape == (m, n // 2) and H.op_budget_usage(glu, want, bf, 2 * k) <= 1, (m, k, n)
+    # the residual add leaves the statistics of the rows it wrote, one part per 16 columns
+    for m, k, n in ((8, 4096, 4096), (1, 12288, 4096), (16, 512, 208)):
+        x, r = _randn(m, k, dtype=bf, seed=53), _randn(m, n, dtype=bf, seed=54)
+        w = _randn(n, k, dtype=bf, seed=55, scale=0.05)
+        tiled = hip.tile_weight(w)
+        want = r.clone()
+        assert hip.linear_add(x, w, tiled, want) is True
+        stats = hip.linear_add(x, w, tiled, r, want_stats=True)
+        assert torch.equal(r, want) and stats.shape == (n // 16, 16)
+        assert torch.allclose(stats.sum(0)[:m], r.float().pow(2).sum(-1), rtol=1e-5) and not stats[:, m:].any()
+    table = _randn(500, 4096, dtype=bf, seed=56)
+    ids = torch.tensor([3, 499, 0, 3, 77], dtype=torch.int32).cuda()
+    rows, stats = hip.embedding(ids, table, None, want_stats=True)
+    assert torch.equal(rows, table[ids.long()]) and torch.allclose(stats[0, :5], rows.float().pow(2).sum(-1), rtol=1e-5)
+    rows, stats = hip.embedding(torch.zeros(40, dtype=torch.int32).cuda(), table, None, want_stats=True)
+    assert stats is None                                                               # more rows than a folded norm serves
+
+
 def test_fused_gate_up_is_the_two_kernels(hip, monkeypatch):
     for m, k, inter in ((1, 4096, 12288), (8, 4096, 12288), (16, 512, 208), (3, 1024, 1024), (5, 256, 48)):
         x = _randn(m, k, dtype=torch.bfloat16, seed=30)

@@ -128,6 +128,31 @@ def test_long_decoding_and_first_tokens(folders, name, dtype, device):
     rep.cache.check()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B-sharp"])
+def test_norms_folded_into_the_products_that_read_them(folders, name, dtype):
+    """Steps of few rows fold each block's norms into the q/k/v and the gate/up products (weights times the norm's
+    weight, rows scaled by the norm's factor from statistics the kernel before left). On the CPU the kernel twin
+    stands in for that path: the parts' logic of deferring a norm, passing the rows' statistics along the residual
+    stream and falling back for portions of more than 16 rows is what runs here. Same logits, every way of cutting."""
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    folder, requests = folders[name], _requests(name)
+    kernels = TorchKernels()
+    kernels.fold_norms = True
+    loaded = load_model(folder, device="cpu", dtype=dtype, kernels=kernels, page_size=MODELS[name][3], max_seqs=4,
+                        max_model_len=512, max_step_tokens=512, cache_tokens=256)
+    block = loaded.model.blocks[0]
+    assert block._mixer_defers and block._ffn_defers and block.mixer.qkv.folded is block.input_norm
+    rep = Replayer(loaded)
+    got = H.run_trace(rep, H.trace_decode_tail("r1", requests["r1"], 40))         # 30 rows whole, then one by one
+    _check(folder, dtype, requests, got, f"{name} {dtype} folded norms, decode tail")
+    got = H.run_trace(rep, H.trace_chunks("r3", requests["r3"], [7, 2, 13, 16, 17, 30, 5]))
+    _check(folder, dtype, requests, got, f"{name} {dtype} folded norms, portions")
+    got = H.run_trace(rep, H.trace_mixed(requests, 2))
+    _check(folder, dtype, requests, got, f"{name} {dtype} folded norms, mixed")
+
+
 @pytest.mark.parametrize("device", DEVICES)
 def test_logits_do_not_depend_on_the_cut_in_float32(folders, device):
     """Beyond the comparison with the plain model: the same position computed whole, in portions and one by one
