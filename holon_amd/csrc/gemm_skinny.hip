@@ -29,12 +29,54 @@ struct RowScale {
   float eps, inv_dim;
 };
 
-// This lane's share of the sum of squares of row c: parts wave * 4 + g, then every 4 * WPB-th.
+// The sums of squares are read 16 parts at a time: lane l of a wave takes four floats of part 16 k + l / 4, columns
+// 4 (l % 4) .. + 3, so a wave's load is one contiguous kilobyte; wave w takes chunks k = w, w + WPB, ... and adds them
+// in that order. The values are asked for a few at a time, at the top of each round of the weight loop, and added one
+// round later: loads return in the order they were issued, so by then they have arrived behind the weights that the
+// round before waited for, and the sum never makes the stream wait.
 template <int WPB>
-__device__ __forceinline__ float row_scale_share(const RowScale& rs, int wave, int g, int c) {
-  float ss = 0.f;
-  for (int j = wave * 4 + g; j < rs.parts; j += 4 * WPB) ss += rs.stats[j * 16 + c];
-  return ss;
+struct RowSums {
+  static constexpr int Q = 4;   // loads in flight per lane
+  const f32x4_t* at;            // this lane's four floats of the next chunk
+  int part, parts;              // the part they belong to; how many there are
+  int n;                        // loads in flight
+  f32x4_t v[Q], ss;
+  __device__ __forceinline__ void start(const RowScale& rs, int wave, int lane) {
+    at = reinterpret_cast<const f32x4_t*>(rs.stats) + wave * 64 + lane;
+    part = wave * 16 + lane / 4;
+    parts = rs.stats != nullptr ? rs.parts : 0;
+    n = 0;
+    ss = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  __device__ __forceinline__ void turn() {   // add what the last turn asked for, ask for the next
+#pragma unroll
+    for (int q = 0; q < Q; ++q)
+      if (q < n) ss += v[q];
+    n = 0;
+#pragma unroll
+    for (int q = 0; q < Q; ++q)
+      if (part + q * 16 * WPB < parts) {
+        v[q] = at[(int64_t)q * 64 * WPB];
+        n = q + 1;
+      }
+    at += (int64_t)n * 64 * WPB;
+    part += n * 16 * WPB;
+  }
+  __device__ __forceinline__ f32x4_t finish() {
+    do turn(); while (n > 0);
+    return ss;
+  }
+};
+// After the waves' shares have been added: the sum over the 16 lanes that hold the same four columns (lanes l, l ^ 4,
+// l ^ 8, l ^ 16, l ^ 32, in that order), then column c out of lane c / 4. Every lane of column c gets the same sum.
+__device__ __forceinline__ float row_sum_of_column(f32x4_t v, int c) {
+#pragma unroll
+  for (int o = 4; o < WAVE; o <<= 1)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] += __shfl_xor(v[i], o, WAVE);
+  const float t0 = __shfl(v[0], c / 4, WAVE), t1 = __shfl(v[1], c / 4, WAVE), t2 = __shfl(v[2], c / 4, WAVE),
+              t3 = __shfl(v[3], c / 4, WAVE);
+  return c % 4 == 0 ? t0 : (c % 4 == 1 ? t1 : (c % 4 == 2 ? t2 : t3));
 }
 // The four lane groups' shares of row c, added in order; every lane of column c gets the same sum.
 __device__ __forceinline__ float over_lane_groups(float v, int c) {
@@ -50,7 +92,7 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
                                                                 int M, int N, int K, int round_first, RowScale rs,
                                                                 float* __restrict__ stats_out) {
   __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * MT * WAVE : 1];
-  __shared__ float red_ss[WPB > 1 ? (WPB - 1) * WAVE : 1];
+  __shared__ f32x4_t red_ss[WPB > 1 ? (WPB - 1) * WAVE : 1];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
   const int n0 = blockIdx.x * 16;
@@ -66,11 +108,12 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
   bool have[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) have[t] = t * 16 + c < M;
-  float ss = 0.f;                                // (asked for now: it arrives while the weights stream)
-  if (MT == 1 && rs.stats != nullptr) ss = row_scale_share<WPB>(rs, wave, g, c);
+  RowSums<WPB> sums;
+  sums.start(rs, wave, lane);
 
   int s = 0;
   for (; s + UNROLL <= steps; s += UNROLL) {
+    if (MT == 1) sums.turn();
     bf16x8_t wf[UNROLL], xf[UNROLL][MT];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
@@ -105,6 +148,7 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc[t], 0, 0, 0);
     }
   }
+  f32x4_t ss = MT == 1 ? sums.finish() : f32x4_t{0.f, 0.f, 0.f, 0.f};
   if (WPB > 1) {
     if (wave > 0) {
 #pragma unroll
@@ -120,7 +164,7 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
     }
   }
   if (MT == 1 && rs.stats != nullptr) {          // the norm's scale of row c, on the float32 sums before they are rounded
-    const float inv = 1.0f / sqrtf(over_lane_groups(ss, c) * rs.inv_dim + rs.eps);
+    const float inv = 1.0f / sqrtf(row_sum_of_column(ss, c) * rs.inv_dim + rs.eps);
     acc[0] *= inv;
   }
   float mine = 0.f;                              // RESID with stats_out: the squares of the residual values written
@@ -258,7 +302,7 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t*
                                                                     bf16_t* __restrict__ y, int M, int I, int K,
                                                                     RowScale rs) {
   __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * 2 * MT * WAVE : 1];
-  __shared__ float red_ss[WPB > 1 ? (WPB - 1) * WAVE : 1];
+  __shared__ f32x4_t red_ss[WPB > 1 ? (WPB - 1) * WAVE : 1];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
   const int n0 = blockIdx.x * 16;
@@ -279,10 +323,11 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t*
     acc[0][t] = acc[1][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     have[t] = t * 16 + c < M;
   }
-  float ss = 0.f;
-  if (MT == 1 && rs.stats != nullptr) ss = row_scale_share<WPB>(rs, wave, g, c);
+  RowSums<WPB> sums;
+  sums.start(rs, wave, lane);
   int s = 0;
   for (; s + UNROLL <= steps; s += UNROLL) {
+    if (MT == 1) sums.turn();
     bf16x8_t wf[2][UNROLL], xf[UNROLL][MT];
 #pragma unroll
     for (int h = 0; h < 2; ++h)
@@ -324,6 +369,7 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t*
       acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, xf, acc[1][t], 0, 0, 0);
     }
   }
+  f32x4_t ss = MT == 1 ? sums.finish() : f32x4_t{0.f, 0.f, 0.f, 0.f};
   if (WPB > 1) {
     if (wave > 0) {
 #pragma unroll
@@ -343,7 +389,7 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t*
     }
   }
   if (MT == 1 && rs.stats != nullptr) {
-    const float inv = 1.0f / sqrtf(over_lane_groups(ss, c) * rs.inv_dim + rs.eps);
+    const float inv = 1.0f / sqrtf(row_sum_of_column(ss, c) * rs.inv_dim + rs.eps);
     acc[0][0] *= inv;
     acc[1][0] *= inv;
   }
