@@ -220,13 +220,13 @@ static void launch_skinny(const void* x, const void* w, void* y, int M, int N, i
 }
 
 // How many waves share a tile, from the shapes alone (so a result never depends on M): wide outputs have tiles
-// enough to fill the GPU with few waves each and long loops; narrow ones split K 16 ways. Measured on MI355X.
+// enough to fill the GPU with eight waves each; narrow ones split K 16 ways. Measured on MI355X.
 template <int MT, typename OutT, bool RESID = false>
 static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s,
                       int round_first = 0, RowScale rs = RowScale{nullptr, 0, 0.f, 0.f}, float* stats_out = nullptr) {
   const int tiles = N / 16;
   int wpb = MT >= 3 ? 8 : 16;                  // 16 waves of 3 or 4 token tiles run out of registers
-  if (tiles >= 1024) wpb = 4;
+  if (tiles >= 320) wpb = 8;                   // (384 tiles, K 4096: 12.7 us against 14.2; 9,496 tiles: 189 against 201 for 4)
   while (wpb > 1 && K % (32 * wpb) != 0) wpb /= 2;
   constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
   switch (wpb) {
@@ -419,13 +419,14 @@ extern "C" int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y,
               M, tiled, parts);
   const RowScale rs{stats, parts, eps, 1.0f / (float)K};
   hipStream_t s = (hipStream_t)stream;
-  const bool few = I / 16 < 512;   // few tile pairs: four waves share each
+  const bool few = I / 16 < 512;   // few tile pairs: four waves share each; otherwise two (measured at 768 pairs, K 4096:
+                                   // 33 us against 36 for one wave a pair at 1 and 8 rows, the same at 16)
 #define GLU(MT, WPB, U)                                                                                              \
   if (tiled) gemm_skinny_glu_kernel<MT, WPB, U, true><<<I / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, \
                                                                                  (bf16_t*)y, M, I, K, rs);           \
   else gemm_skinny_glu_kernel<MT, WPB, U, false><<<I / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,      \
                                                                             (bf16_t*)y, M, I, K, rs)
-  if (M <= 16) { if (few) { GLU(1, 4, 8); } else { GLU(1, 1, 8); } }
+  if (M <= 16) { if (few) { GLU(1, 4, 8); } else { GLU(1, 2, 8); } }
   else { if (few) { GLU(2, 4, 4); } else { GLU(2, 1, 4); } }
 #undef GLU
   HOLON_LAUNCH_OK();
