@@ -364,40 +364,53 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
   constexpr int HPB = 256 / LPH;                     // heads a block covers at a time
   const int t = blockIdx.x;
   const int li = threadIdx.x % LPH;                  // lane within the head
-  // this lane's eight cosines and sines: the same for every head of the token
+  // Everything the block reads is asked for before anything is waited for, the longest chain first: the token's
+  // position (then its cosines and sines, the same for every head of the token), its place in the cache, the head's
+  // values, the norm's weight. A decode step runs this kernel on rows another kernel has just written, and each
+  // round trip for them costs as much as the arithmetic.
+  const int pos = table != nullptr ? positions[t] : 0;
+  const int wpage = pages != nullptr ? write_page[t] : 0, woff = pages != nullptr ? write_off[t] : 0;
   float co[8], si[8];
-  if (table != nullptr) {
-    const float* cs = table + (int64_t)positions[t] * D + (li % (LPH / 2)) * 8;   // the pair's place within the half
-    const float4 c0 = *reinterpret_cast<const float4*>(cs), c1 = *reinterpret_cast<const float4*>(cs + 4);
-    const float4 s0 = *reinterpret_cast<const float4*>(cs + D / 2), s1 = *reinterpret_cast<const float4*>(cs + D / 2 + 4);
-    co[0] = c0.x; co[1] = c0.y; co[2] = c0.z; co[3] = c0.w; co[4] = c1.x; co[5] = c1.y; co[6] = c1.z; co[7] = c1.w;
-    si[0] = s0.x; si[1] = s0.y; si[2] = s0.z; si[3] = s0.w; si[4] = s1.x; si[5] = s1.y; si[6] = s1.z; si[7] = s1.w;
-  }
+  bool have_cs = table == nullptr;
   // a block takes HPB heads, then (with fewer blocks than that along y) the next HPB, ...
   for (int h0 = blockIdx.y * HPB; h0 < total_heads; h0 += gridDim.y * HPB) {
     const int h = h0 + threadIdx.x / LPH;
     const bool active = h < total_heads;             // (shuffles below are executed by every lane)
     const int hh = active ? h : 0;
     const T* src = qkv + (int64_t)t * qkv_stride + (int64_t)hh * D + li * 8;
+    const bool is_v = hh >= heads + kv_heads;
+    const bool is_q = hh < heads;
+    const T* weight = is_q ? q_weight : k_weight;
     float v[8];
+    T w[8];
     if (sizeof(T) == 2) {
       const uint4 raw = *reinterpret_cast<const uint4*>(src);
+      if (weight != nullptr) *reinterpret_cast<uint4*>(w) = *reinterpret_cast<const uint4*>(weight + li * 8);
       const T* e = reinterpret_cast<const T*>(&raw);
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = Elem<T>::load(e[j]);
     } else {
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = Elem<T>::load(src[j]);
+      if (weight != nullptr) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = weight[li * 8 + j];
+      }
     }
-    const bool is_v = hh >= heads + kv_heads;
-    const bool is_q = hh < heads;
+    if (!have_cs) {
+      const float* cs = table + (int64_t)pos * D + (li % (LPH / 2)) * 8;   // the pair's place within the half
+      const float4 c0 = *reinterpret_cast<const float4*>(cs), c1 = *reinterpret_cast<const float4*>(cs + 4);
+      const float4 s0 = *reinterpret_cast<const float4*>(cs + D / 2), s1 = *reinterpret_cast<const float4*>(cs + D / 2 + 4);
+      co[0] = c0.x; co[1] = c0.y; co[2] = c0.z; co[3] = c0.w; co[4] = c1.x; co[5] = c1.y; co[6] = c1.z; co[7] = c1.w;
+      si[0] = s0.x; si[1] = s0.y; si[2] = s0.z; si[3] = s0.w; si[4] = s1.x; si[5] = s1.y; si[6] = s1.z; si[7] = s1.w;
+      have_cs = true;
+    }
     if (active && is_v) {   // a value head: transposed inside the page
       const int hk = hh - heads - kv_heads;
-      T* dst = pages + (((int64_t)write_page[t] * 2 + 1) * kv_heads + hk) * (int64_t)page_size * D + write_off[t];
+      T* dst = pages + (((int64_t)wpage * 2 + 1) * kv_heads + hk) * (int64_t)page_size * D + woff;
 #pragma unroll
       for (int j = 0; j < 8; ++j) dst[(int64_t)(li * 8 + j) * page_size] = Elem<T>::store(v[j]);
     }
-    const T* weight = is_q ? q_weight : k_weight;
     if (weight != nullptr) {
       float ss = 0.f;
 #pragma unroll
@@ -405,13 +418,6 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
 #pragma unroll
       for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
       const float inv = 1.0f / sqrtf(ss / (float)D + eps);
-      T w[8];
-      if (sizeof(T) == 2) {
-        *reinterpret_cast<uint4*>(w) = *reinterpret_cast<const uint4*>(weight + li * 8);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) w[j] = weight[li * 8 + j];
-      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = Elem<T>::round((v[j] * inv) * Elem<T>::load(w[j]));
     }
@@ -424,8 +430,8 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
     }
     if (!active || is_v) continue;
     T* dst = is_q ? q_out + ((int64_t)t * heads + hh) * D + li * 8
-                  : pages + (((int64_t)write_page[t] * 2 + 0) * kv_heads + (hh - heads)) * (int64_t)page_size * D +
-                        (int64_t)write_off[t] * D + li * 8;
+                  : pages + (((int64_t)wpage * 2 + 0) * kv_heads + (hh - heads)) * (int64_t)page_size * D +
+                        (int64_t)woff * D + li * 8;
     if (sizeof(T) == 2) {
       uint4 out;
       T* oe = reinterpret_cast<T*>(&out);

@@ -110,6 +110,12 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
   for (int t = 0; t < MT; ++t) have[t] = t * 16 + c < M;
   RowSums<WPB> sums;
   sums.start(rs, wave, lane);
+  ushort4 before[MT];                            // RESID: the residual values this lane will add to, asked for now so
+  if constexpr (RESID) {                         // that they are here when the sums are
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+      if (wave == 0 && have[t]) before[t] = *reinterpret_cast<const ushort4*>(y + (int64_t)(t * 16 + c) * N + n0 + 4 * g);
+  }
 
   int s = 0;
   for (; s + UNROLL <= steps; s += UNROLL) {
@@ -185,7 +191,7 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
       o.x = float_to_bf16(acc[t][0]); o.y = float_to_bf16(acc[t][1]);
       o.z = float_to_bf16(acc[t][2]); o.w = float_to_bf16(acc[t][3]);
       if constexpr (RESID) {
-        const ushort4 r = *reinterpret_cast<const ushort4*>(yp);
+        const ushort4 r = before[t];
         o.x = float_to_bf16(bf16_to_float(r.x) + bf16_to_float(o.x));
         o.y = float_to_bf16(bf16_to_float(r.y) + bf16_to_float(o.y));
         o.z = float_to_bf16(bf16_to_float(r.z) + bf16_to_float(o.z));
