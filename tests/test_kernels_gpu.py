@@ -68,6 +68,34 @@ def test_embedding_and_silu_mul(hip, dtype):
     assert torch.equal(hip.silu_mul(gu), torch.zeros(2, 4, dtype=dtype).cuda())
 
 
+def test_silu_is_rounded_before_the_multiply(hip):
+    """The reference multiplies silu(gate), rounded to the activation dtype, by up (std/holon_std/ffn/reference.py:
+    7-12). Where rounding first and rounding only the product give different bfloat16 results, the kernels give the
+    first: alone and fused into the gated product."""
+    bf = torch.bfloat16
+    g = torch.Generator().manual_seed(60)
+    gate = (torch.randn(64, 4096, generator=g) * 2).to(bf)
+    up = torch.randn(64, 4096, generator=g).to(bf)
+    s64 = gate.double() * torch.sigmoid(gate.double())
+    first = (s64.to(bf).float() * up.float()).to(bf)                   # rounded, then multiplied (one more rounding)
+    late = (s64 * up.double()).to(bf)                                  # only the product rounded
+    half_ulp = torch.exp2(torch.frexp(s64.to(bf).double())[1].double() - 1 - 8)      # of silu's bfloat16 neighbour
+    edge = half_ulp - (s64 - s64.to(bf).double()).abs() < 1e-2 * half_ulp            # silu on a rounding edge: skip
+    tell = (first != late) & ~edge
+    assert tell.sum() > 10000                                          # the two orders differ in thousands of places
+    got = hip.silu_mul(torch.cat((gate, up), dim=-1).cuda()).cpu()
+    assert torch.equal(got[tell], first[tell])
+    # the gated product: weights that copy x into gate and up make the product exact, the activation is what is left
+    k = 256
+    x = torch.cat((gate[:16, :128], up[:16, :128]), dim=-1).contiguous()                 # [16, 256]
+    w = torch.zeros(256, k)
+    w[:128, :128] = torch.eye(128)                                     # gate_i = x_i
+    w[128:, 128:] = torch.eye(128)                                     # up_i = x_(128 + i)
+    fused = hip.linear_silu_mul(x.cuda(), w.to(bf).cuda()).cpu()
+    t = tell[:16, :128]
+    assert t.sum() > 20 and torch.equal(fused[t], first[:16, :128][t])
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize(("head_dim", "rotary_dim", "theta"), [(128, 128, 1e6), (256, 64, 1e7), (48, 48, 1e4), (16, 8, 1e4)])
 def test_rope(hip, dtype, head_dim, rotary_dim, theta):
