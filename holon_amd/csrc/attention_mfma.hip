@@ -520,7 +520,7 @@ __host__ __device__ inline TileMap32 tile_map32(int group) {
 }
 
 template <int D>
-__global__ void __launch_bounds__(256) attn_prefill_wide_kernel(AttnArgs a) {
+__global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kernel(AttnArgs a) {
   constexpr int KP = D + 8;    // pitch of a key row in LDS (elements)
   constexpr int VP = 40;       // pitch of a value row: 32 keys + 8
   __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][32 * KP];
@@ -632,7 +632,8 @@ __global__ void __launch_bounds__(256) attn_prefill_wide_kernel(AttnArgs a) {
         *reinterpret_cast<bf16x8_t*>(&v_lds[buf][v_dst[i]]) = r.v[i];
       }
     };
-    auto stage = [&](int kb, int buf, Regs& next) {
+    // `last`: the stage holds the row's last key (std::true_type) and may reach past it; nothing is staged behind it.
+    auto stage = [&](auto last, int kb, int buf, Regs& next) {
       if (kb <= tile_last) {
         f32x16_t sc;
 #pragma unroll
@@ -648,7 +649,7 @@ __global__ void __launch_bounds__(256) attn_prefill_wide_kernel(AttnArgs a) {
         for (int db = 0; db < D / 32; ++db) {
           vf[db][0] = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(db * 32 + c) * VP + 8 * h]);
           vf[db][1] = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(db * 32 + c) * VP + 16 + 8 * h]);
-          if (kb + 31 > key_hi) {
+          if constexpr (decltype(last)::value) {
             zero_after(vf[db][0], kb + 8 * h, key_hi);
             zero_after(vf[db][1], kb + 16 + 8 * h, key_hi);
           }
@@ -698,9 +699,11 @@ __global__ void __launch_bounds__(256) attn_prefill_wide_kernel(AttnArgs a) {
           o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][1], pb1, o[db], 0, 0, 0);
         }
       }
-      stash(buf ^ 1, next);
-      fetch(kb + 96, next);
-      lds_barrier();
+      if constexpr (!decltype(last)::value) {
+        stash(buf ^ 1, next);
+        fetch(kb + 96, next);
+        lds_barrier();
+      }
     };
     const int kb_first = (key_lo / 32) * 32;
     lds_barrier();               // the previous pass has finished reading both buffers
@@ -709,9 +712,16 @@ __global__ void __launch_bounds__(256) attn_prefill_wide_kernel(AttnArgs a) {
     stash(0, r0);
     fetch(kb_first + 64, r0);
     lds_barrier();
-    for (int kb = kb_first; kb <= key_hi; kb += 64) {
-      stage(kb, 0, r1);
-      if (kb + 32 <= key_hi) stage(kb + 32, 1, r0);
+    int kb = kb_first;
+    for (; kb + 32 < kb_last; kb += 64) {        // pairs of stages that both lie before the last one
+      stage(std::false_type{}, kb, 0, r1);
+      stage(std::false_type{}, kb + 32, 1, r0);
+    }
+    if (kb < kb_last) {
+      stage(std::false_type{}, kb, 0, r1);
+      stage(std::true_type{}, kb + 32, 1, r0);
+    } else {
+      stage(std::true_type{}, kb, 0, r1);
     }
     float lt = l + __shfl_xor(l, 32, WAVE);
     if (valid) {
