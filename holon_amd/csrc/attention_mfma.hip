@@ -53,6 +53,8 @@ struct AttnArgs {
   float* part_o;           // [n_rows, Hq, splits, D]
   float* part_ml;          // [n_rows, Hq, splits, 2]
   int splits, keys_per_split;
+  // long prompt portions only: a block runs one of its two ranges (blockIdx.z = 2 row + which), not both
+  int unpaired;
 };
 
 // How the 16 rows of a tile map to (position, head) for a group of G heads.
@@ -507,6 +509,9 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
 //   O^T (32 dims x 32 queries) += V^T P^T: A = 32 dims x 16 keys from LDS (values are transposed there as in the
 //     pages), B = P^T from the registers above.
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+#ifndef UNPAIR_BELOW
+#define UNPAIR_BELOW 512
+#endif
 
 struct TileMap32 {
   int rows_per_pos;   // min(G, 32)
@@ -529,7 +534,7 @@ __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kerne
   __shared__ int32_t pg_lds[PG];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, tid = threadIdx.x;
   const int h = lane / 32, c = lane % 32;
-  const int b = a.row_ids[blockIdx.z];
+  const int b = a.row_ids[a.unpaired ? blockIdx.z / 2 : blockIdx.z];
   const int group = a.heads / a.kv_heads;      // <= 32 (the host checks)
   const TileMap32 tm = tile_map32(group);
   const int hk = blockIdx.y;
@@ -569,7 +574,10 @@ __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kerne
   // the row of this lane's column: position c / rows_per_pos of the tile, head c % rows_per_pos of the group
   const int pi = c / tm.rows_per_pos, hi = c % tm.rows_per_pos;
 
-  for (int pass = 0; pass < 2; ++pass) {
+  // Paired, a block runs range x and then its mirror image, which together see the same number of keys in every block.
+  // Unpaired, the two are blocks of their own, the long one first in launch order: twice the blocks for short prompts.
+  const int pass_lo = a.unpaired ? 1 - (int)(blockIdx.z % 2) : 0, pass_hi = a.unpaired ? pass_lo + 1 : 2;
+  for (int pass = pass_lo; pass < pass_hi; ++pass) {
     const int range = pass == 0 ? (int)blockIdx.x : n_ranges - 1 - (int)blockIdx.x;
     if (pass == 1 && range <= (int)blockIdx.x) break;
     const int p_lo = range * 4 * tm.pos_per_tile;
@@ -894,7 +902,10 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
     const int ranges32 = ((max_query + tm32.pos_per_tile - 1) / tm32.pos_per_tile + 3) / 4;
     if (heads / kv_heads <= 32) {   // tiles of 32 rows (measured faster at every length: 2,048 tokens 89 against 95 us,
                                     // 32,768 tokens 11.1 against 13.3 ms); larger groups keep tiles of 16
-      dim3 lgrid((ranges32 + 1) / 2, kv_heads, n_rows);
+      // fewer than two paired blocks a compute unit: the ranges of a pair as blocks of their own, so that a second
+      // wave on every SIMD hides the first one's waits
+      a.unpaired = (int64_t)((ranges32 + 1) / 2) * kv_heads * n_rows < UNPAIR_BELOW ? 1 : 0;
+      dim3 lgrid((ranges32 + 1) / 2, kv_heads, a.unpaired ? 2 * n_rows : n_rows);
       if (head_dim == 64) attn_prefill_wide_kernel<64><<<lgrid, 256, 0, ls>>>(a);
       else attn_prefill_wide_kernel<128><<<lgrid, 256, 0, ls>>>(a);
     } else if (blocks2 >= 512) {
