@@ -1,6 +1,7 @@
-// Sampling on the device: argmax, and temperature / top-k / top-p / min-p sampling by inverse CDF in vocabulary order
-// with a counter-based uniform (a hash of seed and position: no generator state, so a request's draws do not depend on
-// batching). One block per row.
+// Sampling on the device: argmax, and temperature / top-k / top-p / min-p sampling by inverse CDF with a counter-based
+// uniform (a hash of seed and position: no generator state, so a request's draws do not depend on batching). A row
+// without a filter is walked in vocabulary order; a row with one in the order its filters sort it (largest value first,
+// equal values by index), which is the order the kept tokens come out of the filters in. One block per row.
 #include <type_traits>
 
 #include "common.h"
@@ -155,9 +156,9 @@ __device__ __forceinline__ float key_float(uint32_t k) {
 // Filters in order (the reference's): top-k keeps the k largest (ties: lower index first); top-p keeps, in descending
 // order, tokens whose preceding mass is <= top_p of the top-k mass (the largest always stays); min-p keeps q >= min_p
 // times the largest q. A token is identified for ties by (value, index), so the kept set is exact.
-// The general form: any k, any kept set. Bisection on the ordered keys, one pass over the row per step, every thread
-// a contiguous segment of the row (so that ranks among equal values follow the index): exact but slow, for the rows
-// whose kept set does not fit the fast form below.
+// The general form: any k, any kept set, and the draw in sorted order. Bisection on the ordered keys, one pass over the
+// row per step, every thread a contiguous segment of the row (so that ranks among equal values follow the index):
+// exact but slow, for the rows whose kept set does not fit the fast form below.
 __device__ void sample_row_general(const float* __restrict__ row, int32_t* __restrict__ out_r, int vocab, float inv_temp,
                                    ArgMax top, int k, float p_keep, float p_min, float u) {
   const float xmax = top.v;
@@ -182,7 +183,6 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
   const int seg = (vocab + blockDim.x - 1) / blockDim.x;
   const int seg_lo = min(vocab, (int)threadIdx.x * seg), seg_hi = min(vocab, seg_lo + seg);
   __shared__ int scan_i[SAMPLE_THREADS];
-  __shared__ float scan_f[SAMPLE_THREADS];
   int ties_before = 0;           // tokens equal to the k-th value in earlier segments
   if (ties_kept != 0x7fffffff) {
     int mine = 0;
@@ -279,41 +279,68 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
     return qv;
   };
 
-  // --- draw: inverse CDF in vocabulary order over segment sums
+  // --- draw: inverse CDF in sorted order (value descending, equal values by index). The drawn token's key is the
+  // smallest K with kept mass above K (strictly) <= target; among the kept tokens equal to K, the one whose rank times
+  // their common mass first passes what the target leaves.
   float mine = 0.f;
   {
     int tie_rank = ties_before, p_rank = p_ties_before;
     for (int i = seg_lo; i < seg_hi; ++i) mine += law(row[i] * inv_temp, tie_rank, p_rank);
   }
-  scan_f[threadIdx.x] = mine;
+  const float total = block_sum(mine);
+  const float target = u * total;
+  uint32_t d_key;
+  {
+    uint32_t lo = 0, hi = float_key(xmax);
+    while (lo < hi) {
+      const uint32_t mid = lo + (hi - lo) / 2;
+      float above = 0.f;
+      int tie_rank = ties_before, p_rank = p_ties_before;
+      for (int i = seg_lo; i < seg_hi; ++i) {
+        const float x = row[i] * inv_temp;
+        const float qv = law(x, tie_rank, p_rank);
+        if (float_key(x) > mid) above += qv;
+      }
+      if (block_sum(above) <= target) hi = mid; else lo = mid + 1;
+    }
+    d_key = lo;
+  }
+  float above = 0.f;
+  int ties_mine = 0;
+  {
+    int tie_rank = ties_before, p_rank = p_ties_before;
+    for (int i = seg_lo; i < seg_hi; ++i) {
+      const float x = row[i] * inv_temp;
+      const float qv = law(x, tie_rank, p_rank);
+      const uint32_t key = float_key(x);
+      if (key > d_key) above += qv;
+      ties_mine += key == d_key && qv > 0.f;
+    }
+  }
+  above = block_sum(above);
+  scan_i[threadIdx.x] = ties_mine;
   __syncthreads();
-  __shared__ float total_s;
+  __shared__ int n_ties_s;
   if (threadIdx.x == 0) {
-    float run = 0.f;
-    for (int t = 0; t < (int)blockDim.x; ++t) { const float v = scan_f[t]; scan_f[t] = run; run += v; }
-    total_s = run;
+    int run = 0;
+    for (int t = 0; t < (int)blockDim.x; ++t) { const int v = scan_i[t]; scan_i[t] = run; run += v; }
+    n_ties_s = run;
   }
   __syncthreads();
-  const float before = scan_f[threadIdx.x];
-  const float target = u * total_s;
+  const int d_before = scan_i[threadIdx.x], n_ties = n_ties_s;
+  const float each = expf(key_float(d_key) - xmax);
+  int want = each > 0.f ? (int)fminf((target - above) / each, 2147483000.f) : 0;
+  want = max(0, min(want, n_ties - 1));
   __shared__ int chosen;
   if (threadIdx.x == 0) chosen = -1;
   __syncthreads();
-  // the segment whose running mass first exceeds the target; the last segment with mass takes what rounding leaves
-  const float next = (threadIdx.x + 1 < blockDim.x) ? scan_f[threadIdx.x + 1] : total_s;
-  const bool last_with_mass = mine > 0.f && next == total_s;
-  if (mine > 0.f && ((before <= target && target < next) || (last_with_mass && target >= next))) {
-    int tie_rank = ties_before, p_rank = p_ties_before, pick = -1, last = -1;
-    float run = before;
+  if (ties_mine > 0 && d_before <= want && want < d_before + ties_mine) {   // (one thread)
+    int tie_rank = ties_before, p_rank = p_ties_before, rank = d_before;
     for (int i = seg_lo; i < seg_hi; ++i) {
-      const float qv = law(row[i] * inv_temp, tie_rank, p_rank);
-      if (qv > 0.f) {
-        last = i;
-        run += qv;
-        if (pick < 0 && run > target) pick = i;
-      }
+      const float x = row[i] * inv_temp;
+      const float qv = law(x, tie_rank, p_rank);
+      if (float_key(x) == d_key && qv > 0.f && rank++ == want) { chosen = i; break; }
     }
-    atomicMax(&chosen, pick >= 0 ? pick : last);
   }
   __syncthreads();
   if (threadIdx.x == 0) *out_r = chosen >= 0 ? chosen : top.i;
@@ -329,8 +356,9 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
 //      order in which top-k and top-p take tokens. If no such set fits, the row takes the general form;
 //   3. top-k keeps the first k of the sorted set; top-p those whose preceding mass is <= top_p * (mass of what top-k
 //      kept); both keep a prefix, so the kept set is "(value, index) at or before the last kept one": one compare;
-//   4. min-p drops q < min_p (the largest q is 1); the draw is the inverse CDF in vocabulary order over the integer
-//      masses: sums of 256 consecutive tokens, the 256 that hold the target found among those sums, one scan of them.
+//   4. min-p drops q < min_p (the largest q is 1): a prefix again; the draw is the inverse CDF over the integer masses
+//      of the kept tokens as they lie sorted. A row without a filter is drawn in vocabulary order instead: sums of 256
+//      consecutive tokens, the 256 that hold the target found among those sums, one scan of them.
 #define SAMPLE_CANDIDATES 4096
 #define SAMPLE_WAVES (SAMPLE_THREADS / WAVE)
 #define SAMPLE_PER (SAMPLE_CANDIDATES / SAMPLE_THREADS)
@@ -595,147 +623,177 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
   const float u = hashed_uniform((uint64_t)seeds[pr], position);
   const bool k_on = k > 0 && k < vocab, p_on = p_keep < 1.0f;
   const int chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
-  if ((k_on && k > SAMPLE_CANDIDATES) || vocab > 255 * SAMPLE_THREADS) {      // (uniform over the block)
+  const bool m_on = p_min > 0.f;
+  const bool filtered = k > 0 || p_on || m_on;
+  if (filtered && ((k_on && k > SAMPLE_CANDIDATES) || vocab > 255 * SAMPLE_THREADS)) {      // (uniform over the block)
     sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
     return;
   }
 
-  u64 cut = 0;                                  // tokens with order_key >= cut pass top-k and top-p
-  if (k_on || p_on) {
-    u64 z_all = 0;
-    if (p_on && !k_on) {                         // top-p without top-k: the mass of the whole row
-      u64 mass = 0;
-      for_each_token(row, vocab, inv_temp, [&](float x, int) { mass += fixed_mass(__expf(x - xmax)); });
-      z_all = block_sum_u64(mass);
-    }
-    estimate_band_counts(row, vocab, inv_temp, xmax, counts, band_counts);
-    // Which bands to collect: the fewest that should hold twice what is needed (k tokens; 256 for top-p alone). The
-    // collecting counts exactly; too many, or fewer than k, and another set of bands is tried.
-    const int need = k_on ? k : 1;
-    u64 wide_cut = 0;                            // set when the kept set is too large to collect: drawn as below
-    int beyond_at = -1;                          // the most bands found to hold too little of the mass
-    int bands = SAMPLE_BANDS - 1;
-    for (int j = SAMPLE_BANDS - 1; j >= 0; --j)
-      if (counts[j] >= 2 * (k_on ? k : 256) + 64) bands = j;
-    while (bands > 0 && counts[bands] > SAMPLE_CANDIDATES / 2 && counts[bands - 1] >= 2 * need) --bands;
-    int count = 0;
-    for (int attempt = 0;; ++attempt) {
-      if (attempt == 6 || bands < 0 || bands >= SAMPLE_BANDS) {
-        if (p_on && !k_on) wide_cut = top_p_cut_wide(row, vocab, inv_temp, xmax, (u64)((double)p_keep * (double)z_all),
-                                                     cand, &n_cand);
-        if (wide_cut == 0) {
-          sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
-          return;
+  // A row with a filter. Its kept set is a prefix of the sorted order; where that prefix fits the room in LDS it is
+  // collected, sorted and drawn from there, else (`wide`) it is described by `cut`: tokens with order_key >= cut pass
+  // top-k and top-p (0: all do), and min-p is a bound on q.
+  if (filtered) {
+    u64 cut = 0;
+    bool wide = !(k_on || p_on || m_on);         // k >= vocab and nothing else: everything is kept, in sorted order
+    if (k_on || p_on) {
+      u64 z_all = 0;
+      if (!k_on) {                               // top-p without top-k: the mass of the whole row
+        u64 mass = 0;
+        for_each_token(row, vocab, inv_temp, [&](float x, int) { mass += fixed_mass(__expf(x - xmax)); });
+        z_all = block_sum_u64(mass);
+      }
+      estimate_band_counts(row, vocab, inv_temp, xmax, counts, band_counts);
+      // Which bands to collect: the fewest that should hold twice what is needed (k tokens; 256 for top-p alone). The
+      // collecting counts exactly; too many, or fewer than k, and another set of bands is tried.
+      const int need = k_on ? k : 1;
+      int beyond_at = -1;                        // the most bands found to hold too little of the mass
+      int bands = SAMPLE_BANDS - 1;
+      for (int j = SAMPLE_BANDS - 1; j >= 0; --j)
+        if (counts[j] >= 2 * (k_on ? k : 256) + 64) bands = j;
+      while (bands > 0 && counts[bands] > SAMPLE_CANDIDATES / 2 && counts[bands - 1] >= 2 * need) --bands;
+      for (int attempt = 0;; ++attempt) {
+        if (attempt == 6 || bands < 0 || bands >= SAMPLE_BANDS) {
+          if (!k_on) cut = top_p_cut_wide(row, vocab, inv_temp, xmax, (u64)((double)p_keep * (double)z_all), cand, &n_cand);
+          if (cut == 0) {
+            sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
+            return;
+          }
+          wide = true;
+          break;
         }
-        break;
-      }
-      count = collect_bands(row, vocab, inv_temp, xmax, bands, cand, &n_cand);
-      if (count > SAMPLE_CANDIDATES) {
-        --bands;
-        if (bands <= beyond_at) attempt = 5;      // the next fewer bands held too little: no set of bands will do
-        continue;
-      }
-      if (count < need && count < vocab) { ++bands; continue; }
-      int n_pad = WAVE;
-      while (n_pad < count) n_pad <<= 1;
-      for (int i = count + tid; i < n_pad; i += blockDim.x) cand[i] = 0;   // after every real key
-      __syncthreads();
-      bitonic_sort(cand, n_pad, true);
-      // masses in sorted order: a thread holds consecutive ones and the sum of everything before them
-      const int per = max(1, n_pad / SAMPLE_THREADS);     // 1, 2 or 4
-      u64 incl[SAMPLE_PER];
-      u64 run = 0;
-#pragma unroll
-      for (int e = 0; e < SAMPLE_PER; ++e) {
-        const int i = tid * per + e;
-        if (e < per && i < count) run += fixed_mass(__expf(key_float((uint32_t)(cand[i] >> 32)) - xmax));
-        incl[e] = run;
-      }
-      u64 cand_mass;
-      const u64 before = block_scan_u64(run, cand_mass);
-      const int k_eff = k_on ? min(k, count) : count;
-      if (tid == 0) n_keep_s = k_eff;
-#pragma unroll
-      for (int e = 0; e < SAMPLE_PER; ++e)
-        if (e < per && tid * per + e == k_eff - 1) z_k_s = before + incl[e];
-      __syncthreads();
-      if (p_on) {
-        const u64 z_k = k_on ? z_k_s : z_all;
-        const u64 bound = (u64)((double)p_keep * (double)z_k);
-        // the kept ones are those whose preceding mass is within the bound: a prefix, as the sums only grow
-        int mine = 0;
+        const int count = collect_bands(row, vocab, inv_temp, xmax, bands, cand, &n_cand);
+        if (count > SAMPLE_CANDIDATES) {
+          --bands;
+          if (bands <= beyond_at) attempt = 5;    // the next fewer bands held too little: no set of bands will do
+          continue;
+        }
+        if (count < need && count < vocab) { ++bands; continue; }
+        int n_pad = WAVE;
+        while (n_pad < count) n_pad <<= 1;
+        for (int i = count + tid; i < n_pad; i += blockDim.x) cand[i] = 0;   // after every real key
+        __syncthreads();
+        bitonic_sort(cand, n_pad, true);
+        // masses in sorted order: a thread holds consecutive ones and the sum of everything before them
+        const int per = max(1, n_pad / SAMPLE_THREADS);     // 1, 2 or 4
+        u64 incl[SAMPLE_PER];
+        u64 run = 0;
 #pragma unroll
         for (int e = 0; e < SAMPLE_PER; ++e) {
           const int i = tid * per + e;
-          if (e < per && i < k_eff) mine += (before + (e ? incl[e - 1] : 0)) <= bound;
+          if (e < per && i < count) run += fixed_mass(__expf(key_float((uint32_t)(cand[i] >> 32)) - xmax));
+          incl[e] = run;
         }
-        const int kept = block_sum_int(mine);
-        if (tid == 0) n_keep_s = kept;
-        __syncthreads();
-      }
-      // top-p alone, and everything collected was kept: the bound may lie past it, in bands not collected
-      if (p_on && !k_on && count < vocab && n_keep_s == count) {
-        __syncthreads();
-        beyond_at = bands;
-        ++bands;
-        while (bands < SAMPLE_BANDS - 1 && counts[bands] < 4 * count) ++bands;   // a good deal more at once
-        continue;
-      }
-      break;
-    }
-    if (wide_cut == 0) {
-    // min-p drops q < min_p: the values only fall along the sorted order, so this keeps a prefix too
-    int ok = 0;
-    for (int i = tid; i < n_keep_s; i += blockDim.x) ok += __expf(key_float((uint32_t)(cand[i] >> 32)) - xmax) >= p_min;
-    const int n_final = max(1, block_sum_int(ok));
-    // the kept tokens in vocabulary order, their masses, and the first whose running mass exceeds the target
-    int n_pad = WAVE;
-    while (n_pad < n_final) n_pad <<= 1;
-    for (int i = tid; i < n_pad; i += blockDim.x) {
-      const u64 c = cand[i];
-      cand[i] = i < n_final ? ((u64)(0x7fffffffu - (uint32_t)c) << 32) | (c >> 32) : ~0ull;   // (index, value key)
-    }
-    __syncthreads();
-    bitonic_sort(cand, n_pad, false);
-    const int per = max(1, n_pad / SAMPLE_THREADS);
-    uint32_t m[SAMPLE_PER];
-    u64 mine = 0;
+        u64 cand_mass;
+        const u64 before = block_scan_u64(run, cand_mass);
+        const int k_eff = k_on ? min(k, count) : count;
+        if (tid == 0) n_keep_s = k_eff;
 #pragma unroll
-    for (int e = 0; e < SAMPLE_PER; ++e) {
-      const int i = tid * per + e;
-      m[e] = (e < per && i < n_final) ? fixed_mass(__expf(key_float((uint32_t)cand[i]) - xmax)) : 0u;
-      mine += m[e];
+        for (int e = 0; e < SAMPLE_PER; ++e)
+          if (e < per && tid * per + e == k_eff - 1) z_k_s = before + incl[e];
+        __syncthreads();
+        if (p_on) {
+          const u64 z_k = k_on ? z_k_s : z_all;
+          const u64 bound = (u64)((double)p_keep * (double)z_k);
+          // the kept ones are those whose preceding mass is within the bound: a prefix, as the sums only grow
+          int mine = 0;
+#pragma unroll
+          for (int e = 0; e < SAMPLE_PER; ++e) {
+            const int i = tid * per + e;
+            if (e < per && i < k_eff) mine += (before + (e ? incl[e - 1] : 0)) <= bound;
+          }
+          const int kept = block_sum_int(mine);
+          if (tid == 0) n_keep_s = kept;
+          __syncthreads();
+        }
+        // top-p alone, and everything collected was kept: the bound may lie past it, in bands not collected
+        if (p_on && !k_on && count < vocab && n_keep_s == count) {
+          __syncthreads();
+          beyond_at = bands;
+          ++bands;
+          while (bands < SAMPLE_BANDS - 1 && counts[bands] < 4 * count) ++bands;   // a good deal more at once
+          continue;
+        }
+        break;
+      }
+    } else if (m_on) {
+      // min-p alone keeps the tokens within -ln(min_p) of the largest value: the bands that reach that far
+      const float reach = -__logf(p_min) + 0.01f;
+      int bands = 0;
+      while (bands < SAMPLE_BANDS && band_edge(bands) < reach) ++bands;
+      wide = true;
+      if (bands < SAMPLE_BANDS) {
+        const int count = collect_bands(row, vocab, inv_temp, xmax, bands, cand, &n_cand);
+        if (count <= SAMPLE_CANDIDATES) {
+          int n_pad = WAVE;
+          while (n_pad < count) n_pad <<= 1;
+          for (int i = count + tid; i < n_pad; i += blockDim.x) cand[i] = 0;
+          __syncthreads();
+          bitonic_sort(cand, n_pad, true);
+          if (tid == 0) n_keep_s = count;
+          __syncthreads();
+          wide = false;
+        }
+      }
     }
-    u64 total;
-    const u64 before = block_scan_u64(mine, total);
-    const u64 target = (u64)((double)u * (double)total);
-    if (tid == 0) pick_s = -1;
-    __syncthreads();
-    if (mine > 0 && before <= target && target < before + mine) {   // (one thread)
-      u64 run = before;
-      int pick = -1;
+    if (!wide) {
+      // min-p drops q < min_p: the values only fall along the sorted order, so this keeps a prefix too
+      int ok = 0;
+      for (int i = tid; i < n_keep_s; i += blockDim.x) ok += __expf(key_float((uint32_t)(cand[i] >> 32)) - xmax) >= p_min;
+      const int n_final = max(1, block_sum_int(ok));
+      // the draw walks the kept tokens as they lie sorted: the first whose running mass exceeds the target
+      int n_pad = WAVE;
+      while (n_pad < n_final) n_pad <<= 1;
+      const int per = max(1, n_pad / SAMPLE_THREADS);
+      uint32_t m[SAMPLE_PER];
+      u64 mine = 0;
 #pragma unroll
       for (int e = 0; e < SAMPLE_PER; ++e) {
-        run += m[e];
-        if (pick < 0 && m[e] > 0 && run > target) pick = (int)(cand[tid * per + e] >> 32);
+        const int i = tid * per + e;
+        m[e] = (e < per && i < n_final) ? fixed_mass(__expf(key_float((uint32_t)(cand[i] >> 32)) - xmax)) : 0u;
+        mine += m[e];
       }
-      pick_s = pick;
+      u64 total;
+      const u64 before = block_scan_u64(mine, total);
+      const u64 target = (u64)((double)u * (double)total);
+      if (tid == 0) pick_s = -1;
+      __syncthreads();
+      if (mine > 0 && before <= target && target < before + mine) {   // (one thread)
+        u64 run = before;
+        int pick = -1;
+#pragma unroll
+        for (int e = 0; e < SAMPLE_PER; ++e) {
+          run += m[e];
+          if (pick < 0 && m[e] > 0 && run > target) pick = (int)(0x7fffffffu - (uint32_t)cand[tid * per + e]);
+        }
+        pick_s = pick;
+      }
+      __syncthreads();
+      if (tid == 0) out[r] = pick_s >= 0 ? pick_s : top.i;
+      return;
     }
-    __syncthreads();
-    if (tid == 0) out[r] = pick_s >= 0 ? pick_s : top.i;
-    return;
-    }
-    cut = wide_cut;
+    // The kept prefix is too long to collect. Its mass, then the token at which the sorted running mass passes the
+    // target: the search for "the last token whose preceding mass is within a bound" that top-p uses, with the target as
+    // the bound (what precedes a kept token is kept, so the search need not know the filters).
     __syncthreads();                            // `cand` is free from here on
+    u64 mass = 0;
+    for_each_token(row, vocab, inv_temp, [&](float x, int i) {
+      const float q = __expf(x - xmax);
+      if (order_key(x, i) >= cut && q >= p_min) mass += fixed_mass(q);
+    });
+    const u64 total = block_sum_u64(mass);
+    const u64 target = (u64)((double)u * (double)total);
+    const u64 hit = total > 0 ? top_p_cut_wide(row, vocab, inv_temp, xmax, target, cand, &n_cand) : 0;
+    if (total > 0 && hit == 0) {                 // thousands of equal values around the target
+      sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
+      return;
+    }
+    if (tid == 0) out[r] = total > 0 ? (int)(0x7fffffffu - (uint32_t)hit) : top.i;
+    return;
   }
 
-  // the law, and the draw in vocabulary order
-  const bool every = cut == 0 && !(p_min > 0.f);   // nothing is dropped: the law is the mass itself
-  auto law = [&](float x, int i, auto all) -> uint32_t {
-    const float q = __expf(x - xmax);
-    if constexpr (decltype(all)::value) return fixed_mass(q);
-    else return (order_key(x, i) >= cut && q >= p_min) ? fixed_mass(q) : 0u;
-  };
+  // no filter: the law is the mass itself, and the draw walks the vocabulary as it lies
+  auto law = [&](float x, int, auto) -> uint32_t { return fixed_mass(__expf(x - xmax)); };
   u64* chunk_mass = cand;                       // [chunks]: the mass of tokens 256 c .. 256 c + 255, four to a lane
   const bool wide = (vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0;
   auto lane_masses = [&](int c, uint32_t (&m)[4], auto all) {
@@ -759,7 +817,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
       if (lane == 0) chunk_mass[c] = sum;
     }
   };
-  if (every) chunk_sums(std::true_type{}); else chunk_sums(std::false_type{});
+  chunk_sums(std::true_type{});
   if (tid == 0) pick_s = -1;
   __syncthreads();
   // a thread holds consecutive chunks; the one whose chunks hold the target names the chunk
@@ -810,6 +868,8 @@ extern "C" int holon_sample(const float* logits, int32_t* out, int rows, int voc
                             const int32_t* top_k, const float* top_p, const float* min_p, const int64_t* seeds,
                             const void* positions, const int32_t* slots, int positions_i32, void* stream) {
   HOLON_CHECK(rows >= 0 && vocab > 0, "sample: bad sizes");
+  HOLON_CHECK(vocab <= SAMPLE_CANDIDATES * SAMPLE_CHUNK, "sample: a vocabulary of %d tokens exceeds the %d this kernel serves",
+              vocab, SAMPLE_CANDIDATES * SAMPLE_CHUNK);
   if (rows == 0) return 0;
   sample_kernel<<<rows, SAMPLE_THREADS, 0, (hipStream_t)stream>>>(logits, out, vocab, temperature, top_k, top_p,
                                                                   min_p, seeds, positions, slots, positions_i32);

@@ -135,7 +135,8 @@ class Kernels(Protocol):
         """One token per row [R] int32. temperature/top_p/min_p float32, top_k int32, seeds int64: [R], row r's own;
         or, with `slots` [R] int32, tables [S] of which row r reads entry slots[r]. positions [R] int32 or int64 (the
         position of the token being drawn). Rows with temperature 0 take the argmax; the others draw by inverse CDF
-        in vocabulary order with the hashed uniform of (seed, position)."""
+        at the hashed uniform of (seed, position): in vocabulary order when the row has no filter (top_k 0, top_p 1,
+        min_p 0), else in sorted order (scaled logit descending, equal ones by index)."""
 
     def scatter_rows(self, dst: torch.Tensor, idx: torch.Tensor, src: torch.Tensor) -> None:
         """dst[idx[r]] = src[r] for int32 rows: dst [N, W], idx [n], src n * W values."""

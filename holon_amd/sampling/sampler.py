@@ -4,8 +4,11 @@ Semantics follow the reference (std/holon_std/sampling/reference.py:1-30, sample
 top-k, then top-p over the renormalised rest (the most likely token always stays), then min-p against the largest
 probability after top-k; temperature 0 is the first maximal index. The draw is an inverse CDF at a counter-based
 uniform, a hash of (seed, position of the token being drawn): no generator state, so what a request draws does not
-depend on batching, chunking or preemption. Where the reference walks filtered rows in sorted order, this sampler
-walks every row in vocabulary order (the law is the same; the token drawn for one uniform may differ).
+depend on batching, chunking or preemption. The inverse CDF walks a row without a filter in vocabulary order and a row
+with one (top-k, top-p or min-p set) in the filters' sorted order, largest value first and equal values by index, as the
+reference does (sampler.py:43-61). One difference remains on purpose: the reference sorts every row of a batch as soon
+as any of its rows has a filter (sampler.py:134-141), so that an unfiltered request's draw depends on its neighbours;
+here a row's order is its own.
 """
 from __future__ import annotations
 

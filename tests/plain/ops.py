@@ -191,7 +191,8 @@ class TorchKernels:
             if float(min_p[r]) > 0:
                 keep &= q >= float(min_p[r]) * q.max()
             q = torch.where(keep, q, 0.0)
-            c = q.cumsum(-1)
-            idx = torch.searchsorted(c, (u[r] * c[-1]).reshape(1), right=True)[0]
-            out[r] = idx.clamp(max=x.numel() - 1)
+            filtered = int(top_k[r]) > 0 or float(top_p[r]) < 1 or float(min_p[r]) > 0
+            c = (q[order] if filtered else q).cumsum(-1)      # a filtered row is walked in the filters' sorted order
+            idx = torch.searchsorted(c, (u[r] * c[-1]).reshape(1), right=True)[0].clamp(max=x.numel() - 1)
+            out[r] = order[idx] if filtered else idx
         return out.to(torch.int32)

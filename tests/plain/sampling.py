@@ -63,9 +63,22 @@ def probs(logits: torch.Tensor, temperature: float, top_k: int = 0, top_p: float
     return torch.where(keep, x, float("-inf")).softmax(-1)
 
 
-def draw(q: torch.Tensor, u: float) -> int:
-    """Inverse CDF in vocabulary order: the first index whose cumulative mass exceeds u * total.
-    std/holon_std/sampling/sampler.py:57-61."""
-    c = q.double().cumsum(-1)
+def drawing_order(logits: torch.Tensor, temperature: float, top_k: int = 0, top_p: float = 1.0, min_p: float = 0.0
+                  ) -> torch.Tensor | None:
+    """The order in which a row's tokens are walked by the draw: vocabulary order (None) when no filter is set, else
+    by scaled logit, largest first, equal ones by index (the sort the filters use). The reference sorts every row of a
+    batch in which any row has a filter; here a row's order is its own, so that its draws do not depend on the batch.
+    std/holon_std/sampling/sampler.py:43-54,134-141."""
+    if temperature == 0 or not (top_k > 0 or top_p < 1 or min_p > 0):
+        return None
+    return (logits.double() / temperature).argsort(descending=True, stable=True)
+
+
+def draw(q: torch.Tensor, u: float, order: torch.Tensor | None = None) -> int:
+    """Inverse CDF over the tokens in `order` (vocabulary order when None): the first whose cumulative mass exceeds
+    u * total. std/holon_std/sampling/sampler.py:57-61."""
+    q = q.double()
+    c = (q if order is None else q[order]).cumsum(-1)
     idx = int(torch.searchsorted(c, torch.tensor(u, dtype=torch.float64) * c[-1], right=True))
-    return min(idx, q.numel() - 1)
+    idx = min(idx, q.numel() - 1)
+    return idx if order is None else int(order[idx])

@@ -70,8 +70,9 @@ def test_tied_tiny_model_greedy(folders, device):
 def _plain_sampled(plain, prompt, n, seed, temperature, **filters):
     ids, out = list(prompt), []
     for _ in range(n):
-        q = S.probs(plain.logits(ids)[-1], temperature, **filters)
-        token = S.draw(q, S.uniform(seed, len(ids)))
+        logits = plain.logits(ids)[-1]
+        q = S.probs(logits, temperature, **filters)
+        token = S.draw(q, S.uniform(seed, len(ids)), S.drawing_order(logits, temperature, **filters))
         out.append(token)
         ids.append(token)
     return out

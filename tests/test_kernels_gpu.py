@@ -530,8 +530,17 @@ def test_argmax_and_sampling(hip):
     assert toks[[0, 2]].tolist() == big[[0, 2]].argmax(-1).tolist()
 
 
+def _at_uniform(law, order, token, u, slack=2e-5):
+    """Whether `token` is where the inverse CDF of `law`, walked in `order` (None: as it lies), puts the uniform `u`."""
+    walk = law if order is None else law[order]
+    at = token if order is None else int((order == token).nonzero()[0])
+    cdf = walk.cumsum(0)
+    return (cdf[at - 1] if at else 0.0) - slack <= u < cdf[at] + slack
+
+
 def test_sampling_filters_at_the_full_vocabulary(hip):
-    """Every draw is the plain sampler's (float64 law, inverse CDF at the hashed uniform) at 151,936 tokens: peaked
+    """Every draw is the plain sampler's (float64 law, inverse CDF at the hashed uniform, a filtered row walked in
+    sorted order) at 151,936 tokens: peaked
     rows whose kept set is small (the fast form: candidates collected and sorted), flat rows and a large k (the
     general form), ties at the edge of top-k and of top-p, k = 1, a tiny top-p."""
     from tests.plain import sampling as S
@@ -543,12 +552,16 @@ def test_sampling_filters_at_the_full_vocabulary(hip):
     order = peaked.argsort(descending=True)
     tied[order[45:55]] = peaked[order[49]]                       # ten equal values around the 50th place
     tied[order[2:5]] = peaked[order[3]]
+    plateau = peaked.clone()
+    plateau[order[:6000]] = peaked[order[0]]
     cases = [(peaked, 0.8, 50, 1.0, 0.0), (peaked, 0.8, 0, 0.9, 0.0), (peaked, 1.0, 50, 0.9, 0.02), (peaked, 0.7, 0, 1.0, 0.05),
              (peaked, 1.0, 1, 1.0, 0.0), (peaked, 1.0, 0, 1e-6, 0.0), (peaked, 1.2, 2048, 0.99, 0.0), (peaked, 1.0, 5000, 1.0, 0.0),
              (flat, 1.0, 0, 0.9, 0.0), (flat, 1.0, 300, 0.5, 0.0), (tied, 1.0, 50, 1.0, 0.0), (tied, 1.0, 48, 0.95, 0.0),
              (tied, 0.9, 4, 1.0, 0.0), (tied, 1.0, 0, 0.5, 0.0), (peaked, 1.0, 0, 1.0, 0.0),
              (peaked * 8, 1.0, 50, 1.0, 0.0), (peaked * 8, 1.0, 0, 0.999, 0.0), (peaked * 8, 0.5, 20, 0.9, 0.0),
-             (peaked * 40, 1.0, 50, 0.9, 0.0)]      # sharp rows: the 50th token lies tens, or hundreds, below the first
+             (peaked * 40, 1.0, 50, 0.9, 0.0),      # sharp rows: the 50th token lies tens, or hundreds, below the first
+             (flat, 1.0, 0, 1.0, 0.2), (peaked, 1.0, 200_000, 1.0, 0.0),   # kept sets too long to collect: min-p alone, all
+             (plateau, 1.0, 0, 0.5, 0.0), (plateau, 1.0, 0, 1.0, 0.5), (plateau, 1.0, 7000, 1.0, 0.0)]   # 6,000 equal values
     n = 48
     for at, (row, temp, top_k, top_p, min_p) in enumerate(cases):
         f = lambda x, dt: torch.full((n,), x, dtype=dt).cuda()
@@ -557,13 +570,13 @@ def test_sampling_filters_at_the_full_vocabulary(hip):
                             f(top_p, torch.float32), f(min_p, torch.float32), f(seed, torch.int64),
                             torch.arange(n, dtype=torch.int64).cuda()).tolist()
         law = S.probs(row, temp, top_k, top_p, min_p)
+        order = S.drawing_order(row, temp, top_k, top_p, min_p)
+        assert (order is None) == (top_k == 0 and top_p == 1.0 and min_p == 0.0)
         assert all(law[t] > 0 for t in tokens), (at, "a filtered token was drawn")
-        cdf = law.cumsum(0)
         for pos, t in enumerate(tokens):                   # the inverse CDF at the hashed uniform, to float32 rounding
-            u = S.uniform(seed, pos)
-            assert (cdf[t - 1] if t else 0.0) - 2e-5 <= u < cdf[t] + 2e-5, (at, pos, t)
-        if row is not flat:        # few tokens carry the mass: a draw then sits well inside its token's share
-            want = [S.draw(law, S.uniform(seed, pos)) for pos in range(n)]
+            assert _at_uniform(law, order, t, S.uniform(seed, pos)), (at, pos, t)
+        if row is not flat and top_k < v:   # few tokens carry the mass: a draw then sits well inside its token's share
+            want = [S.draw(law, S.uniform(seed, pos), order) for pos in range(n)]
             assert sum(a != b for a, b in zip(tokens, want)) <= 1, (at, temp, top_k, top_p, min_p)
     # rows of one batch with different settings do not disturb each other
     rows = torch.stack([peaked, flat, tied, peaked]).cuda()
@@ -572,9 +585,8 @@ def test_sampling_filters_at_the_full_vocabulary(hip):
     p = torch.tensor([1.0, 0.9, 1.0, 1.0], dtype=torch.float32).cuda()
     m = torch.zeros(4, dtype=torch.float32).cuda()
     got = hip.sample(rows, t, k, p, m, torch.full((4,), 5, dtype=torch.int64).cuda(), torch.arange(4).cuda()).tolist()
-    assert got[0] == S.draw(S.probs(peaked, 0.8, 50), S.uniform(5, 0))
-    cdf = S.probs(flat, 1.0, 0, 0.9).cumsum(0)
-    assert (cdf[got[1] - 1] if got[1] else 0.0) - 2e-5 <= S.uniform(5, 1) < cdf[got[1]] + 2e-5
+    assert got[0] == S.draw(S.probs(peaked, 0.8, 50), S.uniform(5, 0), S.drawing_order(peaked, 0.8, 50))
+    assert _at_uniform(S.probs(flat, 1.0, 0, 0.9), S.drawing_order(flat, 1.0, 0, 0.9), got[1], S.uniform(5, 1))
     assert got[2] == int(tied.argmax()) and got[3] == int(peaked.argmax())
 
 
@@ -601,8 +613,8 @@ def test_sampling_under_random_settings(hip):
             law = S.probs(logits[r], temp[r], top_k[r], top_p[r], min_p[r])
             case = (vocab, r, scales[r], temp[r], top_k[r], top_p[r], min_p[r])
             assert law[got[r]] > 0, case
-            cdf, u = law.cumsum(0), S.uniform(11, r)
-            assert (cdf[got[r] - 1] if got[r] else 0.0) - 2e-5 <= u < cdf[got[r]] + 2e-5, case
+            order = S.drawing_order(logits[r], temp[r], top_k[r], top_p[r], min_p[r])
+            assert _at_uniform(law, order, got[r], S.uniform(11, r)), case
 
 
 def test_kernels_refuse_what_they_do_not_serve(hip):

@@ -205,3 +205,10 @@ def test_sampling_oracle():
     assert plain_sampling.draw(torch.tensor([0.2, 0.0, 0.8]), 0.1) == 0
     assert plain_sampling.draw(torch.tensor([0.2, 0.0, 0.8]), 0.2) == 2        # zero-mass entries are never drawn
     assert plain_sampling.draw(torch.tensor([0.2, 0.0, 0.8]), 0.999999) == 2
+    # a row with a filter is walked in the filters' order (largest first, equal ones by index); one without, as it lies
+    assert plain_sampling.drawing_order(logits, 1.0) is None and plain_sampling.drawing_order(logits, 0.0, top_k=2) is None
+    order = plain_sampling.drawing_order(torch.tensor([1.0, 3.0, 3.0, -1.0]), 0.5, min_p=0.01)
+    assert order.tolist() == [1, 2, 0, 3]
+    q = torch.tensor([0.1, 0.4, 0.4, 0.1])
+    assert [plain_sampling.draw(q, u, order) for u in (0.0, 0.39, 0.41, 0.79, 0.81, 0.95)] == [1, 1, 2, 2, 0, 3]
+    assert [plain_sampling.draw(q, u) for u in (0.0, 0.39, 0.41, 0.79, 0.81, 0.95)] == [0, 1, 1, 2, 2, 3]
