@@ -595,6 +595,55 @@ __device__ u64 top_p_cut_wide(const float* __restrict__ row, int vocab, float in
   return kept_s > 0 ? cand[kept_s - 1] : ((u64)(float_key(x_hi) + 1u) << 32);
 }
 
+// Top-k over a kept set too large to collect (a k beyond the room, or a flat row): the same halving, by count. `above`
+// tokens lie over the range and the k-th lies inside it; the range's tokens are then collected and sorted, and the
+// (k - above)-th of them is the last kept one. Sets `cut` to its order key (0 when fewer than k tokens weigh anything:
+// all are kept); false when the range cannot be narrowed.
+__device__ bool top_k_cut_wide(const float* __restrict__ row, int vocab, float inv_temp, float xmax, int k, u64* cand,
+                               int* n_cand, u64& cut) {
+  const int tid = threadIdx.x;
+  float x_hi = xmax, x_lo = xmax - 128.f;        // (what lies further below weighs nothing)
+  int above = 0;
+  {
+    int within = 0;
+    for_each_token(row, vocab, inv_temp, [&](float x, int) { within += x > x_lo; });
+    if (block_sum_int(within) <= k) { cut = 0; return true; }
+  }
+  for (int step = 0;; ++step) {
+    const float x_mid = 0.5f * (x_lo + x_hi);
+    if (step == 48 || !(x_mid > x_lo && x_mid < x_hi)) return false;
+    int up = 0, down = 0;
+    for_each_token(row, vocab, inv_temp, [&](float x, int) {
+      if (x > x_mid && x <= x_hi) ++up;
+      else if (x > x_lo && x <= x_mid) ++down;
+    });
+    up = block_sum_int(up);
+    down = block_sum_int(down);
+    int inside;
+    if (above + up >= k) { x_lo = x_mid; inside = up; }
+    else { above += up; x_hi = x_mid; inside = down; }
+    if (inside <= SAMPLE_CANDIDATES) break;
+  }
+  if (tid == 0) *n_cand = 0;
+  __syncthreads();
+  for_each_token(row, vocab, inv_temp, [&](float x, int i) {
+    if (x > x_lo && x <= x_hi) {
+      const int at = atomicAdd(n_cand, 1);
+      if (at < SAMPLE_CANDIDATES) cand[at] = order_key(x, i);
+    }
+  });
+  __syncthreads();
+  const int count = *n_cand;
+  int n_pad = WAVE;
+  while (n_pad < count) n_pad <<= 1;
+  for (int i = count + tid; i < n_pad; i += blockDim.x) cand[i] = 0;
+  __syncthreads();
+  bitonic_sort(cand, n_pad, true);
+  cut = cand[min(count, k - above) - 1];
+  __syncthreads();
+  return true;
+}
+
 __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     const float* __restrict__ logits, int32_t* __restrict__ out, int vocab, const float* __restrict__ temperature,
     const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
@@ -625,7 +674,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
   const int chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
   const bool m_on = p_min > 0.f;
   const bool filtered = k > 0 || p_on || m_on;
-  if (filtered && ((k_on && k > SAMPLE_CANDIDATES) || vocab > 255 * SAMPLE_THREADS)) {      // (uniform over the block)
+  if (filtered && vocab > 255 * SAMPLE_THREADS) {      // (uniform over the block)
     sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
     return;
   }
@@ -643,7 +692,8 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
         for_each_token(row, vocab, inv_temp, [&](float x, int) { mass += fixed_mass(__expf(x - xmax)); });
         z_all = block_sum_u64(mass);
       }
-      estimate_band_counts(row, vocab, inv_temp, xmax, counts, band_counts);
+      wide = k_on && k > SAMPLE_CANDIDATES;      // no room for the kept set whatever the bands
+      if (!wide) estimate_band_counts(row, vocab, inv_temp, xmax, counts, band_counts);
       // Which bands to collect: the fewest that should hold twice what is needed (k tokens; 256 for top-p alone). The
       // collecting counts exactly; too many, or fewer than k, and another set of bands is tried.
       const int need = k_on ? k : 1;
@@ -652,13 +702,8 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
       for (int j = SAMPLE_BANDS - 1; j >= 0; --j)
         if (counts[j] >= 2 * (k_on ? k : 256) + 64) bands = j;
       while (bands > 0 && counts[bands] > SAMPLE_CANDIDATES / 2 && counts[bands - 1] >= 2 * need) --bands;
-      for (int attempt = 0;; ++attempt) {
+      for (int attempt = 0; !wide; ++attempt) {
         if (attempt == 6 || bands < 0 || bands >= SAMPLE_BANDS) {
-          if (!k_on) cut = top_p_cut_wide(row, vocab, inv_temp, xmax, (u64)((double)p_keep * (double)z_all), cand, &n_cand);
-          if (cut == 0) {
-            sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
-            return;
-          }
           wide = true;
           break;
         }
@@ -715,6 +760,32 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
           continue;
         }
         break;
+      }
+      if (wide) {
+        // the last token top-k keeps, then the last one top-p keeps of those (what precedes a token is the same with
+        // and without top-k as long as the token is within it): the kept set ends at the earlier of the two
+        __syncthreads();
+        bool found = true;
+        u64 z_k = z_all;
+        if (k_on) {
+          found = top_k_cut_wide(row, vocab, inv_temp, xmax, k, cand, &n_cand, cut);
+          if (found && p_on) {
+            u64 mass = 0;
+            for_each_token(row, vocab, inv_temp, [&](float x, int i) {
+              if (order_key(x, i) >= cut) mass += fixed_mass(__expf(x - xmax));
+            });
+            z_k = block_sum_u64(mass);
+          }
+        }
+        if (found && p_on) {
+          const u64 p_cut = top_p_cut_wide(row, vocab, inv_temp, xmax, (u64)((double)p_keep * (double)z_k), cand, &n_cand);
+          found = p_cut != 0;
+          cut = max(cut, p_cut);
+        }
+        if (!found) {                              // thousands of equal values where a cut falls
+          sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
+          return;
+        }
       }
     } else if (m_on) {
       // min-p alone keeps the tokens within -ln(min_p) of the largest value: the bands that reach that far

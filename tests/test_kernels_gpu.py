@@ -561,7 +561,9 @@ def test_sampling_filters_at_the_full_vocabulary(hip):
              (peaked * 8, 1.0, 50, 1.0, 0.0), (peaked * 8, 1.0, 0, 0.999, 0.0), (peaked * 8, 0.5, 20, 0.9, 0.0),
              (peaked * 40, 1.0, 50, 0.9, 0.0),      # sharp rows: the 50th token lies tens, or hundreds, below the first
              (flat, 1.0, 0, 1.0, 0.2), (peaked, 1.0, 200_000, 1.0, 0.0),   # kept sets too long to collect: min-p alone, all
-             (plateau, 1.0, 0, 0.5, 0.0), (plateau, 1.0, 0, 1.0, 0.5), (plateau, 1.0, 7000, 1.0, 0.0)]   # 6,000 equal values
+             (plateau, 1.0, 0, 0.5, 0.0), (plateau, 1.0, 0, 1.0, 0.5), (plateau, 1.0, 7000, 1.0, 0.0),   # 6,000 equal values
+             (flat, 0.8, 50, 0.9, 0.0), (flat, 0.8, 20, 0.95, 0.05), (peaked, 1.0, 5000, 0.9, 0.01),    # cuts found by halving
+             (plateau, 1.0, 3000, 1.0, 0.0), (peaked * 40, 1.0, 5000, 1.0, 0.0)]   # a cut inside equal values; k beyond what weighs
     n = 48
     for at, (row, temp, top_k, top_p, min_p) in enumerate(cases):
         f = lambda x, dt: torch.full((n,), x, dtype=dt).cuda()
