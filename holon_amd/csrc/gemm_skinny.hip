@@ -1,4 +1,4 @@
-// y[M, N] = x[M, K] w[N, K]^T for few rows (decode steps): bfloat16 operands, float32 accumulation on the matrix
+// y[M, N] = x[M, K] w[N, K]^T for up to 16 rows (decode steps): bfloat16 operands, float32 accumulation on the matrix
 // cores, memory-bound on the weights. A workgroup owns 16 weight rows; its waves split K evenly and add their partial
 // tiles through LDS in wave order, so the result does not depend on M or on anything but the shapes.
 //
@@ -86,12 +86,12 @@ __device__ __forceinline__ float over_lane_groups(float v, int c) {
 
 // RESID: y is the residual stream, y = round(y + round(product)) in place: the add that the next norm's kernel would
 // have done, with its roundings.
-template <int MT, int WPB, int UNROLL, typename OutT, bool TILED, bool RESID = false>
+template <int WPB, int UNROLL, typename OutT, bool TILED, bool RESID = false>
 __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                 const bf16_t* __restrict__ w, OutT* __restrict__ y,
                                                                 int M, int N, int K, int round_first, RowScale rs,
                                                                 float* __restrict__ stats_out) {
-  __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * MT * WAVE : 1];
+  __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * WAVE : 1];
   __shared__ f32x4_t red_ss[WPB > 1 ? (WPB - 1) * WAVE : 1];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
@@ -102,85 +102,63 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
                            : w + (int64_t)(n0 + c) * K + (int64_t)wave * kw + 8 * g;
   constexpr int WSTEP = TILED ? 512 : 32;       // elements between one product's weights and the next
   const bf16_t* xp = x + (int64_t)c * K + (int64_t)wave * kw + 8 * g;
-  f32x4_t acc[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  bool have[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t) have[t] = t * 16 + c < M;
+  const bool have = c < M;                      // token c of the step exists
+  f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
   RowSums<WPB> sums;
   sums.start(rs, wave, lane);
-  ushort4 before[MT];                            // RESID: the residual values this lane will add to, asked for now so
-  if constexpr (RESID) {                         // that they are here when the sums are
-#pragma unroll
-    for (int t = 0; t < MT; ++t)
-      if (wave == 0 && have[t]) before[t] = *reinterpret_cast<const ushort4*>(y + (int64_t)(t * 16 + c) * N + n0 + 4 * g);
+  ushort4 before;                               // RESID: the residual values this lane will add to, asked for now so
+  if constexpr (RESID) {                        // that they are here when the sums are
+    if (wave == 0 && have) before = *reinterpret_cast<const ushort4*>(y + (int64_t)c * N + n0 + 4 * g);
   }
+  auto tokens = [&](int s) -> bf16x8_t {        // the activations of product s: zeros for a token that is not there
+    bf16x8_t xf;
+    if (have) {
+      xf = *reinterpret_cast<const bf16x8_t*>(xp + s * 32);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xf[i] = (__bf16)0.f;
+    }
+    return xf;
+  };
 
   int s = 0;
   for (; s + UNROLL <= steps; s += UNROLL) {
-    if (MT == 1) sums.turn();
-    bf16x8_t wf[UNROLL], xf[UNROLL][MT];
+    sums.turn();
+    bf16x8_t wf[UNROLL], xf[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
       wf[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp + (int64_t)(s + u) * WSTEP));
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
+    for (int u = 0; u < UNROLL; ++u) xf[u] = tokens(s + u);
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        if (have[t]) {
-          xf[u][t] = *reinterpret_cast<const bf16x8_t*>(xp + (int64_t)t * 16 * K + (s + u) * 32);
-        } else {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) xf[u][t][i] = (__bf16)0.f;
-        }
-      }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
-#pragma unroll
-      for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u][t], acc[t], 0, 0, 0);
+    for (int u = 0; u < UNROLL; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u], acc, 0, 0, 0);
   }
   for (; s < steps; ++s) {
     const bf16x8_t wf = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp + (int64_t)s * WSTEP));
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      bf16x8_t xf;
-      if (have[t]) {
-        xf = *reinterpret_cast<const bf16x8_t*>(xp + (int64_t)t * 16 * K + s * 32);
-      } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) xf[i] = (__bf16)0.f;
-      }
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc[t], 0, 0, 0);
-    }
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, tokens(s), acc, 0, 0, 0);
   }
-  f32x4_t ss = MT == 1 ? sums.finish() : f32x4_t{0.f, 0.f, 0.f, 0.f};
+  f32x4_t ss = sums.finish();
   if (WPB > 1) {
     if (wave > 0) {
-#pragma unroll
-      for (int t = 0; t < MT; ++t) red[((wave - 1) * MT + t) * WAVE + lane] = acc[t];
+      red[(wave - 1) * WAVE + lane] = acc;
       red_ss[(wave - 1) * WAVE + lane] = ss;
     }
     __syncthreads();
     if (wave > 0) return;
     for (int ww = 1; ww < WPB; ++ww) {
-#pragma unroll
-      for (int t = 0; t < MT; ++t) acc[t] += red[((ww - 1) * MT + t) * WAVE + lane];
+      acc += red[(ww - 1) * WAVE + lane];
       ss += red_ss[(ww - 1) * WAVE + lane];
     }
   }
-  if (MT == 1 && rs.stats != nullptr) {          // the norm's scale of row c, on the float32 sums before they are rounded
+  if (rs.stats != nullptr) {                     // the norm's scale of row c, on the float32 sums before they are rounded
     const float inv = 1.0f / sqrtf(row_sum_of_column(ss, c) * rs.inv_dim + rs.eps);
-    acc[0] *= inv;
+    acc *= inv;
   }
   float mine = 0.f;                              // RESID with stats_out: the squares of the residual values written
-#pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int m = t * 16 + c;
-    if (m >= M) continue;
-    OutT* yp = y + (int64_t)m * N + n0 + 4 * g;
+  if (have) {
+    OutT* yp = y + (int64_t)c * N + n0 + 4 * g;
     if constexpr (sizeof(OutT) == 4) {
-      f32x4_t o = acc[t];
+      f32x4_t o = acc;
       if (round_first) {        // the bfloat16 product, widened: what the vendor product of more rows gives, cast up
 #pragma unroll
         for (int r = 0; r < 4; ++r) o[r] = bf16_to_float(float_to_bf16(o[r]));
@@ -188,10 +166,10 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
       *reinterpret_cast<f32x4_t*>(yp) = o;
     } else {
       ushort4 o;
-      o.x = float_to_bf16(acc[t][0]); o.y = float_to_bf16(acc[t][1]);
-      o.z = float_to_bf16(acc[t][2]); o.w = float_to_bf16(acc[t][3]);
+      o.x = float_to_bf16(acc[0]); o.y = float_to_bf16(acc[1]);
+      o.z = float_to_bf16(acc[2]); o.w = float_to_bf16(acc[3]);
       if constexpr (RESID) {
-        const ushort4 r = before[t];
+        const ushort4 r = before;
         o.x = float_to_bf16(bf16_to_float(r.x) + bf16_to_float(o.x));
         o.y = float_to_bf16(bf16_to_float(r.y) + bf16_to_float(o.y));
         o.z = float_to_bf16(bf16_to_float(r.z) + bf16_to_float(o.z));
@@ -202,7 +180,7 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
       *reinterpret_cast<ushort4*>(yp) = o;
     }
   }
-  if constexpr (RESID && MT == 1) {
+  if constexpr (RESID) {
     if (stats_out != nullptr) {                  // this block's 16 columns of every row: one partial per row
       const float part = over_lane_groups(mine, c);
       if (g == 0) stats_out[(int64_t)blockIdx.x * 16 + c] = part;
@@ -210,104 +188,93 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
   }
 }
 
-template <int MT, int WPB, int UNROLL, typename OutT, bool RESID>
+template <int WPB, int UNROLL, typename OutT, bool RESID>
 static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s,
                           int round_first, RowScale rs, float* stats_out) {
   const dim3 grid(N / 16), block(WPB * 64);
   if constexpr (RESID)
-    gemm_skinny_kernel<MT, WPB, UNROLL, OutT, true, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                                (OutT*)y, M, N, K, round_first, rs, stats_out);
+    gemm_skinny_kernel<WPB, UNROLL, OutT, true, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
+                                                                            (OutT*)y, M, N, K, round_first, rs, stats_out);
   else if (tiled)
-    gemm_skinny_kernel<MT, WPB, UNROLL, OutT, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                          (OutT*)y, M, N, K, round_first, rs, stats_out);
+    gemm_skinny_kernel<WPB, UNROLL, OutT, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
+                                                                      (OutT*)y, M, N, K, round_first, rs, stats_out);
   else
-    gemm_skinny_kernel<MT, WPB, UNROLL, OutT, false><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                           (OutT*)y, M, N, K, round_first, rs, stats_out);
+    gemm_skinny_kernel<WPB, UNROLL, OutT, false><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
+                                                                       (OutT*)y, M, N, K, round_first, rs, stats_out);
 }
 
 // How many waves share a tile, from the shapes alone (so a result never depends on M): wide outputs have tiles
 // enough to fill the GPU with eight waves each; narrow ones split K 16 ways. Measured on MI355X.
-template <int MT, typename OutT, bool RESID = false>
+template <typename OutT, bool RESID = false>
 static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s,
                       int round_first = 0, RowScale rs = RowScale{nullptr, 0, 0.f, 0.f}, float* stats_out = nullptr) {
   const int tiles = N / 16;
-  int wpb = MT >= 3 ? 8 : 16;                  // 16 waves of 3 or 4 token tiles run out of registers
-  if (tiles >= 320) wpb = 8;                   // (384 tiles, K 4096: 12.7 us against 14.2; 9,496 tiles: 189 against 201 for 4)
+  int wpb = tiles >= 320 ? 8 : 16;             // (384 tiles, K 4096: 12.7 us against 14.2; 9,496 tiles: 189 against 201 for 4)
   while (wpb > 1 && K % (32 * wpb) != 0) wpb /= 2;
-  constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
   switch (wpb) {
-    case 16:
-      if constexpr (MT < 3) launch_skinny<MT, 16, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out);
-      break;
-    case 8: launch_skinny<MT, 8, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
-    case 4:
-      if constexpr (MT == 1) launch_skinny<MT, 4, 16, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out);
-      else launch_skinny<MT, 4, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out);
-      break;
-    case 2: launch_skinny<MT, 2, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
-    default: launch_skinny<MT, 1, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
+    case 16: launch_skinny<16, 8, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
+    case 8: launch_skinny<8, 8, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
+    case 4: launch_skinny<4, 16, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
+    case 2: launch_skinny<2, 8, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
+    default: launch_skinny<1, 8, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
   }
   return 0;
 }
 
 extern "C" int holon_gemm_skinny_supported(int M, int N, int K) {
-  return M >= 1 && M <= 64 && N % 16 == 0 && K % 32 == 0 && K >= 32;
+  return M >= 1 && M <= 16 && N % 16 == 0 && K % 32 == 0 && K >= 32;
 }
 
 // out_f32: 0 writes bfloat16, 1 float32 straight from the accumulators, 2 float32 values that were rounded to bfloat16
 // first (the product in the operands' type, cast up). tiled: 1 when `w` is in the tile layout (see holon_tile_weight_bf16).
 extern "C" int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_f32,
                                       int tiled, void* stream) {
-  HOLON_CHECK(holon_gemm_skinny_supported(M, N, K), "gemm (few rows): M=%d N=%d K=%d not served (M <= 64, N %% 16, K %% 32)",
+  HOLON_CHECK(holon_gemm_skinny_supported(M, N, K), "gemm (few rows): M=%d N=%d K=%d not served (M <= 16, N %% 16, K %% 32)",
               M, N, K);
   hipStream_t s = (hipStream_t)stream;
-  const int mt = (M + 15) / 16;
-#define SKINNY(MT)                                                                 \
-  if (out_f32) pick_waves<MT, float>(x, w, y, M, N, K, tiled != 0, s, out_f32 == 2); \
-  else pick_waves<MT, bf16_t>(x, w, y, M, N, K, tiled != 0, s)
-  if (mt == 1) { SKINNY(1); } else if (mt == 2) { SKINNY(2); } else if (mt == 3) { SKINNY(3); } else { SKINNY(4); }
-#undef SKINNY
+  if (out_f32) pick_waves<float>(x, w, y, M, N, K, tiled != 0, s, out_f32 == 2);
+  else pick_waves<bf16_t>(x, w, y, M, N, K, tiled != 0, s);
   HOLON_LAUNCH_OK();
   return 0;
 }
 
 // The same product over rows that a folded norm has yet to scale: `w_tiled` holds W * diag(g), x the un-normed rows,
 // `stats` [parts, 16] the partial sums of squares of x's rows; row m of the result is scaled by
-// rsqrt(sum(stats[:, m]) / K + eps) before it is rounded. M <= 16.
+// rsqrt(sum(stats[:, m]) / K + eps) before it is rounded.
 extern "C" int holon_gemm_skinny_scaled_bf16(const void* x, const void* w_tiled, void* y, int M, int N, int K,
                                              int out_f32, const float* stats, int parts, float eps, void* stream) {
-  HOLON_CHECK(M >= 1 && M <= 16 && holon_gemm_skinny_supported(M, N, K) && stats != nullptr && parts >= 1,
+  HOLON_CHECK(holon_gemm_skinny_supported(M, N, K) && stats != nullptr && parts >= 1,
               "gemm (few rows, folded norm): M=%d N=%d K=%d parts=%d not served (M <= 16, N %% 16, K %% 32)", M, N, K, parts);
   const RowScale rs{stats, parts, eps, 1.0f / (float)K};
   hipStream_t s = (hipStream_t)stream;
-  if (out_f32) pick_waves<1, float>(x, w_tiled, y, M, N, K, true, s, out_f32 == 2, rs);
-  else pick_waves<1, bf16_t>(x, w_tiled, y, M, N, K, true, s, 0, rs);
+  if (out_f32) pick_waves<float>(x, w_tiled, y, M, N, K, true, s, out_f32 == 2, rs);
+  else pick_waves<bf16_t>(x, w_tiled, y, M, N, K, true, s, 0, rs);
   HOLON_LAUNCH_OK();
   return 0;
 }
 
-// residual[M, N] += x[M, K] w^T in place (the product rounded, then the sum rounded), for one tile of rows (M <= 16)
-// over tiled weights: the output projection's product and the residual add that follows it, in one kernel. With
-// `stats_out` ([N / 16, 16] float32) it also leaves, per block of 16 columns, the sums of squares of the residual
-// values it wrote: what a norm over the new rows needs.
+// residual[M, N] += x[M, K] w^T in place (the product rounded, then the sum rounded) over tiled weights: the output
+// projection's product and the residual add that follows it, in one kernel. With `stats_out` ([N / 16, 16] float32)
+// it also leaves, per block of 16 columns, the sums of squares of the residual values it wrote: what a norm over the
+// new rows needs.
 extern "C" int holon_gemm_skinny_add_bf16(const void* x, const void* w_tiled, void* residual, int M, int N, int K,
                                           float* stats_out, void* stream) {
-  HOLON_CHECK(M >= 1 && M <= 16 && holon_gemm_skinny_supported(M, N, K),
+  HOLON_CHECK(holon_gemm_skinny_supported(M, N, K),
               "gemm (few rows, added to the residual): M=%d N=%d K=%d not served (M <= 16, N %% 16, K %% 32)", M, N, K);
-  pick_waves<1, bf16_t, true>(x, w_tiled, residual, M, N, K, true, (hipStream_t)stream, 0,
-                              RowScale{nullptr, 0, 0.f, 0.f}, stats_out);
+  pick_waves<bf16_t, true>(x, w_tiled, residual, M, N, K, true, (hipStream_t)stream, 0,
+                           RowScale{nullptr, 0, 0.f, 0.f}, stats_out);
   HOLON_LAUNCH_OK();
   return 0;
 }
 
 // The gated form: w = [gate rows; up rows] (2I rows), y[M, I] = round(silu(round(x gate^T))) * round(x up^T), the
 // roundings of the two-kernel composition. A block owns gate tile t and up tile t + I/16 and streams both.
-template <int MT, int WPB, int UNROLL, bool TILED>
+template <int WPB, int UNROLL, bool TILED>
 __global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t* __restrict__ x,
                                                                     const bf16_t* __restrict__ w,
                                                                     bf16_t* __restrict__ y, int M, int I, int K,
                                                                     RowScale rs) {
-  __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * 2 * MT * WAVE : 1];
+  __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * 2 * WAVE : 1];
   __shared__ f32x4_t red_ss[WPB > 1 ? (WPB - 1) * WAVE : 1];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
@@ -322,118 +289,93 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_glu_kernel(const bf16_t*
   }
   constexpr int WSTEP = TILED ? 512 : 32;
   const bf16_t* xp = x + (int64_t)c * K + (int64_t)wave * kw + 8 * g;
-  f32x4_t acc[2][MT];
-  bool have[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    acc[0][t] = acc[1][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    have[t] = t * 16 + c < M;
-  }
+  const bool have = c < M;
+  f32x4_t acc[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
   RowSums<WPB> sums;
   sums.start(rs, wave, lane);
+  auto tokens = [&](int s) -> bf16x8_t {
+    bf16x8_t xf;
+    if (have) {
+      xf = *reinterpret_cast<const bf16x8_t*>(xp + s * 32);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xf[i] = (__bf16)0.f;
+    }
+    return xf;
+  };
   int s = 0;
   for (; s + UNROLL <= steps; s += UNROLL) {
-    if (MT == 1) sums.turn();
-    bf16x8_t wf[2][UNROLL], xf[UNROLL][MT];
+    sums.turn();
+    bf16x8_t wf[2][UNROLL], xf[UNROLL];
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u)
         wf[h][u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp[h] + (int64_t)(s + u) * WSTEP));
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
+    for (int u = 0; u < UNROLL; ++u) xf[u] = tokens(s + u);
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        if (have[t]) {
-          xf[u][t] = *reinterpret_cast<const bf16x8_t*>(xp + (int64_t)t * 16 * K + (s + u) * 32);
-        } else {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) xf[u][t][i] = (__bf16)0.f;
-        }
-      }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
-#pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[0][u], xf[u][t], acc[0][t], 0, 0, 0);
-        acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[1][u], xf[u][t], acc[1][t], 0, 0, 0);
-      }
+    for (int u = 0; u < UNROLL; ++u) {
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[0][u], xf[u], acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[1][u], xf[u], acc[1], 0, 0, 0);
+    }
   }
   for (; s < steps; ++s) {
     const bf16x8_t w0 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp[0] + (int64_t)s * WSTEP));
     const bf16x8_t w1 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp[1] + (int64_t)s * WSTEP));
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      bf16x8_t xf;
-      if (have[t]) {
-        xf = *reinterpret_cast<const bf16x8_t*>(xp + (int64_t)t * 16 * K + s * 32);
-      } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) xf[i] = (__bf16)0.f;
-      }
-      acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, xf, acc[0][t], 0, 0, 0);
-      acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, xf, acc[1][t], 0, 0, 0);
-    }
+    const bf16x8_t xf = tokens(s);
+    acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, xf, acc[0], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, xf, acc[1], 0, 0, 0);
   }
-  f32x4_t ss = MT == 1 ? sums.finish() : f32x4_t{0.f, 0.f, 0.f, 0.f};
+  f32x4_t ss = sums.finish();
   if (WPB > 1) {
     if (wave > 0) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int t = 0; t < MT; ++t) red[(((wave - 1) * 2 + h) * MT + t) * WAVE + lane] = acc[h][t];
+      for (int h = 0; h < 2; ++h) red[((wave - 1) * 2 + h) * WAVE + lane] = acc[h];
       red_ss[(wave - 1) * WAVE + lane] = ss;
     }
     __syncthreads();
     if (wave > 0) return;
     for (int ww = 1; ww < WPB; ++ww) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int t = 0; t < MT; ++t) acc[h][t] += red[(((ww - 1) * 2 + h) * MT + t) * WAVE + lane];
+      for (int h = 0; h < 2; ++h) acc[h] += red[((ww - 1) * 2 + h) * WAVE + lane];
       ss += red_ss[(ww - 1) * WAVE + lane];
     }
   }
-  if (MT == 1 && rs.stats != nullptr) {
+  if (rs.stats != nullptr) {
     const float inv = 1.0f / sqrtf(row_sum_of_column(ss, c) * rs.inv_dim + rs.eps);
-    acc[0][0] *= inv;
-    acc[1][0] *= inv;
+    acc[0] *= inv;
+    acc[1] *= inv;
   }
+  if (!have) return;
+  ushort4 o;
+  bf16_t* oe = reinterpret_cast<bf16_t*>(&o);
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int m = t * 16 + c;
-    if (m >= M) continue;
-    ushort4 o;
-    bf16_t* oe = reinterpret_cast<bf16_t*>(&o);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float gate = bf16_to_float(float_to_bf16(acc[0][t][r]));
-      const float up = bf16_to_float(float_to_bf16(acc[1][t][r]));
-      const float sg = bf16_to_float(float_to_bf16(silu<bf16_t>(gate)));
-      oe[r] = float_to_bf16(sg * up);
-    }
-    *reinterpret_cast<ushort4*>(y + (int64_t)m * I + n0 + 4 * g) = o;
+  for (int r = 0; r < 4; ++r) {
+    const float gate = bf16_to_float(float_to_bf16(acc[0][r]));
+    const float up = bf16_to_float(float_to_bf16(acc[1][r]));
+    const float sg = bf16_to_float(float_to_bf16(silu<bf16_t>(gate)));
+    oe[r] = float_to_bf16(sg * up);
   }
+  *reinterpret_cast<ushort4*>(y + (int64_t)c * I + n0 + 4 * g) = o;
 }
 
 // `stats` (nullable, with `parts` and `eps`): x holds un-normed rows and `w` the tiled weights with the norm's weight
-// folded in; rows are scaled as in holon_gemm_skinny_scaled_bf16 (M <= 16, tiled).
+// folded in; rows are scaled as in holon_gemm_skinny_scaled_bf16 (tiled).
 extern "C" int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int I, int K, int tiled,
                                           const float* stats, int parts, float eps, void* stream) {
-  HOLON_CHECK(M >= 1 && M <= 32 && I % 16 == 0 && K % 128 == 0, "gated gemm (few rows): M=%d I=%d K=%d not served", M, I, K);
-  HOLON_CHECK(stats == nullptr || (M <= 16 && tiled && parts >= 1), "gated gemm (few rows, folded norm): M=%d tiled=%d parts=%d",
-              M, tiled, parts);
+  HOLON_CHECK(M >= 1 && M <= 16 && I % 16 == 0 && K % 128 == 0, "gated gemm (few rows): M=%d I=%d K=%d not served", M, I, K);
+  HOLON_CHECK(stats == nullptr || (tiled && parts >= 1), "gated gemm (few rows, folded norm): tiled=%d parts=%d", tiled, parts);
   const RowScale rs{stats, parts, eps, 1.0f / (float)K};
   hipStream_t s = (hipStream_t)stream;
   const bool few = I / 16 < 512;   // few tile pairs: four waves share each; otherwise two (measured at 768 pairs, K 4096:
                                    // 33 us against 36 for one wave a pair at 1 and 8 rows, the same at 16)
-#define GLU(MT, WPB, U)                                                                                              \
-  if (tiled) gemm_skinny_glu_kernel<MT, WPB, U, true><<<I / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, \
-                                                                                 (bf16_t*)y, M, I, K, rs);           \
-  else gemm_skinny_glu_kernel<MT, WPB, U, false><<<I / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,      \
-                                                                            (bf16_t*)y, M, I, K, rs)
-  if (M <= 16) { if (few) { GLU(1, 4, 8); } else { GLU(1, 2, 8); } }
-  else { if (few) { GLU(2, 4, 4); } else { GLU(2, 1, 4); } }
+#define GLU(WPB, U)                                                                                              \
+  if (tiled) gemm_skinny_glu_kernel<WPB, U, true><<<I / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, \
+                                                                             (bf16_t*)y, M, I, K, rs);           \
+  else gemm_skinny_glu_kernel<WPB, U, false><<<I / 16, WPB * 64, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,      \
+                                                                        (bf16_t*)y, M, I, K, rs)
+  if (few) { GLU(4, 8); } else { GLU(2, 8); }
 #undef GLU
   HOLON_LAUNCH_OK();
   return 0;

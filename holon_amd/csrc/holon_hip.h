@@ -65,24 +65,24 @@ int holon_attention_decode_bf16_static(const void* q, void* out, const void* pag
                                        const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
                                        int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
                                        int splits, int keys_per_split, void* stream);
-// y[M, N] = x[M, K] w[N, K]^T for M <= 64 rows, bfloat16 in, float32 accumulation; out_f32: 0 bfloat16 out, 1 float32
+// y[M, N] = x[M, K] w[N, K]^T for M <= 16 rows, bfloat16 in, float32 accumulation; out_f32: 0 bfloat16 out, 1 float32
 // out, 2 float32 out of values rounded to bfloat16 first;
 // tiled says that `w` is holon_tile_weight_bf16's copy ([N/16, K/32, 64, 8]: lane-major 16-byte pieces).
 int holon_gemm_skinny_supported(int M, int N, int K);
 int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_f32, int tiled,
                            void* stream);
-// residual[M, N] = round(residual + round(x w^T)) in place, M <= 16, tiled weights: the product and the residual add
-// that follows it in one kernel.
+// residual[M, N] = round(residual + round(x w^T)) in place, tiled weights: the product and the residual add that
+// follows it in one kernel.
 // With stats_out ([N / 16, 16] float32): per block of 16 columns, the sums of squares of the residual values written.
 int holon_gemm_skinny_add_bf16(const void* x, const void* w_tiled, void* residual, int M, int N, int K, float* stats_out,
                                void* stream);
 // A norm folded into the product: w_tiled holds W * diag(g) (holon_tile_weight_bf16 with `scale`), x the un-normed rows,
 // stats [parts, 16] partial sums of squares of x's rows (row m in column m); row m of the result is scaled by
-// rsqrt(sum(stats[:, m]) / K + eps) before rounding. M <= 16.
+// rsqrt(sum(stats[:, m]) / K + eps) before rounding.
 int holon_gemm_skinny_scaled_bf16(const void* x, const void* w_tiled, void* y, int M, int N, int K, int out_f32,
                                   const float* stats, int parts, float eps, void* stream);
-// y[M, I] = round(silu(round(x gate^T))) * round(x up^T) with w = [gate; up] ([2I, K]), M <= 32.
-// stats (nullable): as in holon_gemm_skinny_scaled_bf16 (M <= 16, tiled weights with the norm's weight folded in).
+// y[M, I] = round(silu(round(x gate^T))) * round(x up^T) with w = [gate; up] ([2I, K]), M <= 16.
+// stats (nullable): as in holon_gemm_skinny_scaled_bf16 (tiled weights with the norm's weight folded in).
 int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int I, int K, int tiled, const float* stats,
                                int parts, float eps, void* stream);
 // y[M, N] = x[M, K] w[N, K]^T, all float32, true 32-bit products and sums in an order that depends on K alone: a row's

@@ -159,7 +159,7 @@ class HipKernels:
                    x.numel() // dim, dim, float(eps), self._dt(x, "add_rmsnorm"), self._stream())
         return y
 
-    skinny_rows = 16          # up to this many rows the hand-written weight-streaming product runs
+    skinny_rows = 16          # up to this many rows (one tile of tokens) the hand-written weight-streaming product runs
 
     def tile_weight(self, weight, scale=None):
         """A copy of `weight` [N, K] in the layout the few-row product streams fastest, or None when its shape or
@@ -181,7 +181,7 @@ class HipKernels:
     def _row_scale(self, x, tiled, row_scale, what):
         """Checks of a product over un-normed rows with the norm folded into `tiled`; returns (stats, parts, eps)."""
         stats, eps = row_scale
-        if tiled is None or x.shape[0] > min(self.skinny_rows, 16) or x.dtype != torch.bfloat16:
+        if tiled is None or x.shape[0] > self.skinny_rows or x.dtype != torch.bfloat16:
             raise KernelError(f"{what}: a folded norm needs tiled weights and at most 16 bfloat16 rows")
         self._check(stats, f"{what} stats", torch.float32)
         if stats.dim() != 2 or stats.shape[1] != 16:
@@ -191,7 +191,7 @@ class HipKernels:
     def folds_norm(self, rows, weight, tiled):
         """Whether `linear(x, ..., row_scale=...)` serves `rows` rows over this weight."""
         n, k = weight.shape
-        return bool(tiled is not None and weight.dtype == torch.bfloat16 and 1 <= rows <= min(self.skinny_rows, 16)
+        return bool(tiled is not None and weight.dtype == torch.bfloat16 and 1 <= rows <= self.skinny_rows
                     and k >= 256 and self.lib.holon_gemm_skinny_supported(rows, n, k))
 
     def linear(self, x, weight, out_dtype=None, tiled=None, row_scale=None):
@@ -231,7 +231,7 @@ class HipKernels:
         the residual rows as they now are."""
         (m, k), n = x.shape, weight.shape[0]
         if not (tiled is not None and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                and residual.dtype == torch.bfloat16 and 1 <= m <= min(self.skinny_rows, 16) and weight.shape[1] == k
+                and residual.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows and weight.shape[1] == k
                 and k >= 256 and x.is_contiguous() and residual.is_contiguous()
                 and self.lib.holon_gemm_skinny_supported(m, n, k)):
             return False
@@ -247,7 +247,7 @@ class HipKernels:
         after the other (the sums over K may be split differently); None when this shape is not fused (the caller then composes the two)."""
         m, k = x.shape
         two_i = weight.shape[0]
-        if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= min(self.skinny_rows, 32)
+        if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows
                 and two_i % 32 == 0 and k % 128 == 0 and k >= 256 and weight.shape[1] == k and x.is_contiguous()):
             return None
         y = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
