@@ -86,29 +86,39 @@ __device__ __forceinline__ float over_lane_groups(float v, int c) {
 
 // RESID: y is the residual stream, y = round(y + round(product)) in place: the add that the next norm's kernel would
 // have done, with its roundings.
-template <int WPB, int UNROLL, typename OutT, bool TILED, bool RESID = false>
+// NT: tiles of 16 weight rows a block owns, next to one another; its waves run them side by side over one copy of the
+// activations, which halves what the activations cost where every block reads all of them. A tile's sums are the same
+// whatever NT is.
+template <int NT, int WPB, int UNROLL, typename OutT, bool TILED, bool RESID = false>
 __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                 const bf16_t* __restrict__ w, OutT* __restrict__ y,
                                                                 int M, int N, int K, int round_first, RowScale rs,
                                                                 float* __restrict__ stats_out) {
-  __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * WAVE : 1];
+  __shared__ f32x4_t red[WPB > 1 ? (WPB - 1) * NT * WAVE : 1];
   __shared__ f32x4_t red_ss[WPB > 1 ? (WPB - 1) * WAVE : 1];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
-  const int n0 = blockIdx.x * 16;
+  const int tile0 = blockIdx.x * NT;
   const int kw = K / WPB;                       // this wave's slice of K (a multiple of 32)
   const int steps = kw / 32;
-  const bf16_t* wp = TILED ? w + ((int64_t)blockIdx.x * (K / 32) + (int64_t)wave * steps) * 512 + lane * 8
-                           : w + (int64_t)(n0 + c) * K + (int64_t)wave * kw + 8 * g;
+  const bf16_t* wp[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+    wp[j] = TILED ? w + ((int64_t)(tile0 + j) * (K / 32) + (int64_t)wave * steps) * 512 + lane * 8
+                  : w + (int64_t)((tile0 + j) * 16 + c) * K + (int64_t)wave * kw + 8 * g;
   constexpr int WSTEP = TILED ? 512 : 32;       // elements between one product's weights and the next
   const bf16_t* xp = x + (int64_t)c * K + (int64_t)wave * kw + 8 * g;
   const bool have = c < M;                      // token c of the step exists
-  f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  f32x4_t acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   RowSums<WPB> sums;
   sums.start(rs, wave, lane);
-  ushort4 before;                               // RESID: the residual values this lane will add to, asked for now so
+  ushort4 before[NT];                           // RESID: the residual values this lane will add to, asked for now so
   if constexpr (RESID) {                        // that they are here when the sums are
-    if (wave == 0 && have) before = *reinterpret_cast<const ushort4*>(y + (int64_t)c * N + n0 + 4 * g);
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      if (wave == 0 && have) before[j] = *reinterpret_cast<const ushort4*>(y + (int64_t)c * N + (tile0 + j) * 16 + 4 * g);
   }
   auto tokens = [&](int s) -> bf16x8_t {        // the activations of product s: zeros for a token that is not there
     bf16x8_t xf;
@@ -124,100 +134,125 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
   int s = 0;
   for (; s + UNROLL <= steps; s += UNROLL) {
     sums.turn();
-    bf16x8_t wf[UNROLL], xf[UNROLL];
+    bf16x8_t wf[NT][UNROLL], xf[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
-      wf[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp + (int64_t)(s + u) * WSTEP));
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u)
+        wf[j][u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp[j] + (int64_t)(s + u) * WSTEP));
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) xf[u] = tokens(s + u);
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u], acc, 0, 0, 0);
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j][u], xf[u], acc[j], 0, 0, 0);
   }
   for (; s < steps; ++s) {
-    const bf16x8_t wf = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp + (int64_t)s * WSTEP));
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, tokens(s), acc, 0, 0, 0);
+    const bf16x8_t xf = tokens(s);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const bf16x8_t wf = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp[j] + (int64_t)s * WSTEP));
+      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc[j], 0, 0, 0);
+    }
   }
   f32x4_t ss = sums.finish();
   if (WPB > 1) {
     if (wave > 0) {
-      red[(wave - 1) * WAVE + lane] = acc;
+#pragma unroll
+      for (int j = 0; j < NT; ++j) red[((wave - 1) * NT + j) * WAVE + lane] = acc[j];
       red_ss[(wave - 1) * WAVE + lane] = ss;
     }
     __syncthreads();
     if (wave > 0) return;
     for (int ww = 1; ww < WPB; ++ww) {
-      acc += red[(ww - 1) * WAVE + lane];
+#pragma unroll
+      for (int j = 0; j < NT; ++j) acc[j] += red[((ww - 1) * NT + j) * WAVE + lane];
       ss += red_ss[(ww - 1) * WAVE + lane];
     }
   }
   if (rs.stats != nullptr) {                     // the norm's scale of row c, on the float32 sums before they are rounded
     const float inv = 1.0f / sqrtf(row_sum_of_column(ss, c) * rs.inv_dim + rs.eps);
-    acc *= inv;
-  }
-  float mine = 0.f;                              // RESID with stats_out: the squares of the residual values written
-  if (have) {
-    OutT* yp = y + (int64_t)c * N + n0 + 4 * g;
-    if constexpr (sizeof(OutT) == 4) {
-      f32x4_t o = acc;
-      if (round_first) {        // the bfloat16 product, widened: what the vendor product of more rows gives, cast up
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = bf16_to_float(float_to_bf16(o[r]));
-      }
-      *reinterpret_cast<f32x4_t*>(yp) = o;
-    } else {
-      ushort4 o;
-      o.x = float_to_bf16(acc[0]); o.y = float_to_bf16(acc[1]);
-      o.z = float_to_bf16(acc[2]); o.w = float_to_bf16(acc[3]);
-      if constexpr (RESID) {
-        const ushort4 r = before;
-        o.x = float_to_bf16(bf16_to_float(r.x) + bf16_to_float(o.x));
-        o.y = float_to_bf16(bf16_to_float(r.y) + bf16_to_float(o.y));
-        o.z = float_to_bf16(bf16_to_float(r.z) + bf16_to_float(o.z));
-        o.w = float_to_bf16(bf16_to_float(r.w) + bf16_to_float(o.w));
-        const float v0 = bf16_to_float(o.x), v1 = bf16_to_float(o.y), v2 = bf16_to_float(o.z), v3 = bf16_to_float(o.w);
-        mine = ((v0 * v0 + v1 * v1) + v2 * v2) + v3 * v3;
-      }
-      *reinterpret_cast<ushort4*>(yp) = o;
-    }
+    for (int j = 0; j < NT; ++j) acc[j] *= inv;
   }
-  if constexpr (RESID) {
-    if (stats_out != nullptr) {                  // this block's 16 columns of every row: one partial per row
-      const float part = over_lane_groups(mine, c);
-      if (g == 0) stats_out[(int64_t)blockIdx.x * 16 + c] = part;
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    float mine = 0.f;                            // RESID with stats_out: the squares of the residual values written
+    if (have) {
+      OutT* yp = y + (int64_t)c * N + (tile0 + j) * 16 + 4 * g;
+      if constexpr (sizeof(OutT) == 4) {
+        f32x4_t o = acc[j];
+        if (round_first) {      // the bfloat16 product, widened: what the vendor product of more rows gives, cast up
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[r] = bf16_to_float(float_to_bf16(o[r]));
+        }
+        *reinterpret_cast<f32x4_t*>(yp) = o;
+      } else {
+        ushort4 o;
+        o.x = float_to_bf16(acc[j][0]); o.y = float_to_bf16(acc[j][1]);
+        o.z = float_to_bf16(acc[j][2]); o.w = float_to_bf16(acc[j][3]);
+        if constexpr (RESID) {
+          const ushort4 r = before[j];
+          o.x = float_to_bf16(bf16_to_float(r.x) + bf16_to_float(o.x));
+          o.y = float_to_bf16(bf16_to_float(r.y) + bf16_to_float(o.y));
+          o.z = float_to_bf16(bf16_to_float(r.z) + bf16_to_float(o.z));
+          o.w = float_to_bf16(bf16_to_float(r.w) + bf16_to_float(o.w));
+          const float v0 = bf16_to_float(o.x), v1 = bf16_to_float(o.y), v2 = bf16_to_float(o.z), v3 = bf16_to_float(o.w);
+          mine = ((v0 * v0 + v1 * v1) + v2 * v2) + v3 * v3;
+        }
+        *reinterpret_cast<ushort4*>(yp) = o;
+      }
+    }
+    if constexpr (RESID) {
+      if (stats_out != nullptr) {                // a tile's 16 columns of every row: one partial per row
+        const float part = over_lane_groups(mine, c);
+        if (g == 0) stats_out[(int64_t)(tile0 + j) * 16 + c] = part;
+      }
     }
   }
 }
 
-template <int WPB, int UNROLL, typename OutT, bool RESID>
+template <int NT, int WPB, int UNROLL, typename OutT, bool RESID>
 static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s,
                           int round_first, RowScale rs, float* stats_out) {
-  const dim3 grid(N / 16), block(WPB * 64);
+  const dim3 grid(N / 16 / NT), block(WPB * 64);
   if constexpr (RESID)
-    gemm_skinny_kernel<WPB, UNROLL, OutT, true, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                            (OutT*)y, M, N, K, round_first, rs, stats_out);
+    gemm_skinny_kernel<NT, WPB, UNROLL, OutT, true, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
+                                                                                (OutT*)y, M, N, K, round_first, rs, stats_out);
   else if (tiled)
-    gemm_skinny_kernel<WPB, UNROLL, OutT, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                      (OutT*)y, M, N, K, round_first, rs, stats_out);
+    gemm_skinny_kernel<NT, WPB, UNROLL, OutT, true><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
+                                                                          (OutT*)y, M, N, K, round_first, rs, stats_out);
   else
-    gemm_skinny_kernel<WPB, UNROLL, OutT, false><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
-                                                                       (OutT*)y, M, N, K, round_first, rs, stats_out);
+    gemm_skinny_kernel<NT, WPB, UNROLL, OutT, false><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w,
+                                                                           (OutT*)y, M, N, K, round_first, rs, stats_out);
 }
 
-// How many waves share a tile, from the shapes alone (so a result never depends on M): wide outputs have tiles
-// enough to fill the GPU with eight waves each; narrow ones split K 16 ways. Measured on MI355X.
+// How many waves share a tile, from the shapes alone (a result never depends on M), and how many tiles a block owns
+// (which changes no result, so it may follow M). Measured on MI355X, K 4096 to 8192, in us at 1 / 8 / 16 rows:
+//   256 tiles: 16 waves, one tile (two tiles leave half the compute units without a block);
+//   320 to 512 tiles: 8 waves; two tiles 9.9 / 10.7 / 12.2 (320), 11.5 / 12.3 / 13.8 (384), 14.0 / 14.6 / 15.8 (512)
+//     against one 10.8 / 12.8 / 16.1, 11.9 / 14.2 / 16.8, 13.8 / 15.5 / 17.9;
+//   640 tiles: 8 waves, one tile 17.2 / 20.0 / 23.1 against two 19.1 / 21.1 / 23.3;
+//   9,496 tiles: 8 waves; one tile at one row (182 against 187), two from four rows up (8 rows 195 against 210, 16 rows
+//     198 against 255).
 template <typename OutT, bool RESID = false>
 static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s,
                       int round_first = 0, RowScale rs = RowScale{nullptr, 0, 0.f, 0.f}, float* stats_out = nullptr) {
   const int tiles = N / 16;
-  int wpb = tiles >= 320 ? 8 : 16;             // (384 tiles, K 4096: 12.7 us against 14.2; 9,496 tiles: 189 against 201 for 4)
+  int wpb = tiles >= 320 ? 8 : 16;
   while (wpb > 1 && K % (32 * wpb) != 0) wpb /= 2;
+  const bool two = tiles % 2 == 0 && wpb <= 8 && ((tiles >= 320 && tiles <= 512) || (tiles > 4096 && M >= 4));
+#define SKINNY(WPB, U)                                                                                         \
+  if (two) launch_skinny<2, WPB, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out);     \
+  else launch_skinny<1, WPB, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out)
   switch (wpb) {
-    case 16: launch_skinny<16, 8, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
-    case 8: launch_skinny<8, 8, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
-    case 4: launch_skinny<4, 16, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
-    case 2: launch_skinny<2, 8, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
-    default: launch_skinny<1, 8, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
+    case 16: launch_skinny<1, 16, 8, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out); break;
+    case 8: SKINNY(8, 8); break;
+    case 4: if (two) { SKINNY(4, 8); } else { SKINNY(4, 16); } break;
+    case 2: SKINNY(2, 8); break;
+    default: SKINNY(1, 8); break;
   }
+#undef SKINNY
   return 0;
 }
 

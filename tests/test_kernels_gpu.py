@@ -326,7 +326,9 @@ def test_linear(hip, dtype):
     # up to 16 rows the few-row kernel runs (bfloat16, K >= 256), above that the vendor library's product
     for t, k, n in ((1, 4096, 6144), (8, 4096, 1000), (17, 100, 333), (64, 12288, 4096), (300, 120, 1000), (2, 96, 384),
                     (1, 4096, 4096), (16, 12288, 4096), (3, 4096, 24576), (9, 512, 208), (33, 1024, 4096),
-                    (48, 4096, 512), (5, 12288, 151936 // 8), (65, 4096, 512)):
+                    (48, 4096, 512), (5, 12288, 151936 // 8), (65, 4096, 512),
+                    (1, 8192, 5120), (12, 4096, 8192),                   # 320 and 512 tiles: two tiles a block
+                    (5, 512, 80_000), (2, 512, 80_000), (16, 256, 65_568)):   # a vocabulary's worth: two from four rows up
         x, w = _randn(t, k, dtype=dtype, seed=13), _randn(n, k, dtype=dtype, seed=14, scale=0.05)
         want = x.double() @ w.double().T
         got = hip.linear(x, w)
@@ -405,7 +407,7 @@ def test_norm_folded_into_the_product(hip):
             glu = hip.linear_silu_mul(h, w, folded, row_scale=(stats, eps))
             assert glu.shape == (m, n // 2) and H.op_budget_usage(glu, want, bf, 2 * k) <= 1, (m, k, n)
     # the residual add leaves the statistics of the rows it wrote, one part per 16 columns
-    for m, k, n in ((8, 4096, 4096), (1, 12288, 4096), (16, 512, 208)):
+    for m, k, n in ((8, 4096, 4096), (1, 12288, 4096), (16, 512, 208), (7, 8192, 5120), (16, 1024, 6144)):
         x, r = _randn(m, k, dtype=bf, seed=53), _randn(m, n, dtype=bf, seed=54)
         w = _randn(n, k, dtype=bf, seed=55, scale=0.05)
         tiled = hip.tile_weight(w)
