@@ -82,6 +82,7 @@ class HipKernels:
         for name, args in sig.items():
             fn = getattr(lib, name)
             fn.argtypes, fn.restype = args, _I
+        self._mid_choice: dict[tuple, str] = {}    # (weight shape, at most 32 rows) -> the vendor product's faster form
 
     # -- plumbing -------------------------------------------------------------------------------------------------
     def _call(self, fn, *args) -> None:
@@ -160,6 +161,7 @@ class HipKernels:
         return y
 
     skinny_rows = 16          # up to this many rows (one tile of tokens) the hand-written weight-streaming product runs
+    _mid_forms = True         # whether steps of 17 to 64 rows may choose between the vendor product's two forms
 
     def tile_weight(self, weight, scale=None):
         """A copy of `weight` [N, K] in the layout the few-row product streams fastest, or None when its shape or
@@ -223,8 +225,56 @@ class HipKernels:
             self._call(self.lib.holon_gemm_f32, x.data_ptr(), weight.data_ptr(), y.data_ptr(), m, n, k, self._stream())
             return y
         # the vendor library's product of bfloat16 operands, float32 accumulation
-        y = torch.matmul(x, weight.t())
+        y = self._vendor_product(x, weight)
         return y if out_dtype in (None, y.dtype) else y.to(out_dtype)
+
+    def _vendor_product(self, x, weight):
+        """x W^T by the vendor library, rounded once to the operands' type. For steps of 17 to 64 bfloat16 rows the
+        library's choice of kernel has holes at some shapes (a deep, narrow weight, 5120 x 25600: 145 us, where its
+        product of the same operands with a float32 result takes 83, two such products over the halves of K 73, and
+        the weights alone would stream in 42), so for such steps the forms are timed once per weight shape and row
+        bucket, outside graph capture, and the fastest is kept. All accumulate in float32 and round once."""
+        m = x.shape[0]
+        if not (16 < m <= 64 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and self._mid_forms):
+            return torch.matmul(x, weight.t())
+        key = (tuple(weight.shape), m <= 32)
+        form = self._mid_choice.get(key)
+        if form is None:
+            if torch.cuda.is_current_stream_capturing():
+                return torch.matmul(x, weight.t())
+            form = self._mid_choice[key] = self._time_mid_forms(x, weight)
+        return self._MID_FORMS[form](x, weight)
+
+    @staticmethod
+    def _two_halves(x, weight):
+        half = weight.shape[1] // 2
+        low = torch.mm(x[:, :half], weight[:, :half].t(), out_dtype=torch.float32)
+        return low.add_(torch.mm(x[:, half:], weight[:, half:].t(), out_dtype=torch.float32)).to(torch.bfloat16)
+
+    _MID_FORMS = {"bf16": lambda x, w: torch.matmul(x, w.t()),
+                  "f32": lambda x, w: torch.mm(x, w.t(), out_dtype=torch.float32).to(torch.bfloat16),
+                  "f32x2": lambda x, w: HipKernels._two_halves(x, w)}
+
+    def _time_mid_forms(self, x, weight) -> str:
+        took = {}
+        try:
+            for name, fn in self._MID_FORMS.items():
+                if name == "f32x2" and weight.shape[1] % 512:
+                    continue
+                for _ in range(2):
+                    fn(x, weight)
+                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                for _ in range(6):
+                    fn(x, weight)
+                end.record()
+                end.synchronize()
+                took[name] = start.elapsed_time(end)
+        except (RuntimeError, TypeError):           # this torch has no float32 result for a bfloat16 product
+            self._mid_forms = False
+            return "bf16"
+        best = min(took, key=took.get)
+        return best if took[best] < 0.85 * took["bf16"] else "bf16"
 
     def linear_add(self, x, weight, tiled, residual, want_stats=False):
         """-> False when not fused; otherwise True, or with `want_stats` the partial sums of squares [N / 16, 16] of

@@ -354,6 +354,28 @@ def test_linear(hip, dtype):
     assert H.op_budget_usage(hip.linear(x[:1].contiguous(), w), hip.linear(x, w)[:1].float(), dtype, 4096) <= 1
 
 
+def test_vendor_product_forms_for_steps_of_17_to_64_rows(hip):
+    """Steps of 17 to 64 bfloat16 rows take the vendor library's product in the faster of two forms, timed once per
+    weight shape and row bucket: both are the product rounded once, whichever is kept, and the float32 output is the
+    bfloat16 one cast up."""
+    bf = torch.bfloat16
+    for m, k, n in ((32, 25600, 5120), (24, 4096, 6144), (64, 1024, 512)):
+        x, w = _randn(m, k, dtype=bf, seed=70), _randn(n, k, dtype=bf, seed=71, scale=0.02)
+        want = x.double() @ w.double().T
+        key = ((n, k), m <= 32)
+        hip._mid_choice.pop(key, None)
+        got = hip.linear(x, w)
+        assert hip._mid_choice[key] in ("bf16", "f32", "f32x2")           # timed and kept
+        for form in ("bf16", "f32", "f32x2"):
+            hip._mid_choice[key] = form
+            y = hip.linear(x, w)
+            assert y.dtype == bf and H.op_budget_usage(y, want, bf, k) <= 1, (m, k, n, form)
+            assert torch.equal(hip.linear(x, w, torch.float32), y.float())
+        assert H.op_budget_usage(got, want, bf, k) <= 1
+    assert ((5120, 25600), False) not in hip._mid_choice                   # the other bucket was never asked for
+    hip._mid_choice.clear()
+
+
 def test_float32_product_is_true_32_bit_and_its_order_is_fixed(hip):
     """The 32-bit path's own product: close to the float64 product as only true float32 arithmetic is (a
     reduced-precision matrix mode would be a thousand times off), at odd sizes (K no multiple of 4 or 32, N and M
