@@ -5,7 +5,9 @@ folder by itself (config.json, model.safetensors, Hugging Face tensor names) and
 the formulas of the reference engine, cited per function as `file:line` under the reference tree.
 
 `dtype` is the activation and weight dtype. Every part computes in float32 inside and rounds its result to `dtype`
-once, where the reference's oracles round; with `dtype=torch.float32` no rounding happens anywhere.
+once, where the reference's oracles round; with `dtype=torch.float32` no rounding happens anywhere. With
+`dtype=torch.float64` every part computes in float64 instead, the rotation angles included: the same formulas almost
+free of rounding, which tells how far the float32 evaluation itself is from them.
 """
 from __future__ import annotations
 
@@ -16,19 +18,25 @@ import torch
 from safetensors import safe_open
 
 
+def wide(x: torch.Tensor) -> torch.Tensor:
+    """`x` in the type a part computes in: float32, or float64 for a float64 model."""
+    return x if x.dtype == torch.float64 else x.float()
+
+
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """x / sqrt(mean(x^2) + eps) * weight over the last dim, one rounding at the end.
     std/holon_std/ops/reference.py:7-11 (offset 0 for Qwen3)."""
-    x32 = x.float()
+    x32 = wide(x)
     inv = torch.rsqrt((x32 * x32).mean(dim=-1, keepdim=True) + eps)
-    return (x32 * inv * weight.float()).to(x.dtype)
+    return (x32 * inv * wide(weight)).to(x.dtype)
 
 
-def rope_angles(positions: torch.Tensor, head_dim: int, theta: float) -> tuple[torch.Tensor, torch.Tensor]:
-    """cos and sin of position * theta^(-2i/D), i < D/2, all float32.
+def rope_angles(positions: torch.Tensor, head_dim: int, theta: float, work: torch.dtype = torch.float32
+                ) -> tuple[torch.Tensor, torch.Tensor]:
+    """cos and sin of position * theta^(-2i/D), i < D/2, all float32 (`work`: float64 for a float64 model).
     std/holon_std/ops/reference.py:24-26."""
-    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
-    angles = positions.to(torch.float32)[:, None] * inv_freq.to(positions.device)[None, :]
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=work) / head_dim))
+    angles = positions.to(work)[:, None] * inv_freq.to(positions.device)[None, :]
     return angles.cos(), angles.sin()
 
 
@@ -36,9 +44,9 @@ def rope_neox(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.T
     """Half-split rotation of x [T, heads, D]: pairs are (i, i + D/2).
     std/holon_std/ops/reference.py:21-30."""
     half = x.shape[-1] // 2
-    cos, sin = rope_angles(positions, x.shape[-1], theta)
+    cos, sin = rope_angles(positions, x.shape[-1], theta, wide(x).dtype)
     cos, sin = cos[:, None, :], sin[:, None, :]
-    a, b = x[..., :half].float(), x[..., half:].float()
+    a, b = wide(x[..., :half]), wide(x[..., half:])
     return torch.cat((a * cos - b * sin, b * cos + a * sin), dim=-1).to(x.dtype)
 
 
@@ -48,9 +56,9 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: 
     std/holon_std/mixers/gqa/reference.py:7-24."""
     t, hq, d = q.shape
     group = hq // k.shape[1]
-    k32 = k.float().repeat_interleave(group, dim=1)
-    v32 = v.float().repeat_interleave(group, dim=1)
-    scores = torch.einsum("qhd,khd->hqk", q.float(), k32) / d ** 0.5
+    k32 = wide(k).repeat_interleave(group, dim=1)
+    v32 = wide(v).repeat_interleave(group, dim=1)
+    scores = torch.einsum("qhd,khd->hqk", wide(q), k32) / d ** 0.5
     pos = torch.arange(t, device=q.device)
     hidden = pos[None, :] > pos[:, None]
     if window:
@@ -62,13 +70,13 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: 
 def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """x @ weight.T, no bias, float32 accumulation, rounded to x's dtype.
     std/holon_std/ops/units.py:229 (F.linear); std/holon_std/ops/reference.py:33-34."""
-    return (x.float() @ weight.float().T).to(x.dtype)
+    return (wide(x) @ wide(weight).T).to(x.dtype)
 
 
 def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """silu(gate) in float32, rounded, times up in the activation dtype.
     std/holon_std/ffn/reference.py:7-12."""
-    g = gate.float()
+    g = wide(gate)
     return (g * torch.sigmoid(g)).to(gate.dtype) * up
 
 
@@ -114,7 +122,7 @@ def rope_theta(cfg: dict) -> float:
 
 
 def logits_of(ids: list[int], w: dict[str, torch.Tensor], cfg: dict) -> torch.Tensor:
-    """Float32 logits [T, V] of every token of one sequence.
+    """Float32 logits [T, V] of every token of one sequence (float64 from a float64 model).
     core/holon/core/build.py:296-307 (embed, blocks, final norm, head); std/holon_std/ops/units.py:345-348 (head reads
     the embedding when tied; logits are float32)."""
     table = w["model.embed_tokens.weight"]
@@ -124,7 +132,7 @@ def logits_of(ids: list[int], w: dict[str, torch.Tensor], cfg: dict) -> torch.Te
         h = block(h, positions, w, i, cfg)
     h = rms_norm(h, w["model.norm.weight"], cfg["rms_norm_eps"])
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
-    return linear(h, head).float()
+    return wide(linear(h, head))
 
 
 def read_folder(folder: str | pathlib.Path, dtype: torch.dtype = torch.float32, device: str = "cpu"
