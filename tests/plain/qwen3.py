@@ -5,12 +5,14 @@ folder by itself (config.json, model.safetensors, Hugging Face tensor names) and
 the formulas of the reference engine, cited per function as `file:line` under the reference tree.
 
 `dtype` is the activation and weight dtype. Every part computes in float32 inside and rounds its result to `dtype`
-once, where the reference's oracles round; with `dtype=torch.float32` no rounding happens anywhere. With
-`dtype=torch.float64` every part computes in float64 instead, the rotation angles included: the same formulas almost
-free of rounding, which tells how far the float32 evaluation itself is from them.
+once, where the reference's oracles round; with `dtype=torch.float32` no rounding happens anywhere. The whole model
+in float64 (`PlainQwen3(folder, torch.float64)`) computes every part in float64 instead (`computing_in`), rotation
+angles included: the same formulas almost free of rounding, which tells how far the float32 evaluation itself is from
+them.
 """
 from __future__ import annotations
 
+import contextlib
 import json
 import pathlib
 
@@ -18,9 +20,22 @@ import torch
 from safetensors import safe_open
 
 
+_WORK = [torch.float32]
+
+
 def wide(x: torch.Tensor) -> torch.Tensor:
-    """`x` in the type a part computes in: float32, or float64 for a float64 model."""
-    return x if x.dtype == torch.float64 else x.float()
+    """`x` in the type a part computes in: float32, or what `computing_in` says."""
+    return x.to(_WORK[-1])
+
+
+@contextlib.contextmanager
+def computing_in(dtype: torch.dtype):
+    """Inside, every part computes in `dtype` instead of float32."""
+    _WORK.append(dtype)
+    try:
+        yield
+    finally:
+        _WORK.pop()
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
@@ -31,10 +46,10 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return (x32 * inv * wide(weight)).to(x.dtype)
 
 
-def rope_angles(positions: torch.Tensor, head_dim: int, theta: float, work: torch.dtype = torch.float32
-                ) -> tuple[torch.Tensor, torch.Tensor]:
-    """cos and sin of position * theta^(-2i/D), i < D/2, all float32 (`work`: float64 for a float64 model).
+def rope_angles(positions: torch.Tensor, head_dim: int, theta: float) -> tuple[torch.Tensor, torch.Tensor]:
+    """cos and sin of position * theta^(-2i/D), i < D/2, all float32.
     std/holon_std/ops/reference.py:24-26."""
+    work = _WORK[-1]
     inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=work) / head_dim))
     angles = positions.to(work)[:, None] * inv_freq.to(positions.device)[None, :]
     return angles.cos(), angles.sin()
@@ -44,7 +59,7 @@ def rope_neox(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.T
     """Half-split rotation of x [T, heads, D]: pairs are (i, i + D/2).
     std/holon_std/ops/reference.py:21-30."""
     half = x.shape[-1] // 2
-    cos, sin = rope_angles(positions, x.shape[-1], theta, wide(x).dtype)
+    cos, sin = rope_angles(positions, x.shape[-1], theta)
     cos, sin = cos[:, None, :], sin[:, None, :]
     a, b = wide(x[..., :half]), wide(x[..., half:])
     return torch.cat((a * cos - b * sin, b * cos + a * sin), dim=-1).to(x.dtype)
@@ -153,10 +168,12 @@ class PlainQwen3:
 
     def __init__(self, folder: str | pathlib.Path, dtype: torch.dtype = torch.float32, device: str = "cpu") -> None:
         self.cfg, self.weights = read_folder(folder, dtype, device)
+        self.work = torch.float64 if dtype == torch.float64 else torch.float32
 
     @torch.no_grad()
     def logits(self, ids: list[int]) -> torch.Tensor:
-        return logits_of(ids, self.weights, self.cfg)
+        with computing_in(self.work):
+            return logits_of(ids, self.weights, self.cfg)
 
     @torch.no_grad()
     def greedy(self, ids: list[int], n: int) -> list[int]:
