@@ -233,15 +233,16 @@ static void launch_skinny(const void* x, const void* w, void* y, int M, int N, i
 //   320 to 512 tiles: 8 waves; two tiles 9.9 / 10.7 / 12.2 (320), 11.5 / 12.3 / 13.8 (384), 14.0 / 14.6 / 15.8 (512)
 //     against one 10.8 / 12.8 / 16.1, 11.9 / 14.2 / 16.8, 13.8 / 15.5 / 17.9;
 //   640 tiles: 8 waves, one tile 17.2 / 20.0 / 23.1 against two 19.1 / 21.1 / 23.3;
-//   9,496 tiles: 8 waves; one tile at one row (182 against 187), two from four rows up (8 rows 195 against 210, 16 rows
-//     198 against 255).
+//   9,496 tiles (float32 result): 8 waves; one tile up to 8 rows (4 rows 181 against 195, 8 rows 192 against 201), two
+//     from 10 rows up (12 rows 211 against 220, 16 rows 223 against 251).
+constexpr int SKINNY_WIDE_TWO_FROM = 10;   // rows from which a vocabulary's worth of tiles is walked two a block
 template <typename OutT, bool RESID = false>
 static int pick_waves(const void* x, const void* w, void* y, int M, int N, int K, bool tiled, hipStream_t s,
                       int round_first = 0, RowScale rs = RowScale{nullptr, 0, 0.f, 0.f}, float* stats_out = nullptr) {
   const int tiles = N / 16;
   int wpb = tiles >= 320 ? 8 : 16;
   while (wpb > 1 && K % (32 * wpb) != 0) wpb /= 2;
-  const bool two = tiles % 2 == 0 && wpb <= 8 && ((tiles >= 320 && tiles <= 512) || (tiles > 4096 && M >= 4));
+  const bool two = tiles % 2 == 0 && wpb <= 8 && ((tiles >= 320 && tiles <= 512) || (tiles > 4096 && M >= SKINNY_WIDE_TWO_FROM));
 #define SKINNY(WPB, U)                                                                                         \
   if (two) launch_skinny<2, WPB, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out);     \
   else launch_skinny<1, WPB, U, OutT, RESID>(x, w, y, M, N, K, tiled, s, round_first, rs, stats_out)

@@ -328,7 +328,7 @@ def test_linear(hip, dtype):
                     (1, 4096, 4096), (16, 12288, 4096), (3, 4096, 24576), (9, 512, 208), (33, 1024, 4096),
                     (48, 4096, 512), (5, 12288, 151936 // 8), (65, 4096, 512),
                     (1, 8192, 5120), (12, 4096, 8192),                   # 320 and 512 tiles: two tiles a block
-                    (5, 512, 80_000), (2, 512, 80_000), (16, 256, 65_568)):   # a vocabulary's worth: two from four rows up
+                    (5, 512, 80_000), (12, 512, 80_000), (16, 256, 65_568)):  # a vocabulary's worth: two from ten rows up
         x, w = _randn(t, k, dtype=dtype, seed=13), _randn(n, k, dtype=dtype, seed=14, scale=0.05)
         want = x.double() @ w.double().T
         got = hip.linear(x, w)
