@@ -1,0 +1,183 @@
+// y[M, N] = x[M, K] w[N, K]^T for 17 to 64 rows (decode steps of many requests) over weights with many tiles of 16
+// rows (a gated feed-forward's first product, the head): bfloat16 operands, float32 accumulation on the matrix cores.
+//
+// The few-row kernel streams the weights and lets every block read its rows of activations from L2; with 64 rows those
+// reads cost as much as the weights. Here a block's waves walk K together and share the rows through LDS: a chunk of
+// KC columns of all rows is copied in once per block (double buffered, the next chunk's copy under way while this one
+// is used), each wave streams the weights of its own tile (from the tiled copy: a contiguous kilobyte a product) for
+// the next chunk while it multiplies this one, and reads its activations as B operands from LDS. A wave sums its tile
+// over all of K in order, so a result depends on nothing but the operands. Blocks do not split K: the kernel is for
+// weights with tiles enough to fill the GPU (the host refuses others, which stay with the vendor library).
+//
+// v_mfma_f32_16x16x32_bf16 with the weights as A and MT tiles of 16 tokens as B, as in the few-row kernel.
+#include "common.h"
+#include "holon_hip.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+namespace {
+// OUT: 0 bfloat16, 1 float32 of the values rounded to bfloat16 (the product in the operands' type, cast up),
+//      2 the gated form, bfloat16 round(silu(round(gate))) * round(up): the first half of a block's waves own gate
+//      tiles, the second half the up tiles of the same columns (I / 16 tiles further on), and the halves meet in LDS.
+template <int MT, int WAVES, int KC, int OUT>
+__global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(const bf16_t* __restrict__ x,
+                                                               const bf16_t* __restrict__ w, void* __restrict__ y,
+                                                               int M, int N, int K) {
+  constexpr int ROWS = MT * 16, PITCH = KC + 8, STEPS = KC / 32, THREADS = WAVES * 64;
+  constexpr int PIECES = ROWS * KC / 8;                     // 16-byte pieces of a chunk of activations
+  constexpr int XCH = (PIECES + THREADS - 1) / THREADS;     // of which a thread copies this many
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][ROWS * PITCH];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, tid = threadIdx.x;
+  const int g = lane / 16, c = lane % 16;
+  constexpr bool GATED = OUT == 2;
+  constexpr int COLS = GATED ? WAVES / 2 : WAVES;            // output tiles of 16 columns a block writes
+  const bool up_half = GATED && wave >= COLS;                // (gated) this wave owns an up tile
+  const int col_tile = blockIdx.x * COLS + wave % COLS;      // N / 16 is a multiple of COLS
+  const int tile = col_tile + (up_half ? N / 16 : 0);        // the weight's tile: up rows lie I / 16 tiles further on
+  const bf16_t* wp = w + (int64_t)tile * (K / 32) * 512 + lane * 8;
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  bf16x8_t wcur[STEPS], wnext[STEPS], xr[XCH];
+  auto load_w = [&](int chunk, bf16x8_t (&to)[STEPS]) {
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+      to[s] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp + ((int64_t)chunk * STEPS + s) * 512));
+  };
+  auto load_x = [&](int chunk) {                            // rows beyond M are zeros
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) {
+      const int q = tid + i * THREADS;
+      const int row = q / (KC / 8), col = (q % (KC / 8)) * 8;
+      if (q < PIECES && row < M) {
+        xr[i] = *reinterpret_cast<const bf16x8_t*>(x + (int64_t)row * K + (int64_t)chunk * KC + col);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xr[i][j] = (__bf16)0.f;
+      }
+    }
+  };
+  auto store_x = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) {
+      const int q = tid + i * THREADS;
+      const int row = q / (KC / 8), col = (q % (KC / 8)) * 8;
+      if (q < PIECES) *reinterpret_cast<bf16x8_t*>(&xs[buf][row * PITCH + col]) = xr[i];
+    }
+  };
+  const int chunks = K / KC;
+  load_w(0, wcur);
+  load_x(0);
+  store_x(0);
+  __syncthreads();
+  for (int ch = 0; ch < chunks; ++ch) {
+    const int buf = ch & 1;
+    const bool more = ch + 1 < chunks;                      // (uniform)
+    if (more) {
+      load_w(ch + 1, wnext);
+      load_x(ch + 1);
+    }
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(&xs[buf][(t * 16 + c) * PITCH + s * 32 + 8 * g]);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wcur[s], b, acc[t], 0, 0, 0);
+      }
+    if (more) {
+      store_x(buf ^ 1);                                     // the other buffer: last read before the barrier below
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) wcur[s] = wnext[s];
+    }
+    __syncthreads();
+  }
+  if constexpr (GATED) {                                     // the gate waves hand their rounded sums to the up waves
+    f32x4_t* meet = reinterpret_cast<f32x4_t*>(&xs[0][0]);   // (every wave is past its last read of the rows)
+    static_assert(COLS * MT * WAVE * sizeof(f32x4_t) <= sizeof(xs), "the gate tiles fit the rows' buffers");
+    if (!up_half) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t) meet[(wave * MT + t) * WAVE + lane] = acc[t];
+    }
+    __syncthreads();
+    if (!up_half) return;
+  }
+  // lane holds outputs 4 g .. 4 g + 3 of the tile for token 16 t + c
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + c;
+    if (m >= M) continue;
+    if constexpr (OUT == 1) {
+      f32x4_t o;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[r] = bf16_to_float(float_to_bf16(acc[t][r]));
+      *reinterpret_cast<f32x4_t*>((float*)y + (int64_t)m * N + col_tile * 16 + 4 * g) = o;
+    } else {
+      ushort4 o;
+      bf16_t* oe = reinterpret_cast<bf16_t*>(&o);
+      f32x4_t gates;
+      if constexpr (GATED) gates = reinterpret_cast<const f32x4_t*>(&xs[0][0])[((wave - COLS) * MT + t) * WAVE + lane];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if constexpr (GATED) {
+          const float gate = bf16_to_float(float_to_bf16(gates[r]));
+          const float up = bf16_to_float(float_to_bf16(acc[t][r]));
+          const float sg = bf16_to_float(float_to_bf16(silu<bf16_t>(gate)));
+          oe[r] = float_to_bf16(sg * up);
+        } else {
+          oe[r] = float_to_bf16(acc[t][r]);
+        }
+      }
+      *reinterpret_cast<ushort4*>((bf16_t*)y + (int64_t)m * N + col_tile * 16 + 4 * g) = o;
+    }
+  }
+}
+
+constexpr int ROWS_MIN_TILES = 1024;   // tiles (gated: tile pairs times two) from which the kernel fills the GPU
+
+template <int WAVES, int KC, int OUT>
+void launch_rows(const void* x, const void* w, void* y, int M, int N, int K, hipStream_t s) {
+  const dim3 grid(N / 16 / (OUT == 2 ? WAVES / 2 : WAVES)), block(WAVES * 64);
+  const int mt = (M + 15) / 16;
+#define ROWS(MT) gemm_rows_kernel<MT, WAVES, KC, OUT><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, y, M, N, K)
+  if (mt == 2) ROWS(2); else if (mt == 3) ROWS(3); else ROWS(4);
+#undef ROWS
+}
+}  // namespace
+
+// Whether holon_gemm_rows_bf16 serves this product (gated: N is the number of output columns I, the weight has 2 I rows).
+extern "C" int holon_gemm_rows_supported(int M, int N, int K, int gated) {
+  const int tiles = N / 16;
+  return M > 16 && M <= 64 && N % 16 == 0 && K % 256 == 0 && K >= 256 && tiles % 8 == 0 &&
+         tiles * (gated ? 2 : 1) >= ROWS_MIN_TILES;
+}
+
+// y[M, N] = x[M, K] w^T over tiled weights, 17 <= M <= 64; out_f32: 0 bfloat16, otherwise float32 of the values rounded
+// to bfloat16. Measured on MI355X at N = 24,576, K = 4,096: 44 us at 64 rows, 39 at 32 (the vendor library 47 and 46);
+// N = 151,936: 238 and 219 us (267 and 269).
+extern "C" int holon_gemm_rows_bf16(const void* x, const void* w_tiled, void* y, int M, int N, int K, int out_f32,
+                                    void* stream) {
+  HOLON_CHECK(holon_gemm_rows_supported(M, N, K, 0), "gemm (17 to 64 rows): M=%d N=%d K=%d not served", M, N, K);
+  hipStream_t s = (hipStream_t)stream;
+  const bool wide = N / 16 >= 4096;          // a vocabulary's worth of tiles: longer chunks, at 64 rows eight waves
+  if (out_f32) {
+    if (wide && M > 48) launch_rows<8, 256, 1>(x, w_tiled, y, M, N, K, s);
+    else if (wide) launch_rows<4, 256, 1>(x, w_tiled, y, M, N, K, s);
+    else launch_rows<4, 128, 1>(x, w_tiled, y, M, N, K, s);
+  } else {
+    if (wide && M > 48) launch_rows<8, 256, 0>(x, w_tiled, y, M, N, K, s);
+    else if (wide) launch_rows<4, 256, 0>(x, w_tiled, y, M, N, K, s);
+    else launch_rows<4, 128, 0>(x, w_tiled, y, M, N, K, s);
+  }
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+// y[M, I] = round(silu(round(x gate^T))) * round(x up^T) with w = [gate; up] ([2 I, K], tiled), 17 <= M <= 64: four waves
+// a block, two gate tiles and the two up tiles of the same columns.
+extern "C" int holon_gemm_rows_glu_bf16(const void* x, const void* w_tiled, void* y, int M, int I, int K, void* stream) {
+  HOLON_CHECK(holon_gemm_rows_supported(M, I, K, 1), "gated gemm (17 to 64 rows): M=%d I=%d K=%d not served", M, I, K);
+  launch_rows<4, 128, 2>(x, w_tiled, y, M, I, K, (hipStream_t)stream);
+  HOLON_LAUNCH_OK();
+  return 0;
+}

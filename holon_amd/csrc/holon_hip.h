@@ -85,6 +85,12 @@ int holon_gemm_skinny_scaled_bf16(const void* x, const void* w_tiled, void* y, i
 // stats (nullable): as in holon_gemm_skinny_scaled_bf16 (tiled weights with the norm's weight folded in).
 int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int I, int K, int tiled, const float* stats,
                                int parts, float eps, void* stream);
+// The same products for 17 <= M <= 64 rows over tiled weights with many tiles (N / 16 a multiple of 8 and at least
+// 1,024; K a multiple of 256): the rows of activations go through LDS, shared by a block's waves, and every wave sums
+// its tile over all of K in order. `gated`: N is I and the weight has 2 I rows.
+int holon_gemm_rows_supported(int M, int N, int K, int gated);
+int holon_gemm_rows_bf16(const void* x, const void* w_tiled, void* y, int M, int N, int K, int out_f32, void* stream);
+int holon_gemm_rows_glu_bf16(const void* x, const void* w_tiled, void* y, int M, int I, int K, void* stream);
 // y[M, N] = x[M, K] w[N, K]^T, all float32, true 32-bit products and sums in an order that depends on K alone: a row's
 // result is bit for bit the same whatever other rows are in the call.
 int holon_gemm_f32(const void* x, const void* w, void* y, int M, int N, int K, void* stream);

@@ -77,6 +77,12 @@ class Kernels(Protocol):
         """Once per weight after loading: a copy in the layout steps of few rows stream fastest, or None. With
         `scale` [K] the copy holds weight * scale[None, :] (rounded): a norm's weight folded in."""
 
+    def serves_rows(self, rows: int, weight: torch.Tensor, tiled: torch.Tensor | None, gated: bool = False) -> bool:
+        """Whether `linear` (gated: `linear_silu_mul`) reads `tiled` for a step of `rows` rows beyond the few-row
+        kernels' (17 to 64): a caller whose tiled copy has a norm folded in then passes rows normed without the
+        norm's weight."""
+        return False
+
     def linear_add(self, x: torch.Tensor, weight: torch.Tensor, tiled: torch.Tensor | None, residual: torch.Tensor,
                    want_stats: bool = False) -> "bool | torch.Tensor":
         """residual += linear(x, weight) in place in one kernel: the product rounded to dtype, then the sum rounded,

@@ -69,6 +69,9 @@ class HipKernels:
             "holon_gemm_skinny_supported": [_I, _I, _I],
             "holon_gemm_skinny_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
             "holon_tile_weight_bf16": [_P, _P, _I, _I, _P, _P],
+            "holon_gemm_rows_supported": [_I, _I, _I, _I],
+            "holon_gemm_rows_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
+            "holon_gemm_rows_glu_bf16": [_P, _P, _P, _I, _I, _I, _P],
             "holon_gemm_skinny_scaled_bf16": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _F, _P],
             "holon_gemm_f32": [_P, _P, _P, _I, _I, _I, _P],
             "holon_gemm_skinny_add_bf16": [_P, _P, _P, _I, _I, _I, _P, _P],
@@ -217,6 +220,12 @@ class HipKernels:
             self._call(self.lib.holon_gemm_skinny_bf16, x.data_ptr(), source.data_ptr(), y.data_ptr(), m, n, k,
                        2 if to_f32 else 0, int(tiled is not None), self._stream())
             return y
+        if self.serves_rows(m, weight, tiled) and x.dtype == torch.bfloat16 and x.is_contiguous():
+            to_f32 = out_dtype == torch.float32
+            y = torch.empty((m, n), dtype=torch.float32 if to_f32 else torch.bfloat16, device=x.device)
+            self._call(self.lib.holon_gemm_rows_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), m, n, k,
+                       int(to_f32), self._stream())
+            return y
         if x.dtype == torch.float32 and weight.dtype == torch.float32 and out_dtype in (None, torch.float32):
             # the 32-bit path's own product: true float32, every sum in an order that K alone decides
             self._check(x, "linear x")
@@ -276,6 +285,13 @@ class HipKernels:
         best = min(took, key=took.get)
         return best if took[best] < 0.85 * took["bf16"] else "bf16"
 
+    def serves_rows(self, rows, weight, tiled, gated=False):
+        """Whether steps of `rows` rows (17 to 64) over this weight run the product that shares the rows through LDS
+        (`tiled` is then read; a copy with a norm folded in needs rows normed without the norm's weight)."""
+        n, k = weight.shape
+        return bool(tiled is not None and weight.dtype == torch.bfloat16 and 16 < rows <= 64
+                    and self.lib.holon_gemm_rows_supported(rows, n // 2 if gated else n, k, int(gated)))
+
     def linear_add(self, x, weight, tiled, residual, want_stats=False):
         """-> False when not fused; otherwise True, or with `want_stats` the partial sums of squares [N / 16, 16] of
         the residual rows as they now are."""
@@ -297,6 +313,12 @@ class HipKernels:
         after the other (the sums over K may be split differently); None when this shape is not fused (the caller then composes the two)."""
         m, k = x.shape
         two_i = weight.shape[0]
+        if row_scale is None and weight.shape[1] == k and x.dtype == torch.bfloat16 and x.is_contiguous() \
+                and two_i % 2 == 0 and self.serves_rows(m, weight, tiled, gated=True):
+            y = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
+            self._call(self.lib.holon_gemm_rows_glu_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), m, two_i // 2, k,
+                       self._stream())
+            return y
         if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows
                 and two_i % 32 == 0 and k % 128 == 0 and k >= 256 and weight.shape[1] == k and x.is_contiguous()):
             return None

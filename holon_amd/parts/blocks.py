@@ -36,18 +36,18 @@ class PreNorm(Part):
         that can add its result into `h` inside its own kernel (`adds_residual`) is given the stream; it returns None
         when it did (and the kernel leaves the rows' statistics in `stream.stats` for the norm that follows)."""
         h = stream.h
-        if stream.delta is not None:
+        if self._mixer_defers:
+            a = self.input_norm.defer(h, stream.stats, stream.delta)
+        elif stream.delta is not None:
             a = self.input_norm.add(stream.delta, h)[0]
-        elif self._mixer_defers:
-            a = self.input_norm.defer(h, stream.stats)
         else:
             a = self.input_norm(h)
         stream.delta = stream.stats = None
         mixed = self.mixer(a, step, site, **({"residual": stream} if self.mixer.adds_residual else {}))
-        if mixed is not None:
+        if self._ffn_defers:
+            x = self.post_norm.defer(h, stream.stats, mixed)
+        elif mixed is not None:
             x = self.post_norm.add(mixed, h)[0]
-        elif self._ffn_defers:
-            x = self.post_norm.defer(h, stream.stats)
         else:
             x = self.post_norm(h)
         stream.stats = None

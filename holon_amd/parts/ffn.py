@@ -39,6 +39,8 @@ class SwiGLU(Part):
         gate_up, y = self.gate_up, None
         if gate_up.folds(x):
             y = self.kernels.linear_silu_mul(x.h, gate_up.weight, gate_up.tiled, row_scale=gate_up.row_scale(x))
+        elif gate_up.reads_folded(x, gated=True):  # 17 to 64 rows: the folded copy over rows normed without the weight
+            y = self.kernels.linear_silu_mul(x.unit_value(), gate_up.weight, gate_up.tiled)
         elif gate_up.folded is None:               # fused for steps of few rows
             x = x.value() if isinstance(x, Normed) else x
             y = self.kernels.linear_silu_mul(x, gate_up.weight, gate_up.tiled)

@@ -38,9 +38,16 @@ class Linear(Part):
         return True
 
     def folds(self, x: torch.Tensor | Normed) -> bool:
-        """Whether `x` is the deferred norm this projection folded, at a number of rows its kernel serves."""
-        return isinstance(x, Normed) and x.norm is self.folded and \
+        """Whether `x` is the deferred norm this projection folded, with nothing left to add to its rows, at a number
+        of rows its kernel serves."""
+        return isinstance(x, Normed) and x.norm is self.folded and x.delta is None and \
             self.kernels.folds_norm(x.h.shape[0], self.weight, self.tiled)
+
+    def reads_folded(self, x: torch.Tensor | Normed, gated: bool = False) -> bool:
+        """Whether `x` is the deferred norm this projection folded, at a number of rows whose product reads the folded
+        copy over rows normed without the norm's weight."""
+        return isinstance(x, Normed) and x.norm is self.folded and \
+            self.kernels.serves_rows(x.h.shape[0], self.weight, self.tiled, gated)
 
     def row_scale(self, x: Normed) -> tuple[torch.Tensor, float]:
         stats = x.stats if x.stats is not None else self.kernels.row_sumsq(x.h)
@@ -54,6 +61,8 @@ class Linear(Part):
         if isinstance(x, Normed):
             if self.folds(x):
                 return self.kernels.linear(x.h, self.weight, out_dtype, self.tiled, row_scale=self.row_scale(x))
+            if self.reads_folded(x):
+                return self.kernels.linear(x.unit_value(), self.weight, out_dtype, self.tiled)
             x = x.value()
         tiled = self.tiled if self.folded is None else None       # a folded copy is not this weight any more
         if residual is not None and out_dtype is None:

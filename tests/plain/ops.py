@@ -74,6 +74,11 @@ class TorchKernels:
     def folds_norm(self, rows, weight, tiled):
         return tiled is not None and rows <= 16
 
+    def serves_rows(self, rows, weight, tiled, gated=False):
+        """With `fold_norms`, steps of 17 to 64 rows read the stand-in for the tiled copy, as the HIP kernels do for
+        weights with many tiles."""
+        return tiled is not None and self.fold_norms and 16 < rows <= 64
+
     @staticmethod
     def _scaled(x, folded, row_scale):
         stats, eps = row_scale
@@ -83,6 +88,8 @@ class TorchKernels:
     def linear(self, x, weight, out_dtype=None, tiled=None, row_scale=None):
         if row_scale is not None:
             return self._scaled(x, tiled, row_scale).to(x.dtype).to(out_dtype or x.dtype)
+        if self.serves_rows(x.shape[0], weight, tiled):
+            weight = tiled                                   # (folded or not: what the caller's rows were prepared for)
         return (_up(x) @ _up(weight).T).to(x.dtype).to(out_dtype or x.dtype)      # rounded to x's dtype, then cast
 
     def linear_add(self, x, weight, tiled, residual, want_stats=False):
@@ -92,6 +99,8 @@ class TorchKernels:
         return True
 
     def linear_silu_mul(self, x, weight, tiled=None, row_scale=None):
+        if row_scale is None and self.serves_rows(x.shape[0], weight, tiled, gated=True):
+            return self.silu_mul(self.linear(x, weight, None, tiled))
         if row_scale is None:
             return None
         return self.silu_mul(self._scaled(x, tiled, row_scale).to(x.dtype))

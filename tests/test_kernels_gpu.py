@@ -354,6 +354,39 @@ def test_linear(hip, dtype):
     assert H.op_budget_usage(hip.linear(x[:1].contiguous(), w), hip.linear(x, w)[:1].float(), dtype, 4096) <= 1
 
 
+def test_product_for_17_to_64_rows_over_many_tiles(hip):
+    """Steps of 17 to 64 rows over weights with at least 1,024 tiles of 16 rows read the tiled copy through the kernel
+    that shares the rows through LDS: plain, with a float32 result (the bfloat16 one cast up), and gated; against
+    float64 and against the same product over the rows as they are. A row's result is bit for bit the same whatever
+    rows lie beside it, and fewer tiles, other row counts and other K stay where they were."""
+    bf = torch.bfloat16
+    for m, k, n in ((17, 256, 16384), (64, 4096, 24576), (33, 1024, 16512), (48, 512, 65536), (64, 768, 65664), (20, 256, 131072)):
+        x, w = _randn(m, k, dtype=bf, seed=80), _randn(n, k, dtype=bf, seed=81, scale=0.05)
+        tiled = hip.tile_weight(w)
+        assert hip.serves_rows(m, w, tiled) and not hip.serves_rows(16, w, tiled) and not hip.serves_rows(65, w, tiled)
+        want = x.double() @ w.double().T
+        got = hip.linear(x, w, None, tiled)
+        assert got.dtype == bf and H.op_budget_usage(got, want, bf, k) <= 1, (m, k, n)
+        assert H.op_budget_usage(got, hip.linear(x, w).double(), bf, k) <= 1          # the vendor library's, over the rows
+        assert torch.equal(hip.linear(x, w, torch.float32, tiled), got.float())
+        fewer = hip.linear(x[3:21].contiguous(), w, None, tiled)                       # 18 rows, other places
+        assert torch.equal(fewer, got[3:21]) if m >= 21 else True
+    for m, k, inter in ((64, 4096, 12288), (17, 256, 8192), (40, 1024, 8320)):
+        x, w = _randn(m, k, dtype=bf, seed=82), _randn(2 * inter, k, dtype=bf, seed=83, scale=0.05)
+        tiled = hip.tile_weight(w)
+        assert hip.serves_rows(m, w, tiled, gated=True)
+        exact = PLAIN.silu_mul(PLAIN.linear(x.double(), w.double()))
+        got = hip.linear_silu_mul(x, w, tiled)
+        assert got is not None and got.shape == (m, inter) and H.op_budget_usage(got, exact, bf, k) <= 1, (m, k, inter)
+        two = hip.silu_mul(hip.linear(x, w))                                           # the same roundings in two kernels
+        assert (got != two).float().mean() < 0.02
+    w = _randn(4096, 4096, dtype=bf, seed=84)
+    tiled = hip.tile_weight(w)
+    assert not hip.serves_rows(32, w, tiled) and not hip.serves_rows(32, w, None)      # 256 tiles: the vendor library's
+    w = _randn(16384, 384, dtype=bf, seed=85)
+    assert not hip.serves_rows(32, w, hip.tile_weight(w))                              # K no multiple of 256
+
+
 def test_vendor_product_forms_for_steps_of_17_to_64_rows(hip):
     """Steps of 17 to 64 bfloat16 rows take the vendor library's product in the faster of two forms, timed once per
     weight shape and row bucket: both are the product rounded once, whichever is kept, and the float32 output is the
