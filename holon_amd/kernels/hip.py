@@ -105,6 +105,19 @@ class HipKernels:
         if dtype is not None and t.dtype != dtype:
             raise KernelError(f"{what}: expected {dtype}, got {t.dtype}")
 
+    def _check_product(self, what: str, x, weight, tiled=None, *others) -> None:
+        """Before a product is launched on raw pointers: every operand on the GPU and contiguous, the tiled copy (which
+        the kernels index as they index the weight) of the weight's shape and type."""
+        self._check(x, f"{what} x")
+        self._check(weight, f"{what} weight")
+        if tiled is not None:
+            self._check(tiled, f"{what} tiled weight", weight.dtype)
+            if tiled.shape != weight.shape:
+                raise KernelError(f"{what}: a tiled copy of shape {tuple(tiled.shape)} for a weight of {tuple(weight.shape)}")
+        for t in others:
+            if t is not None:
+                self._check(t, f"{what} operand")
+
     @staticmethod
     def _dt(t: torch.Tensor, what: str) -> int:
         if t.dtype not in _DT:
@@ -206,7 +219,7 @@ class HipKernels:
             raise KernelError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(weight.shape)}")
         if row_scale is not None:
             stats, parts, eps = self._row_scale(x, tiled, row_scale, "linear")
-            self._check(x, "linear x")
+            self._check_product("linear", x, weight, tiled)
             to_f32 = out_dtype == torch.float32
             y = torch.empty((m, n), dtype=torch.float32 if to_f32 else torch.bfloat16, device=x.device)
             self._call(self.lib.holon_gemm_skinny_scaled_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), m, n, k,
@@ -215,6 +228,7 @@ class HipKernels:
         if (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows and k >= 256
                 and x.is_contiguous() and weight.is_contiguous() and self.lib.holon_gemm_skinny_supported(m, n, k)):
             to_f32 = out_dtype == torch.float32       # then: the bfloat16 product cast up, as for any number of rows
+            self._check_product("linear", x, weight, tiled)
             y = torch.empty((m, n), dtype=torch.float32 if to_f32 else torch.bfloat16, device=x.device)
             source = tiled if tiled is not None else weight
             self._call(self.lib.holon_gemm_skinny_bf16, x.data_ptr(), source.data_ptr(), y.data_ptr(), m, n, k,
@@ -222,6 +236,7 @@ class HipKernels:
             return y
         if self.serves_rows(m, weight, tiled) and x.dtype == torch.bfloat16 and x.is_contiguous():
             to_f32 = out_dtype == torch.float32
+            self._check_product("linear", x, weight, tiled)
             y = torch.empty((m, n), dtype=torch.float32 if to_f32 else torch.bfloat16, device=x.device)
             self._call(self.lib.holon_gemm_rows_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), m, n, k,
                        int(to_f32), self._stream())
@@ -303,6 +318,7 @@ class HipKernels:
             return False
         if tuple(residual.shape) != (m, n):
             raise KernelError(f"linear_add: residual {tuple(residual.shape)} for a product of {(m, n)}")
+        self._check_product("linear_add", x, weight, tiled, residual)
         stats = torch.empty((n // 16, 16), dtype=torch.float32, device=x.device) if want_stats else None
         self._call(self.lib.holon_gemm_skinny_add_bf16, x.data_ptr(), tiled.data_ptr(), residual.data_ptr(), m, n, k,
                    _ptr(stats), self._stream())
@@ -315,6 +331,7 @@ class HipKernels:
         two_i = weight.shape[0]
         if row_scale is None and weight.shape[1] == k and x.dtype == torch.bfloat16 and x.is_contiguous() \
                 and two_i % 2 == 0 and self.serves_rows(m, weight, tiled, gated=True):
+            self._check_product("linear_silu_mul", x, weight, tiled)
             y = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
             self._call(self.lib.holon_gemm_rows_glu_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), m, two_i // 2, k,
                        self._stream())
@@ -322,6 +339,7 @@ class HipKernels:
         if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows
                 and two_i % 32 == 0 and k % 128 == 0 and k >= 256 and weight.shape[1] == k and x.is_contiguous()):
             return None
+        self._check_product("linear_silu_mul", x, weight, tiled)
         y = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
         source = tiled if tiled is not None else weight
         stats, parts, eps = self._row_scale(x, tiled, row_scale, "linear_silu_mul") if row_scale is not None \

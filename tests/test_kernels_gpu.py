@@ -685,3 +685,19 @@ def test_kernels_refuse_what_they_do_not_serve(hip):
     q, pages, table, attn = _paged_case([(0, 4)], 2, 1, 12, 16, torch.float32)     # head_dim 12: not a multiple of 8
     with pytest.raises(KernelError, match="head_dim"):
         hip.paged_attention(q, pages, table, attn, 16, 1.0, 0)
+    # the products run on raw pointers: an operand off the GPU, or a tiled copy that is not this weight's, is refused
+    bf = torch.bfloat16
+    w, other = _randn(512, 1024, dtype=bf, seed=1), _randn(256, 1024, dtype=bf, seed=2)
+    tiled = hip.tile_weight(w)
+    big = _randn(16384, 256, dtype=bf, seed=3)
+    for rows, weight in ((4, w), (32, big)):
+        with pytest.raises(KernelError):
+            hip.linear(torch.zeros(rows, weight.shape[1], dtype=bf), weight, None, hip.tile_weight(weight))   # rows on the CPU
+    with pytest.raises(KernelError, match="tiled"):
+        hip.linear(_randn(32, 256, dtype=bf), big, None, hip.tile_weight(_randn(8192, 256, dtype=bf)))
+    with pytest.raises(KernelError, match="tiled"):
+        hip.linear(_randn(4, 1024, dtype=bf), w, None, hip.tile_weight(other))
+    with pytest.raises(KernelError, match="tiled"):
+        hip.linear_add(_randn(4, 1024, dtype=bf), w, hip.tile_weight(other), _randn(4, 512, dtype=bf))
+    with pytest.raises(KernelError):
+        hip.linear_add(_randn(4, 1024, dtype=bf), w, tiled, torch.zeros(4, 512, dtype=bf))   # residual on the CPU
