@@ -234,13 +234,8 @@ class HipKernels:
             self._call(self.lib.holon_gemm_skinny_bf16, x.data_ptr(), source.data_ptr(), y.data_ptr(), m, n, k,
                        2 if to_f32 else 0, int(tiled is not None), self._stream())
             return y
-        if self.serves_rows(m, weight, tiled) and x.dtype == torch.bfloat16 and x.is_contiguous():
-            to_f32 = out_dtype == torch.float32
-            self._check_product("linear", x, weight, tiled)
-            y = torch.empty((m, n), dtype=torch.float32 if to_f32 else torch.bfloat16, device=x.device)
-            self._call(self.lib.holon_gemm_rows_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), m, n, k,
-                       int(to_f32), self._stream())
-            return y
+        if x.dtype == torch.bfloat16 and x.is_contiguous() and self.serves_rows(m, weight, tiled):
+            return self._rows_product(x, weight, tiled, False, out_dtype == torch.float32)
         if x.dtype == torch.float32 and weight.dtype == torch.float32 and out_dtype in (None, torch.float32):
             # the 32-bit path's own product: true float32, every sum in an order that K alone decides
             self._check(x, "linear x")
@@ -302,10 +297,50 @@ class HipKernels:
 
     def serves_rows(self, rows, weight, tiled, gated=False):
         """Whether steps of `rows` rows (17 to 64) over this weight run the product that shares the rows through LDS
-        (`tiled` is then read; a copy with a norm folded in needs rows normed without the norm's weight)."""
+        (`tiled` is then read; a copy with a norm folded in needs rows normed without the norm's weight). The kernel
+        must serve the shape and, timed once per weight shape and row bucket against the vendor library's product of
+        the same rows (outside graph capture), be the faster of the two."""
         n, k = weight.shape
-        return bool(tiled is not None and weight.dtype == torch.bfloat16 and 16 < rows <= 64
-                    and self.lib.holon_gemm_rows_supported(rows, n // 2 if gated else n, k, int(gated)))
+        if not (tiled is not None and weight.dtype == torch.bfloat16 and 16 < rows <= 64
+                and self.lib.holon_gemm_rows_supported(rows, n // 2 if gated else n, k, int(gated))):
+            return False
+        key = ("rows", (n, k), rows <= 32, bool(gated))
+        use = self._mid_choice.get(key)
+        if use is None:
+            if torch.cuda.is_current_stream_capturing():
+                return False
+            use = self._mid_choice[key] = self._time_rows(rows, weight, tiled, gated)
+        return use == "rows"
+
+    def _rows_product(self, x, weight, tiled, gated, to_f32=False):
+        m, k = x.shape
+        n = weight.shape[0] // 2 if gated else weight.shape[0]
+        self._check_product("linear", x, weight, tiled)
+        y = torch.empty((m, n), dtype=torch.float32 if to_f32 else torch.bfloat16, device=x.device)
+        if gated:
+            self._call(self.lib.holon_gemm_rows_glu_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), m, n, k, self._stream())
+        else:
+            self._call(self.lib.holon_gemm_rows_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), m, n, k, int(to_f32),
+                       self._stream())
+        return y
+
+    def _time_rows(self, rows, weight, tiled, gated) -> str:
+        x = torch.randn(rows, weight.shape[1], device=weight.device).to(torch.bfloat16)
+        forms = {"rows": lambda: self._rows_product(x, weight, tiled, gated),
+                 "vendor": (lambda: self.silu_mul(self._vendor_product(x, weight))) if gated
+                 else (lambda: self._vendor_product(x, weight))}
+        took = {}
+        for name, fn in forms.items():
+            for _ in range(2):
+                fn()
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(6):
+                fn()
+            end.record()
+            end.synchronize()
+            took[name] = start.elapsed_time(end)
+        return "rows" if took["rows"] < took["vendor"] else "vendor"
 
     def linear_add(self, x, weight, tiled, residual, want_stats=False):
         """-> False when not fused; otherwise True, or with `want_stats` the partial sums of squares [N / 16, 16] of
@@ -331,11 +366,7 @@ class HipKernels:
         two_i = weight.shape[0]
         if row_scale is None and weight.shape[1] == k and x.dtype == torch.bfloat16 and x.is_contiguous() \
                 and two_i % 2 == 0 and self.serves_rows(m, weight, tiled, gated=True):
-            self._check_product("linear_silu_mul", x, weight, tiled)
-            y = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
-            self._call(self.lib.holon_gemm_rows_glu_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), m, two_i // 2, k,
-                       self._stream())
-            return y
+            return self._rows_product(x, weight, tiled, True)
         if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 1 <= m <= self.skinny_rows
                 and two_i % 32 == 0 and k % 128 == 0 and k >= 256 and weight.shape[1] == k and x.is_contiguous()):
             return None

@@ -19,6 +19,7 @@ SHORT = (("_Z18gemm_skinny_kernelILi", "gemm_skinny<"), ("_Z22gemm_skinny_glu_ke
          ("_Z24attn_prefill_wide_kernelILi", "attn_prefill_wide<"), ("_Z23attn_prefill_lds_kernelILi", "attn_prefill_lds<"),
          ("_Z17attn_merge_kernel", "attn_merge"), ("_Z13argmax_kernel", "argmax"), ("_Z16embedding_kernel", "embedding"),
          ("_Z15gemm_f32_kernel", "gemm_f32"), ("_Z13sample_kernel", "sample"),
+         ("_ZN12_GLOBAL__N_116gemm_rows_kernelILi", "gemm_rows<"),
          ("_Z19silu_mul_vec_kernel", "silu_mul_vec"), ("Cijk_Alik_Bljk_BBS_BH_Bias_HA_S_SAV_UserArgs_", "hipBLASLt "),
          ("Custom_Cijk_Alik_Bljk_BBS_BH_Bias_HA_S_SAV_NTD_SK3_UserArgs_", "hipBLASLt custom "))
 

@@ -363,6 +363,10 @@ def test_product_for_17_to_64_rows_over_many_tiles(hip):
     for m, k, n in ((17, 256, 16384), (64, 4096, 24576), (33, 1024, 16512), (48, 512, 65536), (64, 768, 65664), (20, 256, 131072)):
         x, w = _randn(m, k, dtype=bf, seed=80), _randn(n, k, dtype=bf, seed=81, scale=0.05)
         tiled = hip.tile_weight(w)
+        hip.serves_rows(m, w, tiled)                                                   # times the two products once ...
+        key = ("rows", (n, k), m <= 32, False)
+        assert hip._mid_choice[key] in ("rows", "vendor")
+        hip._mid_choice[key] = "rows"                                                  # ... here the kernel is what is tested
         assert hip.serves_rows(m, w, tiled) and not hip.serves_rows(16, w, tiled) and not hip.serves_rows(65, w, tiled)
         want = x.double() @ w.double().T
         got = hip.linear(x, w, None, tiled)
@@ -374,6 +378,7 @@ def test_product_for_17_to_64_rows_over_many_tiles(hip):
     for m, k, inter in ((64, 4096, 12288), (17, 256, 8192), (40, 1024, 8320)):
         x, w = _randn(m, k, dtype=bf, seed=82), _randn(2 * inter, k, dtype=bf, seed=83, scale=0.05)
         tiled = hip.tile_weight(w)
+        hip._mid_choice[("rows", (2 * inter, k), m <= 32, True)] = "rows"
         assert hip.serves_rows(m, w, tiled, gated=True)
         exact = PLAIN.silu_mul(PLAIN.linear(x.double(), w.double()))
         got = hip.linear_silu_mul(x, w, tiled)
@@ -385,6 +390,7 @@ def test_product_for_17_to_64_rows_over_many_tiles(hip):
     assert not hip.serves_rows(32, w, tiled) and not hip.serves_rows(32, w, None)      # 256 tiles: the vendor library's
     w = _randn(16384, 384, dtype=bf, seed=85)
     assert not hip.serves_rows(32, w, hip.tile_weight(w))                              # K no multiple of 256
+    hip._mid_choice.clear()
 
 
 def test_vendor_product_forms_for_steps_of_17_to_64_rows(hip):
@@ -690,6 +696,7 @@ def test_kernels_refuse_what_they_do_not_serve(hip):
     w, other = _randn(512, 1024, dtype=bf, seed=1), _randn(256, 1024, dtype=bf, seed=2)
     tiled = hip.tile_weight(w)
     big = _randn(16384, 256, dtype=bf, seed=3)
+    hip._mid_choice[("rows", (16384, 256), True, False)] = "rows"
     for rows, weight in ((4, w), (32, big)):
         with pytest.raises(KernelError):
             hip.linear(torch.zeros(rows, weight.shape[1], dtype=bf), weight, None, hip.tile_weight(weight))   # rows on the CPU
@@ -701,3 +708,4 @@ def test_kernels_refuse_what_they_do_not_serve(hip):
         hip.linear_add(_randn(4, 1024, dtype=bf), w, hip.tile_weight(other), _randn(4, 512, dtype=bf))
     with pytest.raises(KernelError):
         hip.linear_add(_randn(4, 1024, dtype=bf), w, tiled, torch.zeros(4, 512, dtype=bf))   # residual on the CPU
+    hip._mid_choice.clear()
