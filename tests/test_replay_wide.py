@@ -116,13 +116,20 @@ def _wide_batch_trace(requests: dict[str, tuple[list[int], int]], budget: int) -
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_sixty_four_rows_decode_together_from_graphs(folder, dtype):
+@pytest.mark.parametrize("gated_product", ["rows", "vendor"])
+def test_sixty_four_rows_decode_together_from_graphs(folder, dtype, gated_product):
     """Decode steps of 64 rows shrinking to 7, replayed from graphs of every batch bucket on the way (all but the
-    first with padding rows) and of three length buckets (1,024, 2,048, 4,096): the vendor product for more
-    than 16 rows, the decode attention with 64 rows, the few-row kernels below. Every row's logits in every step
+    first with padding rows) and of three length buckets (1,024, 2,048, 4,096): the products for more than 16 rows
+    (the gated one once in the kernel that shares the rows through LDS, over the folded weights and rows normed
+    without the norm's weight, once in the vendor library's: which of the two a run takes is otherwise decided by
+    timing them), the decode attention with 64 rows, the few-row kernels below. Every row's logits in every step
     against the plain model."""
     from holon_amd.engine.loading import load_model
     from holon_amd.engine.replay import Replayer
+    from holon_amd.kernels import load_hip
+    shape = (2 * WIDE["intermediate_size"], WIDE["hidden_size"])
+    for few in (True, False):
+        load_hip()._mid_choice[("rows", shape, few, True)] = gated_product
     requests = _wide_batch_requests()
     trace = _wide_batch_trace(requests, 2304)
     loaded = load_model(folder, device="cuda", dtype=dtype, page_size=16, max_seqs=64, max_model_len=2304,
@@ -136,6 +143,7 @@ def test_sixty_four_rows_decode_together_from_graphs(folder, dtype):
     _check(folder, dtype, {rid: ids for rid, (ids, _) in requests.items()}, got, f"wide {dtype} 64 rows")
     rep.cache.check()
     assert all(g.pool.free == g.pool.usable for g in rep.cache.groups)
+    load_hip()._mid_choice.clear()
 
 
 def test_engine_at_the_wide_sizes_with_everything_on(folder):
