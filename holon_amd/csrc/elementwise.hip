@@ -81,18 +81,29 @@ extern "C" int holon_embedding(const int32_t* ids, const int32_t* take_slot, con
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// One wave per row. Pass 1: (residual += x, rounded) and the sum of squares; pass 2: scale and weight.
+// What is added to the residual rows when it comes as float32 sums over shares of K, parts [splits, rows, dim] (a
+// product whose blocks split K): the shares added up in order, rounded to T.
+template <typename T>
+__device__ __forceinline__ float sum_of_parts(const float* __restrict__ parts, int splits, int64_t share, int64_t at) {
+  float sum = parts[at];
+  for (int s = 1; s < splits; ++s) sum += parts[s * share + at];
+  return Elem<T>::round(sum);
+}
+
+// One wave per row. Pass 1: (residual += x, rounded) and the sum of squares; pass 2: scale and weight. With `parts`,
+// x is the sum of the parts.
 template <typename T, bool ADD>
 __global__ void rmsnorm_kernel(const T* __restrict__ x, T* __restrict__ residual, const T* __restrict__ weight,
-                               T* __restrict__ y, int64_t rows, int dim, float eps) {
+                               T* __restrict__ y, int64_t rows, int dim, float eps,
+                               const float* __restrict__ parts = nullptr, int splits = 0) {
   const int lane = threadIdx.x % WAVE;
   const int64_t row = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
   if (row >= rows) return;
-  const T* xr = x + row * dim;
+  const T* xr = parts ? nullptr : x + row * dim;
   T* rr = ADD ? residual + row * dim : nullptr;
   float ss = 0.f;
   for (int i = lane; i < dim; i += WAVE) {
-    float v = Elem<T>::load(xr[i]);
+    float v = parts ? sum_of_parts<T>(parts, splits, rows * dim, row * dim + i) : Elem<T>::load(xr[i]);
     if (ADD) {
       v = Elem<T>::round(Elem<T>::load(rr[i]) + v);
       rr[i] = Elem<T>::store(v);
@@ -172,6 +183,77 @@ __global__ void __launch_bounds__(256) rmsnorm_row_kernel(const T* __restrict__ 
   }
 }
 
+// The residual add + norm over a product that comes as float32 sums over shares of K, parts [splits, rows, dim]:
+// residual += round(parts[0] + parts[1] + ...), y = rmsnorm(residual), bfloat16. One block of 1,024 threads per row,
+// eight values a thread (dim <= 8,192), so that all of a thread's loads, eight shares at a time, are under way at once:
+// the parts come from memory (other compute dies wrote them), and with four times the values a thread and the shares
+// read one after the other the kernel took 11 us where this takes half.
+__global__ void __launch_bounds__(1024) rmsnorm_parts_kernel(const float* __restrict__ parts, int splits,
+                                                             bf16_t* __restrict__ residual,
+                                                             const bf16_t* __restrict__ weight, bf16_t* __restrict__ y,
+                                                             int dim, float eps) {
+  using E = Elem<bf16_t>;
+  constexpr int V = 8, AT_ONCE = 8;
+  __shared__ float part[16];
+  const int64_t row = blockIdx.x;
+  const int v = threadIdx.x;
+  const bool live = v < dim / V;
+  float vals[V];
+  float ss = 0.f;
+  uint4 wraw;
+  if (live) {
+    wraw = reinterpret_cast<const uint4*>(weight)[v];
+    uint4* rr = reinterpret_cast<uint4*>(residual + row * dim) + v;
+    uint4 rraw = *rr;
+    const float* pr = parts + (row * dim + (int64_t)v * V);
+    const int64_t share = (int64_t)gridDim.x * dim;
+    float sum[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) sum[j] = 0.f;
+    for (int s0 = 0; s0 < splits; s0 += AT_ONCE) {
+      float4 p[AT_ONCE][V / 4];
+#pragma unroll
+      for (int u = 0; u < AT_ONCE; ++u)
+#pragma unroll
+        for (int j = 0; j < V / 4; ++j)
+          p[u][j] = s0 + u < splits ? *reinterpret_cast<const float4*>(pr + (s0 + u) * share + 4 * j)
+                                    : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int u = 0; u < AT_ONCE; ++u)
+#pragma unroll
+        for (int j = 0; j < V / 4; ++j) {
+          sum[4 * j] += p[u][j].x;
+          sum[4 * j + 1] += p[u][j].y;
+          sum[4 * j + 2] += p[u][j].z;
+          sum[4 * j + 3] += p[u][j].w;
+        }
+    }
+    bf16_t* re = reinterpret_cast<bf16_t*>(&rraw);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      vals[j] = E::round(E::load(re[j]) + E::round(sum[j]));
+      re[j] = E::store(vals[j]);
+      ss += vals[j] * vals[j];
+    }
+    *rr = rraw;
+  }
+  ss = wave_sum(ss);
+  if (threadIdx.x % WAVE == 0) part[threadIdx.x / WAVE] = ss;
+  __syncthreads();
+  ss = 0.f;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) ss += part[w];
+  const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+  if (live) {
+    const bf16_t* we = reinterpret_cast<const bf16_t*>(&wraw);
+    uint4 out;
+    bf16_t* oe = reinterpret_cast<bf16_t*>(&out);
+#pragma unroll
+    for (int j = 0; j < V; ++j) oe[j] = E::store((vals[j] * inv) * E::load(we[j]));
+    reinterpret_cast<uint4*>(y + row * dim)[v] = out;
+  }
+}
+
 template <typename T, bool ADD>
 static bool launch_rmsnorm_rows(const void* x, void* residual, const void* weight, void* y, int64_t rows, int dim,
                                 float eps, hipStream_t s) {
@@ -217,6 +299,26 @@ extern "C" int holon_rmsnorm(const void* x, void* residual, const void* weight, 
     if (residual) RMS_LAUNCH(bf16_t, true); else RMS_LAUNCH(bf16_t, false);
   }
 #undef RMS_LAUNCH
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_rmsnorm_parts(const float* parts, int splits, void* residual, const void* weight, void* y,
+                                   int64_t rows, int dim, float eps, void* stream) {
+  HOLON_CHECK(rows >= 0 && rows <= 0x7fffffff && dim > 0 && splits >= 1 && parts && residual,
+              "rmsnorm of parts: bad sizes rows=%lld dim=%d splits=%d", (long long)rows, dim, splits);
+  if (rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const bool aligned = (((uintptr_t)parts | (uintptr_t)residual | (uintptr_t)weight | (uintptr_t)y) & 15) == 0;
+  if (dim % 8 == 0 && dim >= 1024 && dim <= 8192 && aligned) {
+    rmsnorm_parts_kernel<<<(unsigned)rows, 1024, 0, s>>>(parts, splits, (bf16_t*)residual, (const bf16_t*)weight,
+                                                         (bf16_t*)y, dim, eps);
+  } else {                 // narrow, odd or very wide rows: one wave per row
+    const int waves = 4;
+    const unsigned grid = (unsigned)((rows + waves - 1) / waves);
+    rmsnorm_kernel<bf16_t, true><<<grid, waves * WAVE, 0, s>>>(nullptr, (bf16_t*)residual, (const bf16_t*)weight,
+                                                               (bf16_t*)y, rows, dim, eps, parts, splits);
+  }
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -6,8 +6,12 @@
 // KC columns of all rows is copied in once per block (double buffered, the next chunk's copy under way while this one
 // is used), each wave streams the weights of its own tile (from the tiled copy: a contiguous kilobyte a product) for
 // the next chunk while it multiplies this one, and reads its activations as B operands from LDS. A wave sums its tile
-// over all of K in order, so a result depends on nothing but the operands. Blocks do not split K: the kernel is for
-// weights with tiles enough to fill the GPU (the host refuses others, which stay with the vendor library).
+// over all of K in order, so a result depends on nothing but the operands.
+//
+// Weights with tiles enough to fill the GPU (a gated feed-forward's first product, the head) are served whole. Narrow
+// ones (a few hundred tiles: q/k/v, output and down projections) have K split over blocks as well (grid y): every
+// block writes the float32 sums of its share of K, [splits, M, N], and the reader adds them up in split order (the
+// residual add + norm kernel does so as it reads; `holon_sum_parts` for anyone else), so no block waits for another.
 //
 // v_mfma_f32_16x16x32_bf16 with the weights as A and MT tiles of 16 tokens as B, as in the few-row kernel.
 #include "common.h"
@@ -19,7 +23,8 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 namespace {
 // OUT: 0 bfloat16, 1 float32 of the values rounded to bfloat16 (the product in the operands' type, cast up),
 //      2 the gated form, bfloat16 round(silu(round(gate))) * round(up): the first half of a block's waves own gate
-//      tiles, the second half the up tiles of the same columns (I / 16 tiles further on), and the halves meet in LDS.
+//      tiles, the second half the up tiles of the same columns (I / 16 tiles further on), and the halves meet in LDS,
+//      3 float32 sums over this block's share of K (block y of gridDim.y), unrounded, to y[blockIdx.y][M][N].
 template <int MT, int WAVES, int KC, int OUT>
 __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(const bf16_t* __restrict__ x,
                                                                const bf16_t* __restrict__ w, void* __restrict__ y,
@@ -66,17 +71,18 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(const bf16_t* __r
       if (q < PIECES) *reinterpret_cast<bf16x8_t*>(&xs[buf][row * PITCH + col]) = xr[i];
     }
   };
-  const int chunks = K / KC;
-  load_w(0, wcur);
-  load_x(0);
+  const int chunks = K / KC / (int)gridDim.y;              // this block's share of K (all of it unless OUT == 3)
+  const int first = (int)blockIdx.y * chunks;
+  load_w(first, wcur);
+  load_x(first);
   store_x(0);
   __syncthreads();
   for (int ch = 0; ch < chunks; ++ch) {
     const int buf = ch & 1;
     const bool more = ch + 1 < chunks;                      // (uniform)
     if (more) {
-      load_w(ch + 1, wnext);
-      load_x(ch + 1);
+      load_w(first + ch + 1, wnext);
+      load_x(first + ch + 1);
     }
 #pragma unroll
     for (int s = 0; s < STEPS; ++s)
@@ -107,7 +113,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(const bf16_t* __r
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + c;
     if (m >= M) continue;
-    if constexpr (OUT == 1) {
+    if constexpr (OUT == 3) {
+      *reinterpret_cast<f32x4_t*>((float*)y + ((int64_t)blockIdx.y * M + m) * N + col_tile * 16 + 4 * g) = acc[t];
+    } else if constexpr (OUT == 1) {
       f32x4_t o;
 #pragma unroll
       for (int r = 0; r < 4; ++r) o[r] = bf16_to_float(float_to_bf16(acc[t][r]));
@@ -136,8 +144,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(const bf16_t* __r
 constexpr int ROWS_MIN_TILES = 1024;   // tiles (gated: tile pairs times two) from which the kernel fills the GPU
 
 template <int WAVES, int KC, int OUT>
-void launch_rows(const void* x, const void* w, void* y, int M, int N, int K, hipStream_t s) {
-  const dim3 grid(N / 16 / (OUT == 2 ? WAVES / 2 : WAVES)), block(WAVES * 64);
+void launch_rows(const void* x, const void* w, void* y, int M, int N, int K, hipStream_t s, int splits = 1) {
+  const dim3 grid(N / 16 / (OUT == 2 ? WAVES / 2 : WAVES), splits), block(WAVES * 64);
   const int mt = (M + 15) / 16;
 #define ROWS(MT) gemm_rows_kernel<MT, WAVES, KC, OUT><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, y, M, N, K)
   if (mt == 2) ROWS(2); else if (mt == 3) ROWS(3); else ROWS(4);
@@ -178,6 +186,65 @@ extern "C" int holon_gemm_rows_bf16(const void* x, const void* w_tiled, void* y,
 extern "C" int holon_gemm_rows_glu_bf16(const void* x, const void* w_tiled, void* y, int M, int I, int K, void* stream) {
   HOLON_CHECK(holon_gemm_rows_supported(M, I, K, 1), "gated gemm (17 to 64 rows): M=%d I=%d K=%d not served", M, I, K);
   launch_rows<4, 128, 2>(x, w_tiled, y, M, I, K, (hipStream_t)stream);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+namespace {
+constexpr int PARTS_KC = 128;          // columns of K a chunk of the split form holds
+constexpr int PARTS_MAX_SPLITS = 16;
+constexpr int PARTS_WAVES = 4;         // eight were slower at every shape measured
+
+// y[i] = round(parts[0][i] + parts[1][i] + ...) in split order, four values a thread.
+__global__ void sum_parts_kernel(const float* __restrict__ parts, bf16_t* __restrict__ y, int splits, int64_t count) {
+  const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i >= count) return;
+  f32x4_t sum = *reinterpret_cast<const f32x4_t*>(parts + i);
+  for (int s = 1; s < splits; ++s) sum += *reinterpret_cast<const f32x4_t*>(parts + (int64_t)s * count + i);
+  ushort4 o;
+  bf16_t* oe = reinterpret_cast<bf16_t*>(&o);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) oe[r] = float_to_bf16(sum[r]);
+  *reinterpret_cast<ushort4*>(y + i) = o;
+}
+}  // namespace
+
+// Whether holon_gemm_rows_parts_bf16 serves this product with K cut into `splits` shares (blocks of four waves, each
+// with a tile of 16 columns of its own).
+extern "C" int holon_gemm_rows_parts_supported(int M, int N, int K, int splits) {
+  return M > 16 && M <= 64 && N % 16 == 0 && (N / 16) % PARTS_WAVES == 0 && splits >= 1 &&
+         splits <= PARTS_MAX_SPLITS && K > 0 && K % (PARTS_KC * splits) == 0;
+}
+
+// How many shares of K serve a narrow weight best: measured on MI355X, eight where that gives at most 1,024 blocks of
+// four waves (4096 x 4096 at 64 rows: 9.4 us against the vendor library's 12.4; 4096 x 12288: 20.8 against 27.5;
+// 5120 x 25600: 60 against 78), four for wider weights; 0 when the shape is not served or K has no such shares.
+extern "C" int holon_gemm_rows_splits(int M, int N, int K) {
+  if (N % 16 || K <= 0) return 0;
+  int splits = N / 16 <= 512 ? 8 : 4;
+  while (splits > 1 && K % (PARTS_KC * splits)) splits /= 2;
+  return splits > 1 && holon_gemm_rows_parts_supported(M, N, K, splits) ? splits : 0;
+}
+
+// parts[s][M][N] (float32) = x[:, share s of K] w[:, share s of K]^T over tiled weights, 17 <= M <= 64: the product is
+// the sum of the parts in order, which the reader takes (holon_rmsnorm_parts, holon_sum_parts).
+extern "C" int holon_gemm_rows_parts_bf16(const void* x, const void* w_tiled, void* parts, int M, int N, int K,
+                                          int splits, void* stream) {
+  HOLON_CHECK(holon_gemm_rows_parts_supported(M, N, K, splits),
+              "gemm in parts (17 to 64 rows): M=%d N=%d K=%d splits=%d not served", M, N, K, splits);
+  launch_rows<PARTS_WAVES, PARTS_KC, 3>(x, w_tiled, parts, M, N, K, (hipStream_t)stream, splits);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+// y[count] (bfloat16) = the parts [splits, count] summed in order in float32, rounded once. count % 4 == 0.
+extern "C" int holon_sum_parts(const void* parts, void* y, int splits, int64_t count, void* stream) {
+  HOLON_CHECK(splits >= 1 && count >= 0 && count % 4 == 0, "sum of parts: splits=%d count=%lld", splits, (long long)count);
+  if (count == 0) return 0;
+  const int threads = 256;
+  const int64_t blocks = (count / 4 + threads - 1) / threads;
+  HOLON_CHECK(blocks <= 0x7fffffff, "sum of parts: %lld values are too many", (long long)count);
+  sum_parts_kernel<<<(unsigned)blocks, threads, 0, (hipStream_t)stream>>>((const float*)parts, (bf16_t*)y, splits, count);
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -20,6 +20,10 @@ int holon_row_sumsq(const void* x, float* stats, int rows, int dim, int dtype, v
 // y = rmsnorm(x) over rows of `dim`; with `residual`: residual += x (rounded), y = rmsnorm(residual).
 int holon_rmsnorm(const void* x, void* residual, const void* weight, void* y, int64_t rows, int dim, float eps,
                   int dtype, void* stream);
+// The same with what is added given as float32 sums over shares of K, parts [splits, rows, dim]: residual +=
+// round(parts[0] + parts[1] + ...), y = rmsnorm(residual); residual, weight and y bfloat16.
+int holon_rmsnorm_parts(const float* parts, int splits, void* residual, const void* weight, void* y, int64_t rows,
+                        int dim, float eps, void* stream);
 int holon_silu_mul(const void* gate_up, void* out, int64_t tokens, int inter, int dtype, void* stream);
 // Per (token, head): optional rmsnorm over head_dim, optional half-split rotation with table[pos] = cos|sin, then
 // q -> q_out [T, heads, D]; k, v -> the paged cache (pages == NULL: only q heads are processed).
@@ -91,6 +95,16 @@ int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int
 int holon_gemm_rows_supported(int M, int N, int K, int gated);
 int holon_gemm_rows_bf16(const void* x, const void* w_tiled, void* y, int M, int N, int K, int out_f32, void* stream);
 int holon_gemm_rows_glu_bf16(const void* x, const void* w_tiled, void* y, int M, int I, int K, void* stream);
+// The same for narrow weights (a few hundred tiles), with K cut into `splits` shares over the grid as well: blocks of
+// four waves, N / 16 a multiple of 4, K a multiple of 128 * splits, splits <= 16. parts [splits, M, N]
+// float32 holds each share's sums; the product is their sum in order (holon_sum_parts rounds it to bfloat16;
+// holon_rmsnorm_parts, the residual add + norm, reads them itself). holon_gemm_rows_splits: the number of shares that
+// serves this shape best (0: none does).
+int holon_gemm_rows_splits(int M, int N, int K);
+int holon_gemm_rows_parts_supported(int M, int N, int K, int splits);
+int holon_gemm_rows_parts_bf16(const void* x, const void* w_tiled, void* parts, int M, int N, int K, int splits,
+                               void* stream);
+int holon_sum_parts(const void* parts, void* y, int splits, int64_t count, void* stream);
 // y[M, N] = x[M, K] w[N, K]^T, all float32, true 32-bit products and sums in an order that depends on K alone: a row's
 // result is bit for bit the same whatever other rows are in the call.
 int holon_gemm_f32(const void* x, const void* w, void* y, int M, int N, int K, void* stream);

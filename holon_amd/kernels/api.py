@@ -61,7 +61,9 @@ class Kernels(Protocol):
         """x [..., dim] contiguous -> a new tensor; x is not modified."""
 
     def add_rmsnorm(self, x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
-        """residual += x in place (sum rounded to dtype), returns rmsnorm(residual) as a new tensor."""
+        """residual += x in place (sum rounded to dtype), returns rmsnorm(residual) as a new tensor. `x` may be what
+        `linear_parts` returned, float32 [S, *residual.shape]: what is added is then the parts' sum in order, rounded
+        to the residual's dtype first (the product that `linear` would have returned)."""
 
     def linear(self, x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None = None,
                tiled: torch.Tensor | None = None, row_scale: tuple[torch.Tensor, float] | None = None) -> torch.Tensor:
@@ -82,6 +84,16 @@ class Kernels(Protocol):
         kernels' (17 to 64): a caller whose tiled copy has a norm folded in then passes rows normed without the
         norm's weight."""
         return False
+
+    def linear_parts(self, x: torch.Tensor, weight: torch.Tensor, tiled: torch.Tensor | None) -> torch.Tensor | None:
+        """linear(x, weight) as float32 sums over S shares of K, [S, T, N], for a reader that adds them up itself
+        (`add_rmsnorm`; `sum_parts` for anyone else): their sum in order, rounded to x's dtype, is the product. None
+        when this step is not served that way (then nothing was done); a kernel set serves it only where that is
+        faster than `linear` even with the reader's extra reads."""
+        return None
+
+    def sum_parts(self, parts: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+        """float32 [S, ...] -> [...] in `dtype`: the parts added up in order, rounded once."""
 
     def linear_add(self, x: torch.Tensor, weight: torch.Tensor, tiled: torch.Tensor | None, residual: torch.Tensor,
                    want_stats: bool = False) -> "bool | torch.Tensor":

@@ -72,6 +72,11 @@ class HipKernels:
             "holon_gemm_rows_supported": [_I, _I, _I, _I],
             "holon_gemm_rows_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
             "holon_gemm_rows_glu_bf16": [_P, _P, _P, _I, _I, _I, _P],
+            "holon_gemm_rows_splits": [_I, _I, _I],
+            "holon_gemm_rows_parts_supported": [_I, _I, _I, _I],
+            "holon_gemm_rows_parts_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
+            "holon_sum_parts": [_P, _P, _I, _L, _P],
+            "holon_rmsnorm_parts": [_P, _I, _P, _P, _P, _L, _I, _F, _P],
             "holon_gemm_skinny_scaled_bf16": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _F, _P],
             "holon_gemm_f32": [_P, _P, _P, _I, _I, _I, _P],
             "holon_gemm_skinny_add_bf16": [_P, _P, _P, _I, _I, _I, _P, _P],
@@ -165,6 +170,18 @@ class HipKernels:
         return y
 
     def add_rmsnorm(self, x, residual, weight, eps):
+        if x.dtype == torch.float32 and residual.dtype == torch.bfloat16:     # a product as sums over shares of K
+            self._check(x, "add_rmsnorm parts")
+            self._check(residual, "add_rmsnorm residual")
+            self._check(weight, "add_rmsnorm weight", torch.bfloat16)
+            dim = residual.shape[-1]
+            if x.dim() != residual.dim() + 1 or x.shape[1:] != residual.shape or weight.shape != (dim,):
+                raise KernelError(f"add_rmsnorm: parts {tuple(x.shape)} for rows {tuple(residual.shape)}, "
+                                  f"weight {tuple(weight.shape)}")
+            y = torch.empty_like(residual)
+            self._call(self.lib.holon_rmsnorm_parts, x.data_ptr(), x.shape[0], residual.data_ptr(), weight.data_ptr(),
+                       y.data_ptr(), residual.numel() // dim, dim, float(eps), self._stream())
+            return y
         self._check(x, "add_rmsnorm x")
         self._check(residual, "add_rmsnorm residual", x.dtype)
         self._check(weight, "add_rmsnorm weight", x.dtype)
@@ -322,6 +339,74 @@ class HipKernels:
         else:
             self._call(self.lib.holon_gemm_rows_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), m, n, k, int(to_f32),
                        self._stream())
+        return y
+
+    def linear_parts(self, x, weight, tiled):
+        """-> float32 [splits, M, N], the product over each share of K, when that kernel serves this step (17 to 64
+        bfloat16 rows over a narrow tiled weight) and, timed once per weight shape and row bucket against the vendor
+        library's product (each with the add + norm that reads it), is the faster; None otherwise (nothing was done)."""
+        (m, k), n = x.shape, weight.shape[0]
+        if not (tiled is not None and 16 < m <= 64 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                and weight.shape[1] == k and x.is_contiguous()):
+            return None
+        splits = self.lib.holon_gemm_rows_splits(m, n, k)
+        if not splits:
+            return None
+        key = ("parts", (n, k), m <= 32)
+        use = self._mid_choice.get(key)
+        if use is None:
+            if torch.cuda.is_current_stream_capturing():
+                return None
+            use = self._mid_choice[key] = self._time_parts(x, weight, tiled, splits)
+        return self._rows_parts(x, weight, tiled, splits) if use == "parts" else None
+
+    def _rows_parts(self, x, weight, tiled, splits):
+        (m, k), n = x.shape, weight.shape[0]
+        self._check_product("linear in parts", x, weight, tiled)
+        if tiled is None or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or weight.shape[1] != k:
+            raise KernelError(f"linear in parts: bfloat16 rows {tuple(x.shape)} over a tiled bfloat16 weight "
+                              f"{tuple(weight.shape)} expected")
+        parts = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+        self._call(self.lib.holon_gemm_rows_parts_bf16, x.data_ptr(), tiled.data_ptr(), parts.data_ptr(), m, n, k,
+                   splits, self._stream())
+        return parts
+
+    def _time_parts(self, x, weight, tiled, splits) -> str:
+        """Each way together with the residual add + norm that reads the product (reading parts costs that kernel a
+        few microseconds, which the product must win back). Both are shorter than a launch from here takes, so they
+        are timed as recorded graphs of several calls."""
+        n = weight.shape[0]
+        residual = torch.zeros((x.shape[0], n), dtype=torch.bfloat16, device=x.device)
+        ones = torch.ones(n, dtype=torch.bfloat16, device=x.device)
+        took = {}
+        for name, fn in (("parts", lambda: self._rows_parts(x, weight, tiled, splits)),
+                         ("vendor", lambda: self._vendor_product(x, weight))):
+            self.add_rmsnorm(fn(), residual, ones, 1e-6)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(8):
+                    keep = self.add_rmsnorm(fn(), residual, ones, 1e-6)
+            graph.replay()
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(3):
+                graph.replay()
+            end.record()
+            end.synchronize()
+            took[name] = start.elapsed_time(end)
+            del graph, keep
+        return "parts" if took["parts"] < 0.97 * took["vendor"] else "vendor"
+
+    def sum_parts(self, parts, dtype=torch.bfloat16):
+        """[splits, ...] float32 -> bfloat16 [...]: the parts added up in order, rounded once."""
+        self._check(parts, "sum_parts", torch.float32)
+        if dtype != torch.bfloat16:
+            raise KernelError(f"sum_parts: partial sums are of bfloat16 products, not {dtype}")
+        y = torch.empty(parts.shape[1:], dtype=torch.bfloat16, device=parts.device)
+        if y.numel() % 4:
+            raise KernelError(f"sum_parts: {y.numel()} values are no multiple of 4")
+        self._call(self.lib.holon_sum_parts, parts.data_ptr(), y.data_ptr(), parts.shape[0], y.numel(), self._stream())
         return y
 
     def _time_rows(self, rows, weight, tiled, gated) -> str:

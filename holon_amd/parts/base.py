@@ -49,15 +49,38 @@ class SlotState:
     dtype: torch.dtype | None = None
 
 
+class PartialSums:
+    """A product [T, N] that exists as float32 sums over shares of its inner dimension, `parts` [S, T, N]: the product
+    is their sum in order, rounded once to the activation dtype. A projection may hand this out instead of a tensor,
+    but only to a caller that passed it the residual stream (so one that goes on to add the product into the stream):
+    a norm's `add` reads the parts itself; anyone else calls `value()`."""
+
+    def __init__(self, parts: torch.Tensor, kernels: Any, dtype: torch.dtype) -> None:
+        self.parts, self.kernels, self.dtype = parts, kernels, dtype
+
+    @property
+    def shape(self) -> torch.Size:
+        return self.parts.shape[1:]
+
+    def value(self) -> torch.Tensor:
+        return self.kernels.sum_parts(self.parts, self.dtype)
+
+    def index_select(self, dim: int, index: torch.Tensor) -> "PartialSums":
+        """Rows of the product (dim 0 alone)."""
+        if dim != 0:
+            raise ValueError("PartialSums.index_select: rows only (dim 0)")
+        return PartialSums(self.parts.index_select(1, index), self.kernels, self.dtype)
+
+
 @dataclasses.dataclass
 class Stream:
     """The residual stream between blocks: `h` [T, hidden], updated in place; `delta`, a term not yet added to it (the
-    next norm's kernel fuses the add) or None; `stats`, what the kernel that last wrote `h` left about its rows for a
-    norm that follows (partial sums of squares, see the kernel contract) or None when nothing is known. Whoever
-    changes `h` sets `stats` anew or to None."""
+    next norm's kernel fuses the add; a tensor or `PartialSums`) or None; `stats`, what the kernel that last wrote `h`
+    left about its rows for a norm that follows (partial sums of squares, see the kernel contract) or None when
+    nothing is known. Whoever changes `h` sets `stats` anew or to None."""
 
     h: torch.Tensor
-    delta: torch.Tensor | None = None
+    delta: "torch.Tensor | PartialSums | None" = None
     stats: torch.Tensor | None = None
 
 

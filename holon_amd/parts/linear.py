@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import Build, Part, Stream
+from .base import Build, PartialSums, Part, Stream
 from .norms import Normed, RMSNorm
 
 
@@ -54,10 +54,11 @@ class Linear(Part):
         return stats, x.norm.eps
 
     def forward(self, x: torch.Tensor | Normed, out_dtype: torch.dtype | None = None, residual: Stream | None = None
-                ) -> torch.Tensor | None:
+                ) -> "torch.Tensor | PartialSums | None":
         """x W^T. With `residual`, the product is added into the stream's rows in place when one kernel can do both
         (steps of few rows), which also leaves the rows' statistics there, and None is returned; otherwise the
-        product is returned and the add is the caller's."""
+        product is returned and the add is the caller's. It may then come as `PartialSums` (a narrow weight at 17 to
+        64 rows, K split over blocks), which the norm that adds it reads as they are."""
         if isinstance(x, Normed):
             if self.folds(x):
                 return self.kernels.linear(x.h, self.weight, out_dtype, self.tiled, row_scale=self.row_scale(x))
@@ -70,6 +71,9 @@ class Linear(Part):
             if done is not False:
                 residual.stats = done if isinstance(done, torch.Tensor) else None
                 return None
+            parts = self.kernels.linear_parts(x, self.weight, tiled)
+            if parts is not None:
+                return PartialSums(parts, self.kernels, x.dtype)
         return self.kernels.linear(x, self.weight, out_dtype, tiled)
 
     __call__ = forward

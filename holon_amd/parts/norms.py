@@ -4,7 +4,12 @@ from __future__ import annotations
 import torch
 
 from ..registry import register_part
-from .base import Build, Part
+from .base import Build, PartialSums, Part
+
+
+def _term(x: "torch.Tensor | PartialSums") -> torch.Tensor:
+    """What the add + norm kernel is given: a tensor, or the parts of a product that came as partial sums."""
+    return x.parts if isinstance(x, PartialSums) else x
 
 
 class Normed:
@@ -15,7 +20,7 @@ class Normed:
     `stats`: what the kernel that last wrote `h` left about its rows (partial sums of squares), or None."""
 
     def __init__(self, norm: "RMSNorm", h: torch.Tensor, stats: torch.Tensor | None = None,
-                 delta: torch.Tensor | None = None) -> None:
+                 delta: "torch.Tensor | PartialSums | None" = None) -> None:
         self.norm, self.h, self.stats, self.delta = norm, h, stats, delta
         self._value: torch.Tensor | None = None
         self._unit: torch.Tensor | None = None
@@ -57,9 +62,9 @@ class RMSNorm(Part):
 
     __call__ = forward
 
-    def add(self, x: torch.Tensor, residual: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    def add(self, x: "torch.Tensor | PartialSums", residual: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         """(norm(residual + x), residual + x); the sum replaces `residual` in place."""
-        return self.kernels.add_rmsnorm(x, residual, self.weight, self.eps), residual
+        return self.kernels.add_rmsnorm(_term(x), residual, self.weight, self.eps), residual
 
     def defer(self, h: torch.Tensor, stats: torch.Tensor | None = None, delta: torch.Tensor | None = None) -> Normed:
         """norm(h), or norm(h + delta) with the sum replacing `h`, for a reader that may do the norm, or the
@@ -72,7 +77,7 @@ class RMSNorm(Part):
             self._ones = torch.ones_like(self.weight)
         if delta is None:
             return self.kernels.rmsnorm(h, self._ones, self.eps)
-        return self.kernels.add_rmsnorm(delta, h, self._ones, self.eps)
+        return self.kernels.add_rmsnorm(_term(delta), h, self._ones, self.eps)
 
     _ones: torch.Tensor | None = None
 

@@ -43,6 +43,8 @@ class TorchKernels:
     name = "torch-plain"
 
     fold_norms = False       # a test may switch the folded-norm path on: the twin then stands in for the tiled copy
+    split_products = 0       # a test may set a number of shares: steps of 17 to 64 rows then get their products that
+                             # are added to the residual stream as partial sums over that many shares of K
 
     def embedding(self, ids, table, take=None, want_stats=False):
         if take is not None:
@@ -62,6 +64,8 @@ class TorchKernels:
         return _rmsnorm(x, weight, eps)
 
     def add_rmsnorm(self, x, residual, weight, eps):
+        if x.dim() == residual.dim() + 1:                    # partial sums of a product: added up in order, rounded
+            x = self.sum_parts(x, residual.dtype)
         residual.add_(x)
         return _rmsnorm(residual, weight, eps)
 
@@ -92,7 +96,23 @@ class TorchKernels:
             weight = tiled                                   # (folded or not: what the caller's rows were prepared for)
         return (_up(x) @ _up(weight).T).to(x.dtype).to(out_dtype or x.dtype)      # rounded to x's dtype, then cast
 
+    def linear_parts(self, x, weight, tiled):
+        s, k = self.split_products, x.shape[1]
+        if not s or not 16 < x.shape[0] <= 64 or k % s:
+            return None
+        share = k // s
+        return torch.stack([_up(x[:, i * share:(i + 1) * share]).float() @ _up(weight[:, i * share:(i + 1) * share]).float().T
+                            for i in range(s)])
+
+    def sum_parts(self, parts, dtype):
+        total = parts[0].clone()
+        for part in parts[1:]:
+            total += part
+        return total.to(dtype)
+
     def linear_add(self, x, weight, tiled, residual, want_stats=False):
+        if self.split_products and 16 < x.shape[0] <= 64:
+            return False                                     # as the HIP kernels: not fused at these row counts
         residual.copy_((_up(residual) + _up(self.linear(x, weight))).to(residual.dtype))
         if want_stats and self.fold_norms and residual.shape[0] <= 16:
             return self.row_sumsq(residual)

@@ -393,6 +393,64 @@ def test_product_for_17_to_64_rows_over_many_tiles(hip):
     hip._mid_choice.clear()
 
 
+def test_product_in_shares_of_k_for_narrow_weights(hip):
+    """Steps of 17 to 64 rows over narrow weights (a few hundred tiles: output and down projections) may have K split
+    over blocks: float32 sums of every share, which the residual add + norm kernel (or `sum_parts`) adds up in order.
+    Every share against float64 over its columns; the sum, rounded once, against the whole product; the norm that
+    reads the parts against the norm over their rounded sum (the residual rows bit for bit), in both of its kernels
+    (rows of 1,024 values and more, and narrower ones); a row's result whatever rows lie beside it; and the timed
+    choice."""
+    from holon_amd.kernels.hip import KernelError
+    bf = torch.bfloat16
+    for m, k, n in ((64, 4096, 4096), (17, 12288, 4096), (33, 1024, 5120), (48, 25600, 5120), (40, 512, 320), (64, 256, 64)):
+        x, w = _randn(m, k, dtype=bf, seed=90), _randn(n, k, dtype=bf, seed=91, scale=0.05)
+        tiled = hip.tile_weight(w)
+        splits = hip.lib.holon_gemm_rows_splits(m, n, k)
+        assert splits in (2, 4, 8) and k % (128 * splits) == 0, (m, k, n, splits)
+        parts = hip._rows_parts(x, w, tiled, splits)
+        assert parts.shape == (splits, m, n) and parts.dtype == torch.float32
+        share = k // splits
+        for s in range(splits):
+            want = x[:, s * share:(s + 1) * share].double() @ w[:, s * share:(s + 1) * share].double().T
+            assert H.op_budget_usage(parts[s], want, torch.float32, share) <= 1, (m, k, n, s)
+        total = hip.sum_parts(parts)
+        in_order = parts[0].clone()
+        for s in range(1, splits):
+            in_order += parts[s]
+        assert torch.equal(total, in_order.to(bf))
+        assert H.op_budget_usage(total, x.double() @ w.double().T, bf, k) <= 1
+        assert H.op_budget_usage(total, hip.linear(x, w).double(), bf, k) <= 1           # the vendor library's product
+        fewer = hip._rows_parts(x[3:21].contiguous(), w, tiled, splits) if m >= 21 else None
+        assert fewer is None or torch.equal(fewer, parts[:, 3:21])
+        weight, eps = _randn(n, dtype=bf, seed=92) + 1, 1e-5
+        res_a, res_b = _randn(m, n, dtype=bf, seed=93), _randn(m, n, dtype=bf, seed=93)
+        normed_a = hip.add_rmsnorm(parts, res_a, weight, eps)                             # reads the parts itself
+        normed_b = hip.add_rmsnorm(total, res_b, weight, eps)
+        assert torch.equal(res_a, res_b), (m, k, n)                                       # the same sums, bit for bit
+        assert H.op_budget_usage(normed_a, normed_b.double(), bf, 1) <= 1, (m, k, n)      # (squares summed in another order)
+        plain_res = _randn(m, n, dtype=bf, seed=93)
+        plain_normed = PLAIN.add_rmsnorm(parts, plain_res, weight, eps)                   # the twin takes parts as well
+        assert torch.equal(plain_res, res_a) and H.op_budget_usage(normed_a, plain_normed.double(), bf, 1) <= 1
+    x, w = _randn(32, 4096, dtype=bf, seed=94), _randn(4096, 4096, dtype=bf, seed=95, scale=0.05)
+    tiled = hip.tile_weight(w)
+    got = hip.linear_parts(x, w, tiled)                                                   # timed once, then kept
+    assert hip._mid_choice[("parts", (4096, 4096), True)] in ("parts", "vendor")
+    assert (got is None) == (hip._mid_choice[("parts", (4096, 4096), True)] == "vendor")
+    hip._mid_choice[("parts", (4096, 4096), True)] = "parts"
+    assert hip.linear_parts(x, w, tiled).shape == (8, 32, 4096)
+    assert hip.linear_parts(x[:16].contiguous(), w, tiled) is None and hip.linear_parts(x, w, None) is None
+    assert hip.linear_parts(_randn(32, 4096, dtype=torch.float32, seed=96), w.float(), tiled) is None          # float32 rows: not this path
+    w = _randn(4096, 4224, dtype=bf, seed=97)                                             # K = 33 x 128: no equal shares
+    assert hip.linear_parts(_randn(32, 4224, dtype=bf, seed=98), w, hip.tile_weight(w)) is None
+    with pytest.raises(KernelError):
+        hip._rows_parts(x, w[:, :4096].contiguous(), tiled, 3)                            # 4096 / 128 = 32 chunks, not by 3
+    with pytest.raises(KernelError):
+        hip._rows_parts(x.cpu(), w[:, :4096].contiguous(), tiled, 8)
+    with pytest.raises(KernelError):
+        hip.add_rmsnorm(torch.zeros(8, 32, 4000, device="cuda"), _randn(32, 4096, dtype=bf), _randn(4096, dtype=bf), 1e-5)
+    hip._mid_choice.clear()
+
+
 def test_vendor_product_forms_for_steps_of_17_to_64_rows(hip):
     """Steps of 17 to 64 bfloat16 rows take the vendor library's product in the faster of two forms, timed once per
     weight shape and row bucket: both are the product rounded once, whichever is kept, and the float32 output is the

@@ -10,7 +10,7 @@ import torch
 
 from holon_amd.engine.batch import StepRow
 from holon_amd.engine.loading import attach_cache, build_from_spec
-from holon_amd.parts import Build, Part, SlotState, Stream
+from holon_amd.parts import Build, Part, PartialSums, SlotState, Stream
 from holon_amd.parts.linear import Linear
 from holon_amd.registry import register_part, unregister_part
 from holon_amd.spec import LayerSpec, ModelSpec, PartRef, Run, in_order
@@ -409,7 +409,8 @@ def test_gqa_mixer_and_block_alone(device, dtype):
         cache.reserve(slot, 37)
         step, _ = runner.prepare([StepRow(slot, 0, [0] * 37, [])])
         out = block(Stream(x.clone().to(device)), step, model.sites[0])
-        stream = out.h.float() + (out.delta.float() if out.delta is not None else 0)    # the last add may be done or pending
+        delta = out.delta.value() if isinstance(out.delta, PartialSums) else out.delta
+        stream = out.h.float() + (delta.float() if delta is not None else 0)    # the last add may be done or pending
         def whole(xd, wd):
             a = xd + _plain_attention(plain.rms_norm(xd, wd["layers.0.input_norm.weight"], eps), pos, wd,
                                       "layers.0.mixer.", hq, hkv, d, eps, 1e6)[0]

@@ -128,18 +128,27 @@ def test_long_decoding_and_first_tokens(folders, name, dtype, device):
     rep.cache.check()
 
 
+@pytest.mark.parametrize("shares", [0, 2])
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "B-sharp"])
-def test_norms_folded_into_the_products_that_read_them(folders, name, dtype):
+def test_norms_folded_into_the_products_that_read_them(folders, name, dtype, shares):
     """Steps of few rows fold each block's norms into the q/k/v and the gate/up products (weights times the norm's
     weight, rows scaled by the norm's factor from statistics the kernel before left). On the CPU the kernel twin
     stands in for that path: the parts' logic of deferring a norm, passing the rows' statistics along the residual
-    stream and falling back for portions of more than 16 rows is what runs here. Same logits, every way of cutting."""
+    stream and falling back for portions of more than 16 rows is what runs here. Same logits, every way of cutting.
+    With `shares`, steps of 17 to 64 rows also get the products that are added to the residual stream (output and
+    down projection) as partial sums over shares of K, which the next norm's add, or the final one, takes as they
+    are."""
     from holon_amd.engine.loading import load_model
     from holon_amd.engine.replay import Replayer
     folder, requests = folders[name], _requests(name)
     kernels = TorchKernels()
     kernels.fold_norms = True
+    kernels.split_products = shares
+    taken = []
+    if shares:
+        plain_add = kernels.add_rmsnorm
+        kernels.add_rmsnorm = lambda x, residual, w, eps: (taken.append(x.dim() - residual.dim()), plain_add(x, residual, w, eps))[1]
     loaded = load_model(folder, device="cpu", dtype=dtype, kernels=kernels, page_size=MODELS[name][3], max_seqs=4,
                         max_model_len=512, max_step_tokens=512, cache_tokens=256)
     block = loaded.model.blocks[0]
@@ -151,6 +160,11 @@ def test_norms_folded_into_the_products_that_read_them(folders, name, dtype):
     _check(folder, dtype, requests, got, f"{name} {dtype} folded norms, portions")
     got = H.run_trace(rep, H.trace_mixed(requests, 2))
     _check(folder, dtype, requests, got, f"{name} {dtype} folded norms, mixed")
+    some = H.Trace()                               # a portion of which only some rows are wanted: rows are selected from
+    ids = requests["r1"]                           # the stream and from its pending term alike
+    some.add([("r1", 0, ids[:33], [3, 32])], end=["r1"])
+    _check(folder, dtype, requests, H.run_trace(rep, some), f"{name} {dtype} folded norms, some rows of a portion")
+    assert not shares or 1 in taken, taken                        # terms went through the norms' adds as partial sums
 
 
 @pytest.mark.parametrize("device", DEVICES)

@@ -116,20 +116,23 @@ def _wide_batch_trace(requests: dict[str, tuple[list[int], int]], budget: int) -
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("gated_product", ["rows", "vendor"])
-def test_sixty_four_rows_decode_together_from_graphs(folder, dtype, gated_product):
+@pytest.mark.parametrize("products", ["ours", "vendor"])
+def test_sixty_four_rows_decode_together_from_graphs(folder, dtype, products):
     """Decode steps of 64 rows shrinking to 7, replayed from graphs of every batch bucket on the way (all but the
-    first with padding rows) and of three length buckets (1,024, 2,048, 4,096): the products for more than 16 rows
-    (the gated one once in the kernel that shares the rows through LDS, over the folded weights and rows normed
-    without the norm's weight, once in the vendor library's: which of the two a run takes is otherwise decided by
-    timing them), the decode attention with 64 rows, the few-row kernels below. Every row's logits in every step
-    against the plain model."""
+    first with padding rows) and of three length buckets (1,024, 2,048, 4,096): the products for more than 16 rows,
+    the decode attention with 64 rows, the few-row kernels below. Once with the kernels of our own for 17 to 64 rows
+    (the gated product shares the rows through LDS and reads the folded weights over rows normed without the norm's
+    weight; the output and down projections split K over blocks and hand partial sums to the norm that adds them),
+    once with the vendor library's products: which a run takes is otherwise decided by timing them. Every row's
+    logits in every step against the plain model."""
     from holon_amd.engine.loading import load_model
     from holon_amd.engine.replay import Replayer
     from holon_amd.kernels import load_hip
-    shape = (2 * WIDE["intermediate_size"], WIDE["hidden_size"])
+    hidden, inter, wide = WIDE["hidden_size"], WIDE["intermediate_size"], WIDE["num_attention_heads"] * WIDE["head_dim"]
     for few in (True, False):
-        load_hip()._mid_choice[("rows", shape, few, True)] = gated_product
+        load_hip()._mid_choice[("rows", (2 * inter, hidden), few, True)] = "rows" if products == "ours" else "vendor"
+        for shape in ((hidden, wide), (hidden, inter)):
+            load_hip()._mid_choice[("parts", shape, few)] = "parts" if products == "ours" else "vendor"
     requests = _wide_batch_requests()
     trace = _wide_batch_trace(requests, 2304)
     loaded = load_model(folder, device="cuda", dtype=dtype, page_size=16, max_seqs=64, max_model_len=2304,
