@@ -91,7 +91,8 @@ def main(argv: list[str] | None = None) -> int:
     ap = argparse.ArgumentParser(prog="bench", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
-    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--warmup", type=int, default=24,
+                    help="untimed decode steps first (the first 15 or so after the prompts run 3%% slower)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"],
                     help="fewer layers than the configuration has (recorded in config)")
@@ -130,10 +131,13 @@ def main(argv: list[str] | None = None) -> int:
 
     def decode(batch: int, steps: int, warmup: int) -> tuple[float, float, float, int]:
         """(ms per decode step, mean context, median ms between two steps' ends, prompt length) for `batch` requests
-        whose contexts end at CONTEXT."""
-        start = CONTEXT - steps - warmup - 1
+        whose contexts end at CONTEXT. The requests go on for two steps after the timed ones, so that the host's work
+        for finished requests (not part of a decode step) falls outside the timed region."""
+        after = 2
+        start = CONTEXT - steps - warmup - 1 - after
         for _ in range(batch):
-            engine.add(torch.randint(0, c["vocab_size"], (start,), generator=g).tolist(), greedy(steps + warmup + 1))
+            engine.add(torch.randint(0, c["vocab_size"], (start,), generator=g).tolist(),
+                       greedy(steps + warmup + 1 + after))
         while engine.sched.waiting:                              # prompts, cut by the step budget
             engine.step()
         for _ in range(warmup):
