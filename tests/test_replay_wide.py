@@ -77,6 +77,33 @@ def test_wide_layers_every_way_of_cutting(folder, dtype):
     assert all(g.pool.free == g.pool.usable for g in rep.cache.groups)
 
 
+def test_portions_of_17_to_64_rows_with_some_rows_wanted_over_partial_sums(folder):
+    """Prompt portions of 40, 17 and 64 rows of which a few rows' logits are wanted, with the output and down
+    projections' products forced to come as partial sums over shares of K: the rows are then selected from the
+    residual stream and from its pending term, the last down projection's shares, alike."""
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    from holon_amd.kernels import load_hip
+    hidden, inter, wide = WIDE["hidden_size"], WIDE["intermediate_size"], WIDE["num_attention_heads"] * WIDE["head_dim"]
+    for few in (True, False):
+        for shape in ((hidden, wide), (hidden, inter)):
+            load_hip()._mid_choice[("parts", shape, few)] = "parts"
+    try:
+        ids = _requests()["r1"]                                           # 130 tokens
+        loaded = load_model(folder, device="cuda", dtype="bfloat16", page_size=16, max_seqs=4, max_model_len=512,
+                            max_step_tokens=512, cache_tokens=256)
+        trace = H.Trace()
+        trace.add([("r1", 0, ids[:40], [0, 39])])
+        trace.add([("r1", 40, ids[40:57], [16])])
+        trace.add([("r1", 57, ids[57:121], [3, 40, 63])])
+        trace.add([("r1", 121, ids[121:], [len(ids) - 122])], end=["r1"])  # nine rows: the few-row kernels
+        got = H.run_trace(Replayer(loaded), trace)
+        assert len(got) == 7
+        _check(folder, "bfloat16", {"r1": ids}, got, "wide bfloat16, some rows of portions over partial sums")
+    finally:
+        load_hip()._mid_choice.clear()
+
+
 def _wide_batch_requests() -> dict[str, tuple[list[int], int]]:
     """64 requests as (token ids, prompt length): the rest of each is decoded one token a step, all together. The
     decode counts make the batch shrink 64 -> 45 -> 30 -> 20 -> 12 -> 7 (padded to 48, 32, 24, 16, 8); request `long` goes from 2,042 to 2,062 tokens
