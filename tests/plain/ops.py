@@ -101,7 +101,7 @@ class TorchKernels:
         if not s or not 16 < x.shape[0] <= 64 or k % s:
             return None
         share = k // s
-        return torch.stack([_up(x[:, i * share:(i + 1) * share]).float() @ _up(weight[:, i * share:(i + 1) * share]).float().T
+        return torch.stack([_up(x[:, i * share:(i + 1) * share]) @ _up(weight[:, i * share:(i + 1) * share]).T
                             for i in range(s)])
 
     def sum_parts(self, parts, dtype):
