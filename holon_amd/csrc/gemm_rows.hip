@@ -182,10 +182,16 @@ extern "C" int holon_gemm_rows_bf16(const void* x, const void* w_tiled, void* y,
 }
 
 // y[M, I] = round(silu(round(x gate^T))) * round(x up^T) with w = [gate; up] ([2 I, K], tiled), 17 <= M <= 64: four waves
-// a block, two gate tiles and the two up tiles of the same columns.
+// a block, two gate tiles and the two up tiles of the same columns; where eight waves a block (four and four, chunks of
+// 256 columns: half the reads of the rows) still give a block to every compute unit, those. Measured over weights
+// streamed from memory, 51200 x 5120: 94 us at 32 rows and 104 at 64 against 104 and 119 with four waves (the vendor
+// library's product and SiLU-mul: 101 and 109); 24576 x 4096, where eight waves would leave 192 blocks: 39 and 46 us
+// with four (the vendor library's pair: 50 and 51).
+constexpr int ROWS_GLU_WIDE_BLOCKS = 256;
 extern "C" int holon_gemm_rows_glu_bf16(const void* x, const void* w_tiled, void* y, int M, int I, int K, void* stream) {
   HOLON_CHECK(holon_gemm_rows_supported(M, I, K, 1), "gated gemm (17 to 64 rows): M=%d I=%d K=%d not served", M, I, K);
-  launch_rows<4, 128, 2>(x, w_tiled, y, M, I, K, (hipStream_t)stream);
+  if (I / 16 / 4 >= ROWS_GLU_WIDE_BLOCKS) launch_rows<8, 256, 2>(x, w_tiled, y, M, I, K, (hipStream_t)stream);
+  else launch_rows<4, 128, 2>(x, w_tiled, y, M, I, K, (hipStream_t)stream);
   HOLON_LAUNCH_OK();
   return 0;
 }

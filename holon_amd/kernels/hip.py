@@ -6,6 +6,7 @@ from __future__ import annotations
 
 import ctypes
 import sys
+import weakref
 
 import torch
 
@@ -91,6 +92,7 @@ class HipKernels:
             fn = getattr(lib, name)
             fn.argtypes, fn.restype = args, _I
         self._mid_choice: dict[tuple, str] = {}    # (weight shape, at most 32 rows) -> the vendor product's faster form
+        self._tiled_weights: dict[tuple, list] = {}   # weight shape -> weak (weight, tiled copy) pairs, see _alike
 
     # -- plumbing -------------------------------------------------------------------------------------------------
     def _call(self, fn, *args) -> None:
@@ -211,7 +213,51 @@ class HipKernels:
         tiled = torch.empty_like(weight)
         self._call(self.lib.holon_tile_weight_bf16, weight.data_ptr(), tiled.data_ptr(), n, k, _ptr(scale),
                    self._stream())
+        known = self._tiled_weights.setdefault((n, k), [])
+        known[:] = [(w, t) for w, t in known if w() is not None and t() is not None and w() is not weight]
+        known.append((weakref.ref(weight), weakref.ref(tiled)))
         return tiled
+
+    def _alike(self, weight, tiled, most: int = 16, most_bytes: int = 1 << 30) -> list[tuple]:
+        """(weight, tiled copy) pairs to time a choice on: the given one, then other live weights of its shape that
+        were tiled here (the same projection in other layers). A timing that calls one weight over and over reads it
+        from the memory-side cache (256 MB), which flatters the vendor library's kernels by a third and decides
+        wrongly; a step streams every layer's weights from memory, so the timings rotate over these pairs."""
+        pairs = [(weight, tiled)]
+        for w, t in self._tiled_weights.get(tuple(weight.shape), []):
+            w, t = w(), t()
+            if len(pairs) >= most or len(pairs) * weight.numel() * weight.element_size() >= most_bytes:
+                break
+            if w is not None and t is not None and w is not weight and w.dtype == weight.dtype \
+                    and w.device == weight.device:
+                pairs.append((w, t if tiled is not None else None))
+        return pairs
+
+    @staticmethod
+    def _graph_time(calls: list, replays: int = 3) -> float:
+        """Milliseconds a call, for calls that are shorter than a launch from here takes: recorded as one graph
+        (each call once, in order), replayed. What a call needs at its first use happens before the recording."""
+        for call in calls:
+            call()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            keep = [call() for call in calls]
+        graph.replay()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(replays):
+            graph.replay()
+        end.record()
+        end.synchronize()
+        del graph, keep
+        return start.elapsed_time(end) / (replays * len(calls))
+
+    @staticmethod
+    def _in_turn(pairs: list[tuple], call, at_least: int = 8) -> list:
+        """`call(weight, tiled)` for each pair in turn, at least `at_least` calls in all."""
+        rounds = -(-at_least // len(pairs))
+        return [lambda w=w, t=t: call(w, t) for _ in range(rounds) for w, t in pairs]
 
     def _row_scale(self, x, tiled, row_scale, what):
         """Checks of a product over un-normed rows with the norm folded into `tiled`; returns (stats, parts, eps)."""
@@ -292,20 +338,13 @@ class HipKernels:
                   "f32x2": lambda x, w: HipKernels._two_halves(x, w)}
 
     def _time_mid_forms(self, x, weight) -> str:
+        pairs = self._alike(weight, None)
         took = {}
         try:
             for name, fn in self._MID_FORMS.items():
                 if name == "f32x2" and weight.shape[1] % 512:
                     continue
-                for _ in range(2):
-                    fn(x, weight)
-                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                start.record()
-                for _ in range(6):
-                    fn(x, weight)
-                end.record()
-                end.synchronize()
-                took[name] = start.elapsed_time(end)
+                took[name] = self._graph_time(self._in_turn(pairs, lambda w, _t, fn=fn: fn(x, w)))
         except (RuntimeError, TypeError):           # this torch has no float32 result for a bfloat16 product
             self._mid_forms = False
             return "bf16"
@@ -373,29 +412,16 @@ class HipKernels:
 
     def _time_parts(self, x, weight, tiled, splits) -> str:
         """Each way together with the residual add + norm that reads the product (reading parts costs that kernel a
-        few microseconds, which the product must win back). Both are shorter than a launch from here takes, so they
-        are timed as recorded graphs of several calls."""
+        little, which the product must win back)."""
         n = weight.shape[0]
         residual = torch.zeros((x.shape[0], n), dtype=torch.bfloat16, device=x.device)
         ones = torch.ones(n, dtype=torch.bfloat16, device=x.device)
-        took = {}
-        for name, fn in (("parts", lambda: self._rows_parts(x, weight, tiled, splits)),
-                         ("vendor", lambda: self._vendor_product(x, weight))):
-            self.add_rmsnorm(fn(), residual, ones, 1e-6)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                for _ in range(8):
-                    keep = self.add_rmsnorm(fn(), residual, ones, 1e-6)
-            graph.replay()
-            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record()
-            for _ in range(3):
-                graph.replay()
-            end.record()
-            end.synchronize()
-            took[name] = start.elapsed_time(end)
-            del graph, keep
+        pairs = self._alike(weight, tiled)
+        took = {
+            "parts": self._graph_time(self._in_turn(
+                pairs, lambda w, t: self.add_rmsnorm(self._rows_parts(x, w, t, splits), residual, ones, 1e-6))),
+            "vendor": self._graph_time(self._in_turn(
+                pairs, lambda w, _t: self.add_rmsnorm(self._vendor_product(x, w), residual, ones, 1e-6)))}
         return "parts" if took["parts"] < 0.97 * took["vendor"] else "vendor"
 
     def sum_parts(self, parts, dtype=torch.bfloat16):
@@ -411,20 +437,11 @@ class HipKernels:
 
     def _time_rows(self, rows, weight, tiled, gated) -> str:
         x = torch.randn(rows, weight.shape[1], device=weight.device).to(torch.bfloat16)
-        forms = {"rows": lambda: self._rows_product(x, weight, tiled, gated),
-                 "vendor": (lambda: self.silu_mul(self._vendor_product(x, weight))) if gated
-                 else (lambda: self._vendor_product(x, weight))}
-        took = {}
-        for name, fn in forms.items():
-            for _ in range(2):
-                fn()
-            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record()
-            for _ in range(6):
-                fn()
-            end.record()
-            end.synchronize()
-            took[name] = start.elapsed_time(end)
+        pairs = self._alike(weight, tiled)
+        vendor = (lambda w, _t: self.silu_mul(self._vendor_product(x, w))) if gated \
+            else (lambda w, _t: self._vendor_product(x, w))
+        took = {"rows": self._graph_time(self._in_turn(pairs, lambda w, t: self._rows_product(x, w, t, gated))),
+                "vendor": self._graph_time(self._in_turn(pairs, vendor))}
         return "rows" if took["rows"] < took["vendor"] else "vendor"
 
     def linear_add(self, x, weight, tiled, residual, want_stats=False):

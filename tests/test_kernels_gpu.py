@@ -375,7 +375,7 @@ def test_product_for_17_to_64_rows_over_many_tiles(hip):
         assert torch.equal(hip.linear(x, w, torch.float32, tiled), got.float())
         fewer = hip.linear(x[3:21].contiguous(), w, None, tiled)                       # 18 rows, other places
         assert torch.equal(fewer, got[3:21]) if m >= 21 else True
-    for m, k, inter in ((64, 4096, 12288), (17, 256, 8192), (40, 1024, 8320)):
+    for m, k, inter in ((64, 4096, 12288), (17, 256, 8192), (40, 1024, 8320), (33, 512, 16384), (64, 768, 16512)):   # the last two: eight waves a block
         x, w = _randn(m, k, dtype=bf, seed=82), _randn(2 * inter, k, dtype=bf, seed=83, scale=0.05)
         tiled = hip.tile_weight(w)
         hip._mid_choice[("rows", (2 * inter, k), m <= 32, True)] = "rows"
