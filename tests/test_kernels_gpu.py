@@ -451,6 +451,32 @@ def test_product_in_shares_of_k_for_narrow_weights(hip):
     hip._mid_choice.clear()
 
 
+def test_choices_are_timed_over_the_same_shaped_weights_of_other_layers(hip):
+    """Every weight that got a tiled copy is known by shape (weakly: a weight that is gone is forgotten), and a timing
+    calls its candidates on them in turn, the given one first, up to 16 of them or a gigabyte: one weight called over
+    and over would be read from the memory-side cache, which a step's weights never are."""
+    import gc
+    bf = torch.bfloat16
+    ws = [_randn(2048, 512, dtype=bf, seed=300 + i) for i in range(5)]
+    ts = [hip.tile_weight(w) for w in ws]
+    pairs = hip._alike(ws[2], ts[2])
+    assert pairs[0][0] is ws[2] and pairs[0][1] is ts[2] and len(pairs) == 5
+    assert {id(w) for w, _ in pairs} == {id(w) for w in ws} and all(t is ts[[id(x) for x in ws].index(id(w))] for w, t in pairs)
+    assert all(t is None for _, t in hip._alike(ws[0], None)) and len(hip._alike(ws[0], None)) == 5
+    assert len(hip._alike(ws[0], ts[0], most=3)) == 3 and len(hip._alike(ws[0], ts[0], most_bytes=2 * 2048 * 512 * 2)) == 2
+    folded = hip.tile_weight(ws[1], _randn(512, dtype=bf, seed=310))      # a new copy of a known weight replaces the old
+    assert [t for w, t in hip._alike(ws[0], ts[0]) if w is ws[1]] == [folded]
+    del pairs, ws[3:], ts[3:]
+    gc.collect()
+    assert len(hip._alike(ws[0], ts[0])) == 3
+    calls = hip._in_turn(hip._alike(ws[0], ts[0]), lambda w, t: (w, t))
+    assert len(calls) == 9 and calls[0]()[0] is ws[0] and calls[3]()[0] is ws[0]          # three rounds over three weights
+    assert {id(c()[0]) for c in calls[:3]} == {id(w) for w in ws}
+    x = _randn(32, 512, dtype=bf, seed=311)
+    ms = hip._graph_time(hip._in_turn(hip._alike(ws[0], ts[0]), lambda w, t: torch.matmul(x, w.t())))
+    assert 0 < ms < 5
+
+
 def test_vendor_product_forms_for_steps_of_17_to_64_rows(hip):
     """Steps of 17 to 64 bfloat16 rows take the vendor library's product in the faster of two forms, timed once per
     weight shape and row bucket: both are the product rounded once, whichever is kept, and the float32 output is the
