@@ -176,14 +176,31 @@ def test_sixty_four_rows_decode_together_from_graphs(folder, dtype, products):
     load_hip()._mid_choice.clear()
 
 
-def test_engine_at_the_wide_sizes_with_everything_on(folder):
+def _force_our_products(on: bool) -> None:
+    """The kernels of our own for 17 to 64 rows at the wide sizes (gated product through LDS, output and down
+    projections in shares of K), instead of what timing them against the vendor library's would choose."""
+    from holon_amd.kernels import load_hip
+    hidden, inter, wide = WIDE["hidden_size"], WIDE["intermediate_size"], WIDE["num_attention_heads"] * WIDE["head_dim"]
+    choice = load_hip()._mid_choice
+    choice.clear()
+    if on:
+        for few in (True, False):
+            choice[("rows", (2 * inter, hidden), few, True)] = "rows"
+            for shape in ((hidden, wide), (hidden, inter)):
+                choice[("parts", shape, few)] = "parts"
+
+
+@pytest.mark.parametrize("products", ["timed", "ours"])
+def test_engine_at_the_wide_sizes_with_everything_on(folder, products):
     """The whole engine in bfloat16 at the measured layer sizes (matrix-core attention, the few-row products over
     tiled weights, the residual add and the gated form inside them). One step in flight changes no launch, so it must
     change no token, greedy or seeded. Graph replay shapes the decode attention for its length bucket (other splits
     of the keys, other roundings) and shared prefixes cut the prompts elsewhere, and 20 requests make steps of more
-    than 16 rows: there the greedy tokens are held to the plain model's own greedy decoding in bfloat16."""
+    than 16 rows (their products once as timing chooses, once in the kernels of our own): there the greedy tokens are
+    held to the plain model's own greedy decoding in bfloat16."""
     from holon_amd.config import EngineConfig, SamplingParams
     from holon_amd.engine.engine import Engine
+    _force_our_products(products == "ours")
     start = H.random_ids(40, WIDE["vocab_size"], 300)
     prompts = [start[: 8 + 4 * (i % 9)] + H.random_ids(3 + 5 * i, WIDE["vocab_size"], 301 + i) for i in range(20)]
     shape = dict(model=str(folder), device="cuda", dtype="bfloat16", page_size=16, max_seqs=24, max_model_len=256,
@@ -200,6 +217,7 @@ def test_engine_at_the_wide_sizes_with_everything_on(folder):
         for prompt, got in zip(prompts, full.generate(prompts, params)):
             H.assert_greedy_follows(plain, prompt, got)
     assert full.cache.tokens_saved > 0 and full.stats()["graphs"] >= 1 and full.runner.graph_replays > 10
+    _force_our_products(False)
 
 
 def test_long_context_attention_kernels():
