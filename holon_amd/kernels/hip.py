@@ -197,6 +197,7 @@ class HipKernels:
 
     skinny_rows = 16          # up to this many rows (one tile of tokens) the hand-written weight-streaming product runs
     _mid_forms = True         # whether steps of 17 to 64 rows may choose between the vendor product's two forms
+    deep_k = 8192             # from this K on, prompt portions of up to 1,024 rows choose between them as well
 
     def tile_weight(self, weight, scale=None):
         """A copy of `weight` [N, K] in the layout the few-row product streams fastest, or None when its shape or
@@ -315,11 +316,15 @@ class HipKernels:
         library's choice of kernel has holes at some shapes (a deep, narrow weight, 5120 x 25600: 145 us, where its
         product of the same operands with a float32 result takes 83, two such products over the halves of K 73, and
         the weights alone would stream in 42), so for such steps the forms are timed once per weight shape and row
-        bucket, outside graph capture, and the fastest is kept. All accumulate in float32 and round once."""
-        m = x.shape[0]
-        if not (16 < m <= 64 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and self._mid_forms):
+        bucket, outside graph capture, and the fastest is kept. Over deep weights (K of 8,192 and more) the same
+        holds for prompt portions of up to 1,024 rows (the same weight at 544 rows: 260 us, over the halves of K 213;
+        at 256 rows 263, with a float32 result 184), in buckets of 128, 256, 512 and 1,024 rows. All forms accumulate
+        in float32 and round once."""
+        m, k = x.shape[0], weight.shape[1]
+        if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and self._mid_forms
+                and (16 < m <= 64 or (64 < m <= 1024 and k >= self.deep_k))):
             return torch.matmul(x, weight.t())
-        key = (tuple(weight.shape), m <= 32)
+        key = (tuple(weight.shape), m <= 32 if m <= 64 else 1 << (m - 1).bit_length())
         form = self._mid_choice.get(key)
         if form is None:
             if torch.cuda.is_current_stream_capturing():
@@ -349,7 +354,7 @@ class HipKernels:
             self._mid_forms = False
             return "bf16"
         best = min(took, key=took.get)
-        return best if took[best] < 0.85 * took["bf16"] else "bf16"
+        return best if took[best] < 0.92 * took["bf16"] else "bf16"
 
     def serves_rows(self, rows, weight, tiled, gated=False):
         """Whether steps of `rows` rows (17 to 64) over this weight run the product that shares the rows through LDS

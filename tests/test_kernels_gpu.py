@@ -478,14 +478,14 @@ def test_choices_are_timed_over_the_same_shaped_weights_of_other_layers(hip):
 
 
 def test_vendor_product_forms_for_steps_of_17_to_64_rows(hip):
-    """Steps of 17 to 64 bfloat16 rows take the vendor library's product in the faster of two forms, timed once per
-    weight shape and row bucket: both are the product rounded once, whichever is kept, and the float32 output is the
-    bfloat16 one cast up."""
+    """Steps of 17 to 64 bfloat16 rows (over deep weights also prompt portions of up to 1,024 rows) take the vendor
+    library's product in the fastest of three forms, timed once per weight shape and row bucket: each is the product
+    rounded once, whichever is kept, and the float32 output is the bfloat16 one cast up."""
     bf = torch.bfloat16
-    for m, k, n in ((32, 25600, 5120), (24, 4096, 6144), (64, 1024, 512)):
+    for m, k, n in ((32, 25600, 5120), (24, 4096, 6144), (64, 1024, 512), (300, 25600, 5120), (1000, 8192, 512)):
         x, w = _randn(m, k, dtype=bf, seed=70), _randn(n, k, dtype=bf, seed=71, scale=0.02)
         want = x.double() @ w.double().T
-        key = ((n, k), m <= 32)
+        key = ((n, k), m <= 32 if m <= 64 else {300: 512, 1000: 1024}[m])
         hip._mid_choice.pop(key, None)
         got = hip.linear(x, w)
         assert hip._mid_choice[key] in ("bf16", "f32", "f32x2")           # timed and kept
@@ -495,6 +495,10 @@ def test_vendor_product_forms_for_steps_of_17_to_64_rows(hip):
             assert y.dtype == bf and H.op_budget_usage(y, want, bf, k) <= 1, (m, k, n, form)
             assert torch.equal(hip.linear(x, w, torch.float32), y.float())
         assert H.op_budget_usage(got, want, bf, k) <= 1
+    before = dict(hip._mid_choice)
+    hip.linear(_randn(300, 4096, dtype=bf, seed=72), _randn(512, 4096, dtype=bf, seed=73))      # a shallow weight, and
+    hip.linear(_randn(1025, 8192, dtype=bf, seed=74), _randn(512, 8192, dtype=bf, seed=75))     # more rows: not timed
+    assert hip._mid_choice == before
     assert ((5120, 25600), False) not in hip._mid_choice                   # the other bucket was never asked for
     hip._mid_choice.clear()
 
