@@ -237,21 +237,26 @@ class HipKernels:
     @staticmethod
     def _graph_time(calls: list, replays: int = 3) -> float:
         """Milliseconds a call, for calls that are shorter than a launch from here takes: recorded as one graph
-        (each call once, in order), replayed. What a call needs at its first use happens before the recording."""
-        for call in calls:
-            call()
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            keep = [call() for call in calls]
-        graph.replay()
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for _ in range(replays):
+        (each call once, in order), replayed. What a call needs at its first use happens before the recording. A
+        candidate that there is no memory to try takes forever (and so is not chosen)."""
+        try:
+            for call in calls:
+                call()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                keep = [call() for call in calls]
             graph.replay()
-        end.record()
-        end.synchronize()
-        del graph, keep
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(replays):
+                graph.replay()
+            end.record()
+            end.synchronize()
+            del graph, keep
+        except torch.OutOfMemoryError:            # no room to try it: it does not win
+            torch.cuda.empty_cache()
+            return float("inf")
         return start.elapsed_time(end) / (replays * len(calls))
 
     @staticmethod
