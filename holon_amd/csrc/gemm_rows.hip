@@ -151,6 +151,21 @@ void launch_rows(const void* x, const void* w, void* y, int M, int N, int K, hip
   if (mt == 2) ROWS(2); else if (mt == 3) ROWS(3); else ROWS(4);
 #undef ROWS
 }
+
+// The same for 65 to 128 rows (five to eight tiles of tokens): chunks of 64 columns keep the rows' two buffers within
+// the LDS a block may have without asking.
+template <int WAVES, int OUT>
+void launch_rows_tall(const void* x, const void* w, void* y, int M, int N, int K, hipStream_t s, int splits) {
+  const dim3 grid(N / 16 / WAVES, splits), block(WAVES * 64);
+#define ROWS(MT) gemm_rows_kernel<MT, WAVES, 64, OUT><<<grid, block, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, y, M, N, K)
+  switch ((M + 15) / 16) {
+    case 5: ROWS(5); break;
+    case 6: ROWS(6); break;
+    case 7: ROWS(7); break;
+    default: ROWS(8); break;
+  }
+#undef ROWS
+}
 }  // namespace
 
 // Whether holon_gemm_rows_bf16 serves this product (gated: N is the number of output columns I, the weight has 2 I rows).
@@ -199,6 +214,7 @@ extern "C" int holon_gemm_rows_glu_bf16(const void* x, const void* w_tiled, void
 namespace {
 constexpr int PARTS_KC = 128;          // columns of K a chunk of the split form holds
 constexpr int PARTS_MAX_SPLITS = 16;
+constexpr int PARTS_MAX_ROWS = 128;    // (the forms that write whole products serve up to 64)
 constexpr int PARTS_WAVES = 4;         // eight were slower at every shape measured
 
 // y[i] = round(parts[0][i] + parts[1][i] + ...) in split order, four values a thread.
@@ -218,7 +234,7 @@ __global__ void sum_parts_kernel(const float* __restrict__ parts, bf16_t* __rest
 // Whether holon_gemm_rows_parts_bf16 serves this product with K cut into `splits` shares (blocks of four waves, each
 // with a tile of 16 columns of its own).
 extern "C" int holon_gemm_rows_parts_supported(int M, int N, int K, int splits) {
-  return M > 16 && M <= 64 && N % 16 == 0 && (N / 16) % PARTS_WAVES == 0 && splits >= 1 &&
+  return M > 16 && M <= PARTS_MAX_ROWS && N % 16 == 0 && (N / 16) % PARTS_WAVES == 0 && splits >= 1 &&
          splits <= PARTS_MAX_SPLITS && K > 0 && K % (PARTS_KC * splits) == 0;
 }
 
@@ -232,13 +248,14 @@ extern "C" int holon_gemm_rows_splits(int M, int N, int K) {
   return splits > 1 && holon_gemm_rows_parts_supported(M, N, K, splits) ? splits : 0;
 }
 
-// parts[s][M][N] (float32) = x[:, share s of K] w[:, share s of K]^T over tiled weights, 17 <= M <= 64: the product is
+// parts[s][M][N] (float32) = x[:, share s of K] w[:, share s of K]^T over tiled weights, 17 <= M <= 128: the product is
 // the sum of the parts in order, which the reader takes (holon_rmsnorm_parts, holon_sum_parts).
 extern "C" int holon_gemm_rows_parts_bf16(const void* x, const void* w_tiled, void* parts, int M, int N, int K,
                                           int splits, void* stream) {
   HOLON_CHECK(holon_gemm_rows_parts_supported(M, N, K, splits),
               "gemm in parts (17 to 64 rows): M=%d N=%d K=%d splits=%d not served", M, N, K, splits);
-  launch_rows<PARTS_WAVES, PARTS_KC, 3>(x, w_tiled, parts, M, N, K, (hipStream_t)stream, splits);
+  if (M > 64) launch_rows_tall<PARTS_WAVES, 3>(x, w_tiled, parts, M, N, K, (hipStream_t)stream, splits);
+  else launch_rows<PARTS_WAVES, PARTS_KC, 3>(x, w_tiled, parts, M, N, K, (hipStream_t)stream, splits);
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -95,7 +95,7 @@ int holon_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, int M, int
 int holon_gemm_rows_supported(int M, int N, int K, int gated);
 int holon_gemm_rows_bf16(const void* x, const void* w_tiled, void* y, int M, int N, int K, int out_f32, void* stream);
 int holon_gemm_rows_glu_bf16(const void* x, const void* w_tiled, void* y, int M, int I, int K, void* stream);
-// The same for narrow weights (a few hundred tiles), with K cut into `splits` shares over the grid as well: blocks of
+// The same for narrow weights (a few hundred tiles) and up to 128 rows, with K cut into `splits` shares over the grid as well: blocks of
 // four waves, N / 16 a multiple of 4, K a multiple of 128 * splits, splits <= 16. parts [splits, M, N]
 // float32 holds each share's sums; the product is their sum in order (holon_sum_parts rounds it to bfloat16;
 // holon_rmsnorm_parts, the residual add + norm, reads them itself). holon_gemm_rows_splits: the number of shares that

@@ -390,18 +390,20 @@ class HipKernels:
                        self._stream())
         return y
 
+    parts_rows = 128          # the product in shares of K serves steps of 17 to this many rows
+
     def linear_parts(self, x, weight, tiled):
-        """-> float32 [splits, M, N], the product over each share of K, when that kernel serves this step (17 to 64
+        """-> float32 [splits, M, N], the product over each share of K, when that kernel serves this step (17 to 128
         bfloat16 rows over a narrow tiled weight) and, timed once per weight shape and row bucket against the vendor
         library's product (each with the add + norm that reads it), is the faster; None otherwise (nothing was done)."""
         (m, k), n = x.shape, weight.shape[0]
-        if not (tiled is not None and 16 < m <= 64 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                and weight.shape[1] == k and x.is_contiguous()):
+        if not (tiled is not None and 16 < m <= self.parts_rows and x.dtype == torch.bfloat16
+                and weight.dtype == torch.bfloat16 and weight.shape[1] == k and x.is_contiguous()):
             return None
         splits = self.lib.holon_gemm_rows_splits(m, n, k)
         if not splits:
             return None
-        key = ("parts", (n, k), m <= 32)
+        key = ("parts", (n, k), m <= 32 if m <= 64 else 128)
         use = self._mid_choice.get(key)
         if use is None:
             if torch.cuda.is_current_stream_capturing():

@@ -43,7 +43,7 @@ class TorchKernels:
     name = "torch-plain"
 
     fold_norms = False       # a test may switch the folded-norm path on: the twin then stands in for the tiled copy
-    split_products = 0       # a test may set a number of shares: steps of 17 to 64 rows then get their products that
+    split_products = 0       # a test may set a number of shares: steps of 17 to 128 rows then get their products that
                              # are added to the residual stream as partial sums over that many shares of K
 
     def embedding(self, ids, table, take=None, want_stats=False):
@@ -98,7 +98,7 @@ class TorchKernels:
 
     def linear_parts(self, x, weight, tiled):
         s, k = self.split_products, x.shape[1]
-        if not s or not 16 < x.shape[0] <= 64 or k % s:
+        if not s or not 16 < x.shape[0] <= 128 or k % s:
             return None
         share = k // s
         return torch.stack([_up(x[:, i * share:(i + 1) * share]) @ _up(weight[:, i * share:(i + 1) * share]).T
@@ -111,7 +111,7 @@ class TorchKernels:
         return total.to(dtype)
 
     def linear_add(self, x, weight, tiled, residual, want_stats=False):
-        if self.split_products and 16 < x.shape[0] <= 64:
+        if self.split_products and 16 < x.shape[0] <= 128:
             return False                                     # as the HIP kernels: not fused at these row counts
         residual.copy_((_up(residual) + _up(self.linear(x, weight))).to(residual.dtype))
         if want_stats and self.fold_norms and residual.shape[0] <= 16:

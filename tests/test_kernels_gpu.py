@@ -402,7 +402,8 @@ def test_product_in_shares_of_k_for_narrow_weights(hip):
     choice."""
     from holon_amd.kernels.hip import KernelError
     bf = torch.bfloat16
-    for m, k, n in ((64, 4096, 4096), (17, 12288, 4096), (33, 1024, 5120), (48, 25600, 5120), (40, 512, 320), (64, 256, 64)):
+    for m, k, n in ((64, 4096, 4096), (17, 12288, 4096), (33, 1024, 5120), (48, 25600, 5120), (40, 512, 320), (64, 256, 64),
+                    (65, 4096, 4096), (100, 12288, 4096), (128, 1024, 5120), (90, 256, 64), (113, 2560, 1024)):
         x, w = _randn(m, k, dtype=bf, seed=90), _randn(n, k, dtype=bf, seed=91, scale=0.05)
         tiled = hip.tile_weight(w)
         splits = hip.lib.holon_gemm_rows_splits(m, n, k)
@@ -439,6 +440,7 @@ def test_product_in_shares_of_k_for_narrow_weights(hip):
     hip._mid_choice[("parts", (4096, 4096), True)] = "parts"
     assert hip.linear_parts(x, w, tiled).shape == (8, 32, 4096)
     assert hip.linear_parts(x[:16].contiguous(), w, tiled) is None and hip.linear_parts(x, w, None) is None
+    assert hip.linear_parts(_randn(129, 4096, dtype=bf, seed=99), w, tiled) is None            # beyond 128 rows
     assert hip.linear_parts(_randn(32, 4096, dtype=torch.float32, seed=96), w.float(), tiled) is None          # float32 rows: not this path
     w = _randn(4096, 4224, dtype=bf, seed=97)                                             # K = 33 x 128: no equal shares
     assert hip.linear_parts(_randn(32, 4224, dtype=bf, seed=98), w, hip.tile_weight(w)) is None

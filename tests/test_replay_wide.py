@@ -190,6 +190,31 @@ def _force_our_products(on: bool) -> None:
                 choice[("parts", shape, few)] = "parts"
 
 
+def test_a_hundred_rows_decode_together(folder):
+    """Decode steps of 100 rows shrinking to 70 (graph buckets 128 and 96), the output and down projections' products
+    as partial sums over shares of K, which serve up to 128 rows: every row's logits against the plain model."""
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    from holon_amd.kernels import load_hip
+    hidden, inter, wide = WIDE["hidden_size"], WIDE["intermediate_size"], WIDE["num_attention_heads"] * WIDE["head_dim"]
+    for shape in ((hidden, wide), (hidden, inter)):
+        load_hip()._mid_choice[("parts", shape, 128)] = "parts"
+    try:
+        requests = {f"q{i}": (H.random_ids(1 + (5 * i) % 37 + (3 if i < 70 else 2), WIDE["vocab_size"], 1500 + i),
+                              1 + (5 * i) % 37) for i in range(100)}          # 70 decode three tokens, 30 two
+        trace = _wide_batch_trace(requests, 2304)
+        loaded = load_model(folder, device="cuda", dtype="bfloat16", page_size=16, max_seqs=128, max_model_len=256,
+                            max_step_tokens=2304, cache_tokens=H.peak_live_tokens(trace), graphs=True)
+        rep = Replayer(loaded)
+        got = H.run_trace(rep, trace)
+        assert len(got) == 100 + 70 * 3 + 30 * 2
+        assert {(128, 1024), (96, 1024)} <= set(loaded.runner.graphs), set(loaded.runner.graphs)
+        _check(folder, "bfloat16", {rid: ids for rid, (ids, _) in requests.items()}, got, "wide bfloat16 100 rows")
+        rep.cache.check()
+    finally:
+        load_hip()._mid_choice.clear()
+
+
 @pytest.mark.parametrize("products", ["timed", "ours"])
 def test_engine_at_the_wide_sizes_with_everything_on(folder, products):
     """The whole engine in bfloat16 at the measured layer sizes (matrix-core attention, the few-row products over
