@@ -35,7 +35,7 @@ QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention
 QWEN3_4B = dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, tie_word_embeddings=True)
 
 
-def workload(name: str, layers: int | None, dtype: str) -> int:
+def workload(name: str, layers: int | None, dtype: str, products: str = "timed") -> int:
     """A whole job: every request added at once, stepped until all are finished."""
     import random
 
@@ -56,7 +56,7 @@ def workload(name: str, layers: int | None, dtype: str) -> int:
         ecfg = dict(max_seqs=8, max_model_len=40960, max_step_tokens=4096)
     cfg_json = dict(shape, num_hidden_layers=layers or shape["num_hidden_layers"])
     engine = Engine.from_random(cfg_json, seed=0, cfg=EngineConfig(
-        model=f"random:{name}", device="cuda:0", dtype=dtype, page_size=16,
+        model=f"random:{name}", device="cuda:0", dtype=dtype, page_size=16, products=products,
         cache_tokens=len(prompts) * (max(map(len, prompts)) + params.max_tokens + 64), **ecfg))
     for p in prompts:
         engine.add(p, params)
@@ -83,7 +83,8 @@ def workload(name: str, layers: int | None, dtype: str) -> int:
                    "requests": len(prompts), "prompt_tokens": prompt_tokens, "output_tokens": out, **ecfg},
         "until_prompts_done": {"seconds": round(t_prompts, 3), "prompt_tokens_per_s": round(prompt_tokens / t_prompts, 1)},
         "decode_tail": {"tokens_per_s": round((out - out_at) / max(total - t_prompts, 1e-9), 1)},
-        "steps": steps, "mixed_steps": stats["mixed_steps"], "preemptions": stats["preemptions"]}), flush=True)
+        "steps": steps, "mixed_steps": stats["mixed_steps"], "preemptions": stats["preemptions"],
+        "products": {"mode": products, "took": stats["products"]}}), flush=True)
     return 0
 
 
@@ -100,6 +101,8 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--workload", choices=("decode", "mixed", "long"), default="decode")
+    ap.add_argument("--products", choices=("own", "vendor", "timed"), default="timed",
+                    help="EngineConfig.products: which kernel products of 17 to 1,024 rows take (reported in the line)")
     a = ap.parse_args(argv)
     if a.gpus != 1:
         print(f"bench.py: this engine serves on one GPU; --gpus {a.gpus} is not a configuration it has", flush=True)
@@ -108,7 +111,7 @@ def main(argv: list[str] | None = None) -> int:
         from .kernels import build as kernel_build
         if kernel_build.find_library() is None:
             kernel_build.build()
-        return workload(a.workload, None if "--layers" not in (argv or sys.argv) else a.layers, a.dtype)
+        return workload(a.workload, None if "--layers" not in (argv or sys.argv) else a.layers, a.dtype, a.products)
 
     import torch
 
@@ -123,7 +126,7 @@ def main(argv: list[str] | None = None) -> int:
     engine = Engine.from_random(cfg_json, seed=0, cfg=EngineConfig(
         model="random:qwen3-8b", device="cuda:0", dtype=a.dtype, page_size=16, max_seqs=max_batch,
         max_model_len=CONTEXT + 16, max_step_tokens=4096, cache_tokens=max_batch * (CONTEXT + 16),
-        graphs=not a.no_graphs))
+        graphs=not a.no_graphs, products=a.products))
     spec, c = engine.spec, cfg_json
     item = 2 if a.dtype == "bfloat16" else 4
     g = torch.Generator().manual_seed(0)
@@ -197,12 +200,14 @@ def main(argv: list[str] | None = None) -> int:
                    "hidden": h, "heads": hq, "kv_heads": hkv, "head_dim": d, "intermediate": inter, "vocab": v,
                    "tied": False, "global_batch": a.batch, "seq_len": CONTEXT, "prefill_tokens": PROMPT,
                    "decode_prompt_len": decode_prompt, "page_size": 16,
-                   "parallelism": "single GPU", "graphs": not a.no_graphs, "mean_context": round(ctx, 1)},
+                   "parallelism": "single GPU", "graphs": not a.no_graphs, "mean_context": round(ctx, 1),
+                   "products": a.products},
         "prefill": {"value": round(PROMPT / (pre_ms * 1e-3), 1), "tokens": PROMPT, "ms": round(pre_ms, 3),
                     "frac": round(pre_flops / (pre_ms * 1e-3) / PEAK_FLOPS[a.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},
         "points": points,
+        "products": engine.products(),
         "latency": {"ttft_ms_p50": round(ttft_ms, 3), "ttft_tokens": PROMPT, "tpot_ms_p50": round(tpot_ms, 4),
                     "tpot_batch": a.batch},
     }

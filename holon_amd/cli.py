@@ -36,10 +36,20 @@ def engine_flags(parser: argparse.ArgumentParser | argparse._ArgumentGroup) -> N
         elif f.name == "max_model_len":            # also `auto` (core/holon/core/cli.py:44-47, 76)
             parser.add_argument(flag, type=lambda s: s if s == "auto" else int(s), default=f.default,
                                 help=help_ + f"; auto: the model's trained context, at most {AUTO_CONTEXT}")
+        elif f.name == "product_pins":
+            parser.add_argument(flag, type=_pins, default=None, help=help_)
         elif kind in (int, float, str):
             parser.add_argument(flag, type=kind, default=f.default, help=help_)
         else:                                         # int | None
             parser.add_argument(flag, type=int, default=f.default, help=help_)
+
+
+def _pins(text: str) -> dict[str, str]:
+    """`kind:NxK:rows=form,kind:NxK:rows=form` -> {key: form}."""
+    pairs = [item.split("=", 1) for item in text.split(",") if item.strip()]
+    if any(len(pair) != 2 for pair in pairs):
+        raise argparse.ArgumentTypeError("expected kind:NxK:rows=form, separated by commas")
+    return {key.strip(): form.strip() for key, form in pairs}
 
 
 def engine_config(model: str, args: argparse.Namespace) -> EngineConfig:

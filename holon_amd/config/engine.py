@@ -35,6 +35,12 @@ class EngineConfig:
     graphs: bool = _setting(True, "replay decode steps from HIP graphs, per batch-size bucket")
     decode_weight_copy: bool = _setting(True, "keep a second copy of every projection in the tile layout that steps of "
                                               "few rows stream fastest (doubles the weights' memory)")
+    products: str = _setting("own", "which kernel a matrix product of 17 to 1,024 rows takes where several serve it: "
+                                    "own (this package's wherever one serves), vendor (the vendor library's plain "
+                                    "product), timed (candidates are timed once while the engine starts)")
+    product_pins: dict | None = _setting(None, "single products pinned whatever the mode, as kind:NxK:rows=form,... "
+                                               "(what stats()['products'] lists; on the command line a comma-"
+                                               "separated list)")
 
     def __post_init__(self) -> None:
         for name in ("page_size", "max_seqs", "max_model_len", "max_step_tokens"):
@@ -46,6 +52,10 @@ class EngineConfig:
             raise ValueError(f"EngineConfig.dtype must be one of {DTYPES}, got {self.dtype!r}")
         if self.chunk_with_decode and self.max_step_tokens < self.max_seqs + self.chunk_with_decode:
             raise ValueError("mixed steps need max_step_tokens >= max_seqs + chunk_with_decode")
+        from .products import MODES, check_pins
+        if self.products not in MODES:
+            raise ValueError(f"EngineConfig.products must be one of {MODES}, got {self.products!r}")
+        self.product_pins = check_pins(self.product_pins) or None
 
 
 @dataclasses.dataclass

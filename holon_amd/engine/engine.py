@@ -23,13 +23,9 @@ import torch
 
 from ..cache.pool import OutOfPages
 from ..config.engine import EngineConfig, SamplingParams
-from ..config.model import read_config_json
-from ..registry import resolve
 from ..sampling.sampler import Sampler, sequence_seed
-from ..weights.loader import load_weights
-from ..weights.random_init import fill_random
 from .batch import StepRow
-from .loading import attach_cache, build_from_spec, default_kernels, torch_dtype
+from .loading import assemble, attach_cache
 from .request import Logprobs, Seq, Status, TokenDelta
 from .scheduler import Scheduler
 
@@ -51,23 +47,13 @@ class _Launched:
 class Engine:
     def __init__(self, cfg: EngineConfig, kernels=None, *, random_config: dict | None = None, seed: int = 0) -> None:
         self.cfg = cfg
-        device, dtype = torch.device(cfg.device), torch_dtype(cfg.dtype)
-        self.device, self.dtype = device, dtype
-        self.kernels = kernels if kernels is not None else default_kernels(device)
-        config_json, generation = (random_config, None) if random_config is not None else read_config_json(cfg.model)
-        self.model_config, self.spec = resolve(config_json, generation)
+        self._assembled = assemble(cfg, kernels, random_config=random_config, seed=seed)
+        a = self._assembled
+        self.device, self.dtype, self.kernels = a.device, a.dtype, a.kernels
+        self.model_config, self.spec, self.model = a.config, a.spec, a.model
         self.eos = set(self.spec.eos_token_ids)
-        shape = dict(page_size=cfg.page_size, max_seqs=cfg.max_seqs, max_model_len=cfg.max_model_len,
-                     max_step_tokens=cfg.max_step_tokens)
-        self.model, _ = build_from_spec(self.spec, device=device, dtype=dtype, kernels=self.kernels,
-                                        decode_copy=cfg.decode_weight_copy, **shape)
-        if random_config is not None:
-            fill_random(self.model, self.spec, seed, device, dtype)
-        else:
-            load_weights(self.model, self.spec, cfg.model, device, dtype)
         tokens = self._cache_tokens()
-        self.cache, self.runner = attach_cache(self.model, device=device, dtype=dtype, kernels=self.kernels,
-                                               cache_tokens=tokens, graphs=cfg.graphs, **shape)
+        self.cache, self.runner = attach_cache(self.model, cache_tokens=tokens, graphs=cfg.graphs, **a.shape(cfg))
         if not self.cache.fits_alone(cfg.max_model_len):
             raise OutOfPages(f"the cache holds {tokens} tokens, fewer than one request of max_model_len "
                              f"{cfg.max_model_len}; lower max_model_len or give the cache more memory")
@@ -76,7 +62,7 @@ class Engine:
             if not self.cache.enable_prefix(hashlib.blake2b(identity, digest_size=16).digest()):
                 print("holon_amd: this model keeps state that pages do not hold whole; prompts share nothing",
                       file=sys.stderr)
-        self.sampler = Sampler(self.kernels, cfg.max_seqs, device)
+        self.sampler = Sampler(self.kernels, cfg.max_seqs, self.device)
         budget = min(cfg.max_step_tokens, cfg.chunk_with_decode or cfg.max_step_tokens)
         if self.model.cut(0, budget) < 1:
             raise ValueError(f"no prompt portion of {budget} tokens (max_step_tokens, chunk_with_decode) ends where this "
@@ -88,7 +74,7 @@ class Engine:
         self._siblings: dict[Seq, list[Seq]] = {}         # n > 1: waiting until the first sequence's prompt is cached
         self._prompt_lp: dict[Seq, Logprobs] = {}         # sequences still gathering prompt log-probabilities
         self._inflight: _Launched | None = None           # the step that runs while the next one is scheduled
-        self._token_bufs = [torch.empty(cfg.max_seqs, dtype=torch.int32, pin_memory=device.type == "cuda")
+        self._token_bufs = [torch.empty(cfg.max_seqs, dtype=torch.int32, pin_memory=self.device.type == "cuda")
                             for _ in range(2)]
         self._turn = 0
         self.steps = 0
@@ -140,10 +126,8 @@ class Engine:
         rows = min(cfg.max_seqs, max(1, -(-cfg.max_step_tokens // longest)))
         per_row = min(longest, cfg.max_step_tokens // rows)
         pages = rows * -(-(per_row + 1) // cfg.page_size) + cfg.max_seqs
-        cache, runner = attach_cache(self.model, device=device, dtype=self.dtype, kernels=self.kernels,
-                                     cache_tokens=pages * cfg.page_size, graphs=False, page_size=cfg.page_size,
-                                     max_seqs=cfg.max_seqs, max_model_len=cfg.max_model_len,
-                                     max_step_tokens=cfg.max_step_tokens)
+        cache, runner = attach_cache(self.model, cache_tokens=pages * cfg.page_size, graphs=False,
+                                     **self._assembled.shape(cfg))
         sampler = Sampler(self.kernels, cfg.max_seqs, device)
         torch.cuda.synchronize(device)
         torch.cuda.reset_peak_memory_stats(device)
@@ -235,13 +219,20 @@ class Engine:
         closing.sort(key=lambda d: d.index)
         return closing + self._settle()
 
-    def stats(self) -> dict[str, int]:
+    def stats(self) -> dict:
         return {"waiting": len(self.sched) - self.sched.n_running, "running": self.sched.n_running,
                 "preemptions": self.sched.preemptions, "mixed_steps": self.sched.mixed_steps, "steps": self.steps,
                 "free_pages": min((g.pool.free for g in self.cache.groups), default=0),
                 "graphs": len(getattr(self.runner, "graphs", {})),
                 "prefix_tokens_saved": self.cache.tokens_saved,
-                "cached_pages": len(self.cache.prefix.entries) if self.cache.prefix is not None else 0}
+                "cached_pages": len(self.cache.prefix.entries) if self.cache.prefix is not None else 0,
+                "products": self.products()}
+
+    def products(self) -> dict[str, str]:
+        """What every matrix product with a choice took so far, as `kind:NxK:rows` -> form: the syntax
+        `EngineConfig.product_pins` accepts, so a timed run's choices can be pinned for the next."""
+        plan = getattr(self.kernels, "plan", None)
+        return plan.report() if plan is not None else {}
 
     def flush_prefix(self) -> list[TokenDelta]:
         """Drop the cached prompt blocks (core/holon/core/engine.py:418-420); the step in flight is committed first."""

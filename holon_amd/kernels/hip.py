@@ -4,6 +4,7 @@ library for them (std/holon_std/ops/units.py:229); everything else is this packa
 a missing library is built, and if that fails, loading raises."""
 from __future__ import annotations
 
+import copy
 import ctypes
 import sys
 import weakref
@@ -12,6 +13,7 @@ import torch
 
 from . import build as _build
 from .api import AttnRows
+from ..config.products import ProductPlan, row_bucket
 
 _P, _I, _L, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
 _DT = {torch.float32: 0, torch.bfloat16: 1}
@@ -91,8 +93,24 @@ class HipKernels:
         for name, args in sig.items():
             fn = getattr(lib, name)
             fn.argtypes, fn.restype = args, _I
-        self._mid_choice: dict[tuple, str] = {}    # (weight shape, at most 32 rows) -> the vendor product's faster form
+        self.plan = ProductPlan("own")            # which form a product takes where several serve it: see `configured`
         self._tiled_weights: dict[tuple, list] = {}   # weight shape -> weak (weight, tiled copy) pairs, see _alike
+        self._f32_result: bool | None = None      # whether torch has a float32 result for a bfloat16 product (probed once)
+
+    def configured(self, products: str = "own", pins=None) -> "HipKernels":
+        """The same kernels with product choices of their own: an engine's `products` mode and `product_pins`. The
+        library, and the record of tiled weights by shape, are shared; what a product took is per engine
+        (`plan.taken`)."""
+        other = copy.copy(self)
+        other.plan = ProductPlan(products, pins)
+        return other
+
+    def product_choice(self, kind: str, weight, rows: int, time=None) -> str:
+        """The one place a product's form is resolved: pinned, else by the engine's mode, else (mode `timed`, while
+        the engine starts and outside graph capture) by timing the candidates once."""
+        if time is not None and (not self.plan.resolving or torch.cuda.is_current_stream_capturing()):
+            time = None
+        return self.plan.choose(kind, tuple(weight.shape), row_bucket(rows), time)
 
     # -- plumbing -------------------------------------------------------------------------------------------------
     def _call(self, fn, *args) -> None:
@@ -196,8 +214,7 @@ class HipKernels:
         return y
 
     skinny_rows = 16          # up to this many rows (one tile of tokens) the hand-written weight-streaming product runs
-    _mid_forms = True         # whether steps of 17 to 64 rows may choose between the vendor product's two forms
-    deep_k = 8192             # from this K on, prompt portions of up to 1,024 rows choose between them as well
+    deep_k = 8192             # from this K on, prompt portions of up to 1,024 rows choose between the vendor's forms too
 
     def tile_weight(self, weight, scale=None):
         """A copy of `weight` [N, K] in the layout the few-row product streams fastest, or None when its shape or
@@ -254,8 +271,11 @@ class HipKernels:
             end.record()
             end.synchronize()
             del graph, keep
-        except torch.OutOfMemoryError:            # no room to try it: it does not win
+        except RuntimeError as e:                 # no room to try it (out of memory surfaces from the capture's end as
+            torch.cuda.synchronize()              # a plain RuntimeError too), or it cannot be recorded: it does not win
             torch.cuda.empty_cache()
+            print(f"holon_amd: a product candidate could not be timed and is not chosen: {str(e).splitlines()[0]}",
+                  file=sys.stderr)
             return float("inf")
         return start.elapsed_time(end) / (replays * len(calls))
 
@@ -320,22 +340,28 @@ class HipKernels:
         """x W^T by the vendor library, rounded once to the operands' type. For steps of 17 to 64 bfloat16 rows the
         library's choice of kernel has holes at some shapes (a deep, narrow weight, 5120 x 25600: 145 us, where its
         product of the same operands with a float32 result takes 83, two such products over the halves of K 73, and
-        the weights alone would stream in 42), so for such steps the forms are timed once per weight shape and row
-        bucket, outside graph capture, and the fastest is kept. Over deep weights (K of 8,192 and more) the same
-        holds for prompt portions of up to 1,024 rows (the same weight at 544 rows: 260 us, over the halves of K 213;
-        at 256 rows 263, with a float32 result 184), in buckets of 128, 256, 512 and 1,024 rows. All forms accumulate
-        in float32 and round once."""
+        the weights alone would stream in 42); over deep weights (K of 8,192 and more) the same holds for prompt
+        portions of up to 1,024 rows. Which form such a step takes is a product choice of kind `vendor` (pinned, or
+        timed at start in mode `timed`, else the plain form). All forms accumulate in float32 and round once."""
         m, k = x.shape[0], weight.shape[1]
-        if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and self._mid_forms
+        if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
                 and (16 < m <= 64 or (64 < m <= 1024 and k >= self.deep_k))):
             return torch.matmul(x, weight.t())
-        key = (tuple(weight.shape), m <= 32 if m <= 64 else 1 << (m - 1).bit_length())
-        form = self._mid_choice.get(key)
-        if form is None:
-            if torch.cuda.is_current_stream_capturing():
-                return torch.matmul(x, weight.t())
-            form = self._mid_choice[key] = self._time_mid_forms(x, weight)
+        form = self.product_choice("vendor", weight, m, lambda: self._time_mid_forms(x, weight))
+        if form != "bf16" and not self.has_f32_result():
+            raise KernelError(f"product form {form!r} needs torch.mm(..., out_dtype=float32), which this torch lacks")
         return self._MID_FORMS[form](x, weight)
+
+    def has_f32_result(self) -> bool:
+        """Whether this torch multiplies bfloat16 operands into a float32 result; probed once, eagerly."""
+        if self._f32_result is None:
+            try:
+                a = torch.zeros((32, 64), dtype=torch.bfloat16, device="cuda")
+                torch.mm(a, a.t(), out_dtype=torch.float32)
+                self._f32_result = True
+            except (RuntimeError, TypeError):
+                self._f32_result = False
+        return self._f32_result
 
     @staticmethod
     def _two_halves(x, weight):
@@ -348,16 +374,14 @@ class HipKernels:
                   "f32x2": lambda x, w: HipKernels._two_halves(x, w)}
 
     def _time_mid_forms(self, x, weight) -> str:
+        if not self.has_f32_result():
+            return "bf16"
         pairs = self._alike(weight, None)
         took = {}
-        try:
-            for name, fn in self._MID_FORMS.items():
-                if name == "f32x2" and weight.shape[1] % 512:
-                    continue
-                took[name] = self._graph_time(self._in_turn(pairs, lambda w, _t, fn=fn: fn(x, w)))
-        except (RuntimeError, TypeError):           # this torch has no float32 result for a bfloat16 product
-            self._mid_forms = False
-            return "bf16"
+        for name, fn in self._MID_FORMS.items():
+            if name == "f32x2" and weight.shape[1] % 512:
+                continue
+            took[name] = self._graph_time(self._in_turn(pairs, lambda w, _t, fn=fn: fn(x, w)))
         best = min(took, key=took.get)
         return best if took[best] < 0.92 * took["bf16"] else "bf16"
 
@@ -370,13 +394,8 @@ class HipKernels:
         if not (tiled is not None and weight.dtype == torch.bfloat16 and 16 < rows <= 64
                 and self.lib.holon_gemm_rows_supported(rows, n // 2 if gated else n, k, int(gated))):
             return False
-        key = ("rows", (n, k), rows <= 32, bool(gated))
-        use = self._mid_choice.get(key)
-        if use is None:
-            if torch.cuda.is_current_stream_capturing():
-                return False
-            use = self._mid_choice[key] = self._time_rows(rows, weight, tiled, gated)
-        return use == "rows"
+        return self.product_choice("glu" if gated else "rows", weight, rows,
+                                   lambda: self._time_rows(rows, weight, tiled, gated)) == "rows"
 
     def _rows_product(self, x, weight, tiled, gated, to_f32=False):
         m, k = x.shape
@@ -403,12 +422,7 @@ class HipKernels:
         splits = self.lib.holon_gemm_rows_splits(m, n, k)
         if not splits:
             return None
-        key = ("parts", (n, k), m <= 32 if m <= 64 else 128)
-        use = self._mid_choice.get(key)
-        if use is None:
-            if torch.cuda.is_current_stream_capturing():
-                return None
-            use = self._mid_choice[key] = self._time_parts(x, weight, tiled, splits)
+        use = self.product_choice("parts", weight, m, lambda: self._time_parts(x, weight, tiled, splits))
         return self._rows_parts(x, weight, tiled, splits) if use == "parts" else None
 
     def _rows_parts(self, x, weight, tiled, splits):

@@ -127,3 +127,52 @@ def test_command_line_makes_engine_settings_and_takes_auto_for_the_context(tmp_p
     (tmp_path / "config.json").write_text(json.dumps({"architectures": ["Qwen3ForCausalLM"], "max_position_embeddings": 512}))
     assert cli.engine_config(str(tmp_path), ap.parse_args(["--max-model-len", "auto"])).max_model_len == 512
     assert cli.engine_config(str(tmp_path), ap.parse_args(["--max-model-len", "100"])).max_model_len == 100
+
+
+def test_product_choices_resolve_pinned_then_by_mode_then_timed_at_start_only():
+    """Which form a matrix product takes where several serve it: a pin wins, else the engine's mode; mode `timed`
+    times once while the engine starts and falls back to this package's form, recorded as untimed, afterwards. The
+    reference's order is pinned, preferred, priority (core/holon/core/build.py:89-106)."""
+    import argparse
+
+    from holon_amd import cli
+    from holon_amd.config.products import ProductError, ProductPlan, key_of, row_bucket
+    assert [row_bucket(r) for r in (17, 32, 33, 64, 65, 128, 129, 1000)] == [32, 32, 64, 64, 128, 128, 256, 1024]
+    assert key_of("parts", (4096, 12288), 64) == "parts:4096x12288:64"
+    calls = []
+
+    def timer():
+        calls.append(1)
+        return "vendor"
+    own = ProductPlan("own", {"parts:8x16:64": "vendor"})
+    assert own.choose("parts", (8, 16), 64, timer) == "vendor" and own.how["parts:8x16:64"] == "pinned"
+    assert own.choose("parts", (8, 16), 32, timer) == "parts" and own.choose("vendor", (8, 16), 32, timer) == "bf16"
+    assert own.choose("glu", (8, 16), 32) == "rows" and not calls
+    vendor = ProductPlan("vendor")
+    assert [vendor.choose(k, (8, 16), 32, timer) for k in ("rows", "glu", "parts", "vendor")] == ["vendor"] * 3 + ["bf16"]
+    timed = ProductPlan("timed", {"rows:8x16:32": "rows"})
+    assert timed.choose("parts", (8, 16), 32, timer) == "parts" and timed.how["parts:8x16:32"] == "untimed" and not calls
+    timed.resolving = True
+    assert timed.choose("parts", (8, 16), 32, timer) == "parts" and not calls          # kept: one answer a key, for good
+    assert timed.choose("parts", (8, 16), 64, timer) == "vendor" and calls == [1] and timed.how["parts:8x16:64"] == "timed"
+    assert timed.choose("parts", (8, 16), 64, timer) == "vendor" and calls == [1]
+    assert timed.choose("rows", (8, 16), 32, timer) == "rows" and calls == [1]          # pinned: not timed
+    assert timed.report() == {"parts:8x16:32": "parts", "parts:8x16:64": "vendor", "rows:8x16:32": "rows"}
+    assert ProductPlan("own", timed.report()).choose("parts", (8, 16), 64) == "vendor"   # a report is a set of pins
+    timed.resolving = True
+    with pytest.raises(ProductError, match="not one of"):
+        timed.choose("vendor", (8, 16), 32, lambda: "rows")
+    for bad in ({"parts:8x16": "parts"}, {"shares:8x16:32": "parts"}, {"parts:8x16:32": "f32"}, {"parts:ax16:32": "parts"}):
+        with pytest.raises(ProductError):
+            ProductPlan("own", bad)
+    with pytest.raises(ProductError):
+        ProductPlan("fastest")
+    with pytest.raises(ValueError, match="products"):
+        EngineConfig(model="m", products="fastest")
+    with pytest.raises(ValueError):
+        EngineConfig(model="m", product_pins={"parts:8x16:32": "rows"})
+    ap = argparse.ArgumentParser()
+    cli.engine_flags(ap)
+    got = cli.engine_config("m", ap.parse_args(["--products", "timed", "--product-pins",
+                                                "parts:8x16:32=vendor, vendor:8x16:512=f32x2"]))
+    assert got.products == "timed" and got.product_pins == {"parts:8x16:32": "vendor", "vendor:8x16:512": "f32x2"}

@@ -363,10 +363,15 @@ def test_product_for_17_to_64_rows_over_many_tiles(hip):
     for m, k, n in ((17, 256, 16384), (64, 4096, 24576), (33, 1024, 16512), (48, 512, 65536), (64, 768, 65664), (20, 256, 131072)):
         x, w = _randn(m, k, dtype=bf, seed=80), _randn(n, k, dtype=bf, seed=81, scale=0.05)
         tiled = hip.tile_weight(w)
-        hip.serves_rows(m, w, tiled)                                                   # times the two products once ...
-        key = ("rows", (n, k), m <= 32, False)
-        assert hip._mid_choice[key] in ("rows", "vendor")
-        hip._mid_choice[key] = "rows"                                                  # ... here the kernel is what is tested
+        timed = hip.configured("timed")
+        assert timed.serves_rows(m, w, tiled)                                          # outside an engine's start: untimed, ours
+        assert timed.plan.how == {f"rows:{n}x{k}:{32 if m <= 32 else 64}": "untimed"}
+        timed = hip.configured("timed")
+        timed.plan.resolving = True                                                    # as while an engine starts: timed once
+        timed.serves_rows(m, w, tiled)
+        assert timed.plan.how == {f"rows:{n}x{k}:{32 if m <= 32 else 64}": "timed"} and timed.plan.seconds > 0
+        assert timed.plan.report()[f"rows:{n}x{k}:{32 if m <= 32 else 64}"] in ("rows", "vendor")
+        assert not hip.configured("vendor").serves_rows(m, w, tiled)
         assert hip.serves_rows(m, w, tiled) and not hip.serves_rows(16, w, tiled) and not hip.serves_rows(65, w, tiled)
         want = x.double() @ w.double().T
         got = hip.linear(x, w, None, tiled)
@@ -378,8 +383,9 @@ def test_product_for_17_to_64_rows_over_many_tiles(hip):
     for m, k, inter in ((64, 4096, 12288), (17, 256, 8192), (40, 1024, 8320), (33, 512, 16384), (64, 768, 16512)):   # the last two: eight waves a block
         x, w = _randn(m, k, dtype=bf, seed=82), _randn(2 * inter, k, dtype=bf, seed=83, scale=0.05)
         tiled = hip.tile_weight(w)
-        hip._mid_choice[("rows", (2 * inter, k), m <= 32, True)] = "rows"
         assert hip.serves_rows(m, w, tiled, gated=True)
+        pinned = hip.configured("own", {f"glu:{2 * inter}x{k}:{32 if m <= 32 else 64}": "vendor"})
+        assert not pinned.serves_rows(m, w, tiled, gated=True) and pinned.plan.how.popitem()[1] == "pinned"
         exact = PLAIN.silu_mul(PLAIN.linear(x.double(), w.double()))
         got = hip.linear_silu_mul(x, w, tiled)
         assert got is not None and got.shape == (m, inter) and H.op_budget_usage(got, exact, bf, k) <= 1, (m, k, inter)
@@ -390,7 +396,6 @@ def test_product_for_17_to_64_rows_over_many_tiles(hip):
     assert not hip.serves_rows(32, w, tiled) and not hip.serves_rows(32, w, None)      # 256 tiles: the vendor library's
     w = _randn(16384, 384, dtype=bf, seed=85)
     assert not hip.serves_rows(32, w, hip.tile_weight(w))                              # K no multiple of 256
-    hip._mid_choice.clear()
 
 
 def test_product_in_shares_of_k_for_narrow_weights(hip):
@@ -434,10 +439,13 @@ def test_product_in_shares_of_k_for_narrow_weights(hip):
         assert torch.equal(plain_res, res_a) and H.op_budget_usage(normed_a, plain_normed.double(), bf, 1) <= 1
     x, w = _randn(32, 4096, dtype=bf, seed=94), _randn(4096, 4096, dtype=bf, seed=95, scale=0.05)
     tiled = hip.tile_weight(w)
-    got = hip.linear_parts(x, w, tiled)                                                   # timed once, then kept
-    assert hip._mid_choice[("parts", (4096, 4096), True)] in ("parts", "vendor")
-    assert (got is None) == (hip._mid_choice[("parts", (4096, 4096), True)] == "vendor")
-    hip._mid_choice[("parts", (4096, 4096), True)] = "parts"
+    timed = hip.configured("timed")
+    timed.plan.resolving = True
+    got = timed.linear_parts(x, w, tiled)                                                 # timed once, then kept
+    assert timed.plan.report()["parts:4096x4096:32"] in ("parts", "vendor")
+    assert (got is None) == (timed.plan.report()["parts:4096x4096:32"] == "vendor")
+    assert hip.configured("vendor").linear_parts(x, w, tiled) is None
+    assert hip.configured("vendor", {"parts:4096x4096:32": "parts"}).linear_parts(x, w, tiled).shape == (8, 32, 4096)
     assert hip.linear_parts(x, w, tiled).shape == (8, 32, 4096)
     assert hip.linear_parts(x[:16].contiguous(), w, tiled) is None and hip.linear_parts(x, w, None) is None
     assert hip.linear_parts(_randn(129, 4096, dtype=bf, seed=99), w, tiled) is None            # beyond 128 rows
@@ -450,7 +458,6 @@ def test_product_in_shares_of_k_for_narrow_weights(hip):
         hip._rows_parts(x.cpu(), w[:, :4096].contiguous(), tiled, 8)
     with pytest.raises(KernelError):
         hip.add_rmsnorm(torch.zeros(8, 32, 4000, device="cuda"), _randn(32, 4096, dtype=bf), _randn(4096, dtype=bf), 1e-5)
-    hip._mid_choice.clear()
 
 
 def test_choices_are_timed_over_the_same_shaped_weights_of_other_layers(hip):
@@ -487,22 +494,22 @@ def test_vendor_product_forms_for_steps_of_17_to_64_rows(hip):
     for m, k, n in ((32, 25600, 5120), (24, 4096, 6144), (64, 1024, 512), (300, 25600, 5120), (1000, 8192, 512)):
         x, w = _randn(m, k, dtype=bf, seed=70), _randn(n, k, dtype=bf, seed=71, scale=0.02)
         want = x.double() @ w.double().T
-        key = ((n, k), m <= 32 if m <= 64 else {300: 512, 1000: 1024}[m])
-        hip._mid_choice.pop(key, None)
-        got = hip.linear(x, w)
-        assert hip._mid_choice[key] in ("bf16", "f32", "f32x2")           # timed and kept
+        key = f"vendor:{n}x{k}:{32 if m <= 32 else 1 << (m - 1).bit_length()}"
+        timed = hip.configured("timed")
+        timed.plan.resolving = True
+        got = timed.linear(x, w)
+        assert timed.plan.report()[key] in ("bf16", "f32", "f32x2")       # timed and kept
         for form in ("bf16", "f32", "f32x2"):
-            hip._mid_choice[key] = form
-            y = hip.linear(x, w)
+            y = hip.configured("own", {key: form}).linear(x, w)
             assert y.dtype == bf and H.op_budget_usage(y, want, bf, k) <= 1, (m, k, n, form)
-            assert torch.equal(hip.linear(x, w, torch.float32), y.float())
+            assert torch.equal(hip.configured("own", {key: form}).linear(x, w, torch.float32), y.float())
+        assert torch.equal(hip.linear(x, w), hip.configured("vendor").linear(x, w))          # both: the plain form
         assert H.op_budget_usage(got, want, bf, k) <= 1
-    before = dict(hip._mid_choice)
-    hip.linear(_randn(300, 4096, dtype=bf, seed=72), _randn(512, 4096, dtype=bf, seed=73))      # a shallow weight, and
-    hip.linear(_randn(1025, 8192, dtype=bf, seed=74), _randn(512, 8192, dtype=bf, seed=75))     # more rows: not timed
-    assert hip._mid_choice == before
-    assert ((5120, 25600), False) not in hip._mid_choice                   # the other bucket was never asked for
-    hip._mid_choice.clear()
+    timed = hip.configured("timed")
+    timed.plan.resolving = True
+    timed.linear(_randn(300, 4096, dtype=bf, seed=72), _randn(512, 4096, dtype=bf, seed=73))    # a shallow weight, and
+    timed.linear(_randn(1025, 8192, dtype=bf, seed=74), _randn(512, 8192, dtype=bf, seed=75))   # more rows: no choice
+    assert timed.plan.report() == {}
 
 
 def test_float32_product_is_true_32_bit_and_its_order_is_fixed(hip):
@@ -786,7 +793,6 @@ def test_kernels_refuse_what_they_do_not_serve(hip):
     w, other = _randn(512, 1024, dtype=bf, seed=1), _randn(256, 1024, dtype=bf, seed=2)
     tiled = hip.tile_weight(w)
     big = _randn(16384, 256, dtype=bf, seed=3)
-    hip._mid_choice[("rows", (16384, 256), True, False)] = "rows"
     for rows, weight in ((4, w), (32, big)):
         with pytest.raises(KernelError):
             hip.linear(torch.zeros(rows, weight.shape[1], dtype=bf), weight, None, hip.tile_weight(weight))   # rows on the CPU
@@ -798,4 +804,3 @@ def test_kernels_refuse_what_they_do_not_serve(hip):
         hip.linear_add(_randn(4, 1024, dtype=bf), w, hip.tile_weight(other), _randn(4, 512, dtype=bf))
     with pytest.raises(KernelError):
         hip.linear_add(_randn(4, 1024, dtype=bf), w, tiled, torch.zeros(4, 512, dtype=bf))   # residual on the CPU
-    hip._mid_choice.clear()

@@ -83,25 +83,19 @@ def test_portions_of_17_to_64_rows_with_some_rows_wanted_over_partial_sums(folde
     residual stream and from its pending term, the last down projection's shares, alike."""
     from holon_amd.engine.loading import load_model
     from holon_amd.engine.replay import Replayer
-    from holon_amd.kernels import load_hip
-    hidden, inter, wide = WIDE["hidden_size"], WIDE["intermediate_size"], WIDE["num_attention_heads"] * WIDE["head_dim"]
-    for few in (True, False):
-        for shape in ((hidden, wide), (hidden, inter)):
-            load_hip()._mid_choice[("parts", shape, few)] = "parts"
-    try:
-        ids = _requests()["r1"]                                           # 130 tokens
-        loaded = load_model(folder, device="cuda", dtype="bfloat16", page_size=16, max_seqs=4, max_model_len=512,
-                            max_step_tokens=512, cache_tokens=256)
-        trace = H.Trace()
-        trace.add([("r1", 0, ids[:40], [0, 39])])
-        trace.add([("r1", 40, ids[40:57], [16])])
-        trace.add([("r1", 57, ids[57:121], [3, 40, 63])])
-        trace.add([("r1", 121, ids[121:], [len(ids) - 122])], end=["r1"])  # nine rows: the few-row kernels
-        got = H.run_trace(Replayer(loaded), trace)
-        assert len(got) == 7
-        _check(folder, "bfloat16", {"r1": ids}, got, "wide bfloat16, some rows of portions over partial sums")
-    finally:
-        load_hip()._mid_choice.clear()
+    ids = _requests()["r1"]                                           # 130 tokens
+    loaded = load_model(folder, device="cuda", dtype="bfloat16", page_size=16, max_seqs=4, max_model_len=512,
+                        max_step_tokens=512, cache_tokens=256, products="own")
+    trace = H.Trace()
+    trace.add([("r1", 0, ids[:40], [0, 39])])
+    trace.add([("r1", 40, ids[40:57], [16])])
+    trace.add([("r1", 57, ids[57:121], [3, 40, 63])])
+    trace.add([("r1", 121, ids[121:], [len(ids) - 122])], end=["r1"])  # nine rows: the few-row kernels
+    got = H.run_trace(Replayer(loaded), trace)
+    assert len(got) == 7
+    taken = loaded.kernels.plan.report()
+    assert taken["parts:4096x4096:64"] == taken["parts:4096x12288:64"] == taken["parts:4096x12288:32"] == "parts", taken
+    _check(folder, "bfloat16", {"r1": ids}, got, "wide bfloat16, some rows of portions over partial sums")
 
 
 def _wide_batch_requests() -> dict[str, tuple[list[int], int]]:
@@ -143,27 +137,21 @@ def _wide_batch_trace(requests: dict[str, tuple[list[int], int]], budget: int) -
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("products", ["ours", "vendor"])
+@pytest.mark.parametrize("products", ["own", "vendor"])
 def test_sixty_four_rows_decode_together_from_graphs(folder, dtype, products):
     """Decode steps of 64 rows shrinking to 7, replayed from graphs of every batch bucket on the way (all but the
     first with padding rows) and of three length buckets (1,024, 2,048, 4,096): the products for more than 16 rows,
     the decode attention with 64 rows, the few-row kernels below. Once with the kernels of our own for 17 to 64 rows
     (the gated product shares the rows through LDS and reads the folded weights over rows normed without the norm's
     weight; the output and down projections split K over blocks and hand partial sums to the norm that adds them),
-    once with the vendor library's products: which a run takes is otherwise decided by timing them. Every row's
-    logits in every step against the plain model."""
+    once with the vendor library's products (the engine's `products` setting). Every row's logits in every step
+    against the plain model."""
     from holon_amd.engine.loading import load_model
     from holon_amd.engine.replay import Replayer
-    from holon_amd.kernels import load_hip
-    hidden, inter, wide = WIDE["hidden_size"], WIDE["intermediate_size"], WIDE["num_attention_heads"] * WIDE["head_dim"]
-    for few in (True, False):
-        load_hip()._mid_choice[("rows", (2 * inter, hidden), few, True)] = "rows" if products == "ours" else "vendor"
-        for shape in ((hidden, wide), (hidden, inter)):
-            load_hip()._mid_choice[("parts", shape, few)] = "parts" if products == "ours" else "vendor"
     requests = _wide_batch_requests()
     trace = _wide_batch_trace(requests, 2304)
     loaded = load_model(folder, device="cuda", dtype=dtype, page_size=16, max_seqs=64, max_model_len=2304,
-                        max_step_tokens=2304, cache_tokens=H.peak_live_tokens(trace), graphs=True)
+                        max_step_tokens=2304, cache_tokens=H.peak_live_tokens(trace), graphs=True, products=products)
     rep = Replayer(loaded)
     got = H.run_trace(rep, trace)
     assert len(got) == 64 + sum(len(ids) - p for ids, p in requests.values())
@@ -173,21 +161,41 @@ def test_sixty_four_rows_decode_together_from_graphs(folder, dtype, products):
     _check(folder, dtype, {rid: ids for rid, (ids, _) in requests.items()}, got, f"wide {dtype} 64 rows")
     rep.cache.check()
     assert all(g.pool.free == g.pool.usable for g in rep.cache.groups)
-    load_hip()._mid_choice.clear()
+    if dtype == "bfloat16":
+        taken = set(loaded.kernels.plan.report().values())
+        assert taken <= ({"rows", "parts", "bf16"} if products == "own" else {"vendor", "bf16"}), loaded.kernels.plan.report()
 
 
-def _force_our_products(on: bool) -> None:
-    """The kernels of our own for 17 to 64 rows at the wide sizes (gated product through LDS, output and down
-    projections in shares of K), instead of what timing them against the vendor library's would choose."""
-    from holon_amd.kernels import load_hip
-    hidden, inter, wide = WIDE["hidden_size"], WIDE["intermediate_size"], WIDE["num_attention_heads"] * WIDE["head_dim"]
-    choice = load_hip()._mid_choice
-    choice.clear()
-    if on:
-        for few in (True, False):
-            choice[("rows", (2 * inter, hidden), few, True)] = "rows"
-            for shape in ((hidden, wide), (hidden, inter)):
-                choice[("parts", shape, few)] = "parts"
+def test_timed_choices_are_made_at_start_reported_and_repeatable_when_pinned(folder):
+    """Mode `timed` times every product with a choice while the model is put together, in every row bucket the engine
+    can reach, and never later; what each took is reported in the syntax pins are given in. Two further launches with
+    those pins (whatever their mode) then compute a 64-row decode trace bit for bit alike."""
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    requests = {rid: v for rid, v in _wide_batch_requests().items() if rid not in ("long", "mid")}
+    trace = _wide_batch_trace(requests, 2304)
+    shape = dict(device="cuda", dtype="bfloat16", page_size=16, max_seqs=64, max_model_len=512, max_step_tokens=2304,
+                 cache_tokens=H.peak_live_tokens(trace), graphs=True)
+    timed = load_model(folder, products="timed", **shape)
+    plan = timed.kernels.plan
+    taken = plan.report()
+    assert plan.seconds > 0 and not plan.resolving and set(plan.how.values()) == {"timed"}, plan.how
+    for key in ("glu:24576x4096:32", "glu:24576x4096:64", "parts:4096x12288:32", "parts:4096x12288:64",
+                "parts:4096x4096:64", "parts:4096x12288:128", "vendor:6144x4096:64"):
+        assert key in taken or key.startswith("vendor:"), (key, taken)
+    first = H.run_trace(Replayer(timed), trace)
+    assert plan.report() == taken and set(plan.how.values()) == {"timed"}        # nothing was chosen inside a step
+    del timed
+    again = []
+    for mode in ("own", "vendor"):
+        loaded = load_model(folder, products=mode, product_pins=taken, **shape)
+        again.append(H.run_trace(Replayer(loaded), trace))
+        assert loaded.kernels.plan.report() == taken, (mode, loaded.kernels.plan.report())
+        assert set(loaded.kernels.plan.how.values()) == {"pinned"}
+        del loaded
+    for key, row in first.items():
+        assert torch.equal(row, again[0][key]) and torch.equal(row, again[1][key]), key
+    _check(folder, "bfloat16", {rid: ids for rid, (ids, _) in requests.items()}, first, "wide bfloat16 timed products")
 
 
 def test_a_hundred_rows_decode_together(folder):
@@ -195,27 +203,21 @@ def test_a_hundred_rows_decode_together(folder):
     as partial sums over shares of K, which serve up to 128 rows: every row's logits against the plain model."""
     from holon_amd.engine.loading import load_model
     from holon_amd.engine.replay import Replayer
-    from holon_amd.kernels import load_hip
-    hidden, inter, wide = WIDE["hidden_size"], WIDE["intermediate_size"], WIDE["num_attention_heads"] * WIDE["head_dim"]
-    for shape in ((hidden, wide), (hidden, inter)):
-        load_hip()._mid_choice[("parts", shape, 128)] = "parts"
-    try:
-        requests = {f"q{i}": (H.random_ids(1 + (5 * i) % 37 + (3 if i < 70 else 2), WIDE["vocab_size"], 1500 + i),
-                              1 + (5 * i) % 37) for i in range(100)}          # 70 decode three tokens, 30 two
-        trace = _wide_batch_trace(requests, 2304)
-        loaded = load_model(folder, device="cuda", dtype="bfloat16", page_size=16, max_seqs=128, max_model_len=256,
-                            max_step_tokens=2304, cache_tokens=H.peak_live_tokens(trace), graphs=True)
-        rep = Replayer(loaded)
-        got = H.run_trace(rep, trace)
-        assert len(got) == 100 + 70 * 3 + 30 * 2
-        assert {(128, 1024), (96, 1024)} <= set(loaded.runner.graphs), set(loaded.runner.graphs)
-        _check(folder, "bfloat16", {rid: ids for rid, (ids, _) in requests.items()}, got, "wide bfloat16 100 rows")
-        rep.cache.check()
-    finally:
-        load_hip()._mid_choice.clear()
+    requests = {f"q{i}": (H.random_ids(1 + (5 * i) % 37 + (3 if i < 70 else 2), WIDE["vocab_size"], 1500 + i),
+                          1 + (5 * i) % 37) for i in range(100)}          # 70 decode three tokens, 30 two
+    trace = _wide_batch_trace(requests, 2304)
+    loaded = load_model(folder, device="cuda", dtype="bfloat16", page_size=16, max_seqs=128, max_model_len=256,
+                        max_step_tokens=2304, cache_tokens=H.peak_live_tokens(trace), graphs=True, products="own")
+    rep = Replayer(loaded)
+    got = H.run_trace(rep, trace)
+    assert len(got) == 100 + 70 * 3 + 30 * 2
+    assert {(128, 1024), (96, 1024)} <= set(loaded.runner.graphs), set(loaded.runner.graphs)
+    assert loaded.kernels.plan.report()["parts:4096x12288:128"] == "parts"
+    _check(folder, "bfloat16", {rid: ids for rid, (ids, _) in requests.items()}, got, "wide bfloat16 100 rows")
+    rep.cache.check()
 
 
-@pytest.mark.parametrize("products", ["timed", "ours"])
+@pytest.mark.parametrize("products", ["timed", "own"])
 def test_engine_at_the_wide_sizes_with_everything_on(folder, products):
     """The whole engine in bfloat16 at the measured layer sizes (matrix-core attention, the few-row products over
     tiled weights, the residual add and the gated form inside them). One step in flight changes no launch, so it must
@@ -225,12 +227,14 @@ def test_engine_at_the_wide_sizes_with_everything_on(folder, products):
     held to the plain model's own greedy decoding in bfloat16."""
     from holon_amd.config import EngineConfig, SamplingParams
     from holon_amd.engine.engine import Engine
-    _force_our_products(products == "ours")
     start = H.random_ids(40, WIDE["vocab_size"], 300)
     prompts = [start[: 8 + 4 * (i % 9)] + H.random_ids(3 + 5 * i, WIDE["vocab_size"], 301 + i) for i in range(20)]
     shape = dict(model=str(folder), device="cuda", dtype="bfloat16", page_size=16, max_seqs=24, max_model_len=256,
-                 max_step_tokens=256, cache_tokens=24 * 256)
+                 max_step_tokens=256, cache_tokens=24 * 256, products=products)
     bare = Engine(EngineConfig(overlap=False, graphs=False, prefix_cache=False, **shape))
+    if products == "timed":                  # the next engines take what this one's timings chose: pinned, repeatable
+        assert bare.kernels.plan.seconds > 0 and set(bare.kernels.plan.how.values()) == {"timed"}
+        shape["product_pins"] = bare.products()
     ahead = Engine(EngineConfig(overlap=True, graphs=False, prefix_cache=False, **shape))
     for params in (SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True),
                    SamplingParams(temperature=0.8, top_k=40, top_p=0.95, seed=5, max_tokens=24, ignore_eos=True)):
@@ -242,7 +246,8 @@ def test_engine_at_the_wide_sizes_with_everything_on(folder, products):
         for prompt, got in zip(prompts, full.generate(prompts, params)):
             H.assert_greedy_follows(plain, prompt, got)
     assert full.cache.tokens_saved > 0 and full.stats()["graphs"] >= 1 and full.runner.graph_replays > 10
-    _force_our_products(False)
+    how = {"timed": "pinned", "own": "own"}[products]
+    assert full.stats()["products"] == bare.products() and set(full.kernels.plan.how.values()) == {how}, full.kernels.plan.how
 
 
 def test_long_context_attention_kernels():
