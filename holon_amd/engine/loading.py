@@ -155,13 +155,15 @@ def time_products(a: Assembled, cfg: EngineConfig) -> None:
 def load_model(folder: str | pathlib.Path, *, device: str | torch.device = "cuda", dtype: str | torch.dtype = "bfloat16",
                kernels=None, page_size: int = 16, max_seqs: int = 64, max_model_len: int = 8192,
                max_step_tokens: int = 4096, cache_tokens: int | None = None, graphs: bool = False,
-               products: str = "own", product_pins: dict | None = None, decode_weight_copy: bool = True) -> Loaded:
-    """Read config.json, pick the model by its architecture name, load the weights, allocate the cache."""
+               products: str = "own", product_pins: dict | None = None, decode_weight_copy: bool = True,
+               random_config: dict | None = None, seed: int = 0) -> Loaded:
+    """Read config.json, pick the model by its architecture name, load the weights, allocate the cache. With
+    `random_config` (a config.json as a dict) no folder is read: the weights are drawn on the device from `seed`."""
     dtype_name = dtype if isinstance(dtype, str) else {v: k for k, v in TORCH_DTYPES.items()}[torch_dtype(dtype)]
     cfg = EngineConfig(model=str(folder), device=str(device), dtype=dtype_name, page_size=page_size, max_seqs=max_seqs,
                        max_model_len=max_model_len, max_step_tokens=max_step_tokens, graphs=graphs, products=products,
                        product_pins=product_pins, decode_weight_copy=decode_weight_copy)
-    a = assemble(cfg, kernels)
+    a = assemble(cfg, kernels, random_config=random_config, seed=seed)
     tokens = cache_tokens if cache_tokens is not None else max_model_len
     cache, runner = attach_cache(a.model, cache_tokens=tokens, graphs=graphs, **a.shape(cfg))
     return Loaded(a.config, a.spec, a.model, cache, runner, a.kernels, a.device, a.dtype)

@@ -36,7 +36,8 @@ def random_tensor(name: str, decl: ParamDecl, seed: int, device: torch.device | 
     return x.bfloat16().float()
 
 
-def _meta_model(config_json: dict[str, Any]):
+def meta_model(config_json: dict[str, Any]):
+    """(typed configuration, spec, the model built without storage): what tensors a configuration has."""
     from ..model import build_model
     cfg, spec = resolve(config_json)
     build = Build(kernels=None, device=torch.device("meta"), dtype=torch.float32, max_model_len=2)
@@ -46,7 +47,7 @@ def _meta_model(config_json: dict[str, Any]):
 def write_random_model(config_json: dict[str, Any], seed: int, folder: str | pathlib.Path,
                        store_dtype: torch.dtype = torch.bfloat16) -> pathlib.Path:
     """A model folder (config.json, model.safetensors) for `config_json`, every tensor under its checkpoint name."""
-    cfg, spec, model = _meta_model(config_json)
+    cfg, spec, model = meta_model(config_json)
     folder = pathlib.Path(folder)
     folder.mkdir(parents=True, exist_ok=True)
     tensors = {}

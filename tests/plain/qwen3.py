@@ -73,13 +73,20 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: 
     group = hq // k.shape[1]
     k32 = wide(k).repeat_interleave(group, dim=1)
     v32 = wide(v).repeat_interleave(group, dim=1)
-    scores = torch.einsum("qhd,khd->hqk", wide(q), k32) / d ** 0.5
     pos = torch.arange(t, device=q.device)
-    hidden = pos[None, :] > pos[:, None]
-    if window:
-        hidden = hidden | (pos[:, None] - pos[None, :] >= window)
-    probs = scores.masked_fill(hidden, float("-inf")).softmax(dim=-1)
-    return torch.einsum("hqk,khd->qhd", probs, v32).to(q.dtype)
+    out = []
+    for lo in range(0, t, QUERY_ROWS):     # a query row's result does not depend on the other rows: the rows are taken
+        rows = pos[lo: lo + QUERY_ROWS]    # some at a time only so that the [heads, rows, T] scores fit in memory
+        scores = torch.einsum("qhd,khd->hqk", wide(q[lo: lo + QUERY_ROWS]), k32) / d ** 0.5
+        hidden = pos[None, :] > rows[:, None]
+        if window:
+            hidden = hidden | (rows[:, None] - pos[None, :] >= window)
+        probs = scores.masked_fill(hidden, float("-inf")).softmax(dim=-1)
+        out.append(torch.einsum("hqk,khd->qhd", probs, v32).to(q.dtype))
+    return torch.cat(out)
+
+
+QUERY_ROWS = 4096
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
@@ -169,6 +176,16 @@ class PlainQwen3:
     def __init__(self, folder: str | pathlib.Path, dtype: torch.dtype = torch.float32, device: str = "cpu") -> None:
         self.cfg, self.weights = read_folder(folder, dtype, device)
         self.work = torch.float64 if dtype == torch.float64 else torch.float32
+
+    @classmethod
+    def from_tensors(cls, cfg: dict, weights: dict[str, torch.Tensor], dtype: torch.dtype = torch.float32
+                     ) -> "PlainQwen3":
+        """The plain model over tensors that are already in memory (config.json's keys, Hugging Face tensor names),
+        cast to `dtype` where they lie: for models too large to write as a folder in a test."""
+        self = cls.__new__(cls)
+        self.cfg, self.weights = dict(cfg), {name: t.to(dtype) for name, t in weights.items()}
+        self.work = torch.float64 if dtype == torch.float64 else torch.float32
+        return self
 
     @torch.no_grad()
     def logits(self, ids: list[int]) -> torch.Tensor:

@@ -190,7 +190,8 @@ def test_timed_choices_are_made_at_start_reported_and_repeatable_when_pinned(fol
     for mode in ("own", "vendor"):
         loaded = load_model(folder, products=mode, product_pins=taken, **shape)
         again.append(H.run_trace(Replayer(loaded), trace))
-        assert loaded.kernels.plan.report() == taken, (mode, loaded.kernels.plan.report())
+        reached = loaded.kernels.plan.report()                                     # what the trace's steps came to
+        assert reached and reached.items() <= taken.items(), (mode, reached)
         assert set(loaded.kernels.plan.how.values()) == {"pinned"}
         del loaded
     for key, row in first.items():
