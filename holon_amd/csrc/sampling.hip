@@ -17,7 +17,7 @@ __device__ __forceinline__ ArgMax better(ArgMax a, ArgMax b) {   // larger value
   return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
 }
 
-__device__ ArgMax block_argmax(const float* __restrict__ row, int vocab, float inv_temp) {
+__device__ ArgMax block_argmax(const float* __restrict__ row, int vocab, float temp) {
   __shared__ ArgMax part[SAMPLE_THREADS / WAVE];
   __shared__ ArgMax result;
   ArgMax best{-INFINITY, 0x7fffffff};
@@ -25,13 +25,13 @@ __device__ ArgMax block_argmax(const float* __restrict__ row, int vocab, float i
     const float4* row4 = reinterpret_cast<const float4*>(row);
     for (int i = threadIdx.x; i < vocab / 4; i += blockDim.x) {
       const float4 v = row4[i];
-      best = better(best, ArgMax{v.x * inv_temp, 4 * i});
-      best = better(best, ArgMax{v.y * inv_temp, 4 * i + 1});
-      best = better(best, ArgMax{v.z * inv_temp, 4 * i + 2});
-      best = better(best, ArgMax{v.w * inv_temp, 4 * i + 3});
+      best = better(best, ArgMax{v.x / temp, 4 * i});
+      best = better(best, ArgMax{v.y / temp, 4 * i + 1});
+      best = better(best, ArgMax{v.z / temp, 4 * i + 2});
+      best = better(best, ArgMax{v.w / temp, 4 * i + 3});
     }
   } else {
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) best = better(best, ArgMax{row[i] * inv_temp, i});
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) best = better(best, ArgMax{row[i] / temp, i});
   }
 #pragma unroll
   for (int o = WAVE / 2; o > 0; o >>= 1) {
@@ -159,7 +159,7 @@ __device__ __forceinline__ float key_float(uint32_t k) {
 // The general form: any k, any kept set, and the draw in sorted order. Bisection on the ordered keys, one pass over the
 // row per step, every thread a contiguous segment of the row (so that ranks among equal values follow the index):
 // exact but slow, for the rows whose kept set does not fit the fast form below.
-__device__ void sample_row_general(const float* __restrict__ row, int32_t* __restrict__ out_r, int vocab, float inv_temp,
+__device__ void sample_row_general(const float* __restrict__ row, int32_t* __restrict__ out_r, int vocab, float temp,
                                    ArgMax top, int k, float p_keep, float p_min, float u) {
   const float xmax = top.v;
 
@@ -171,12 +171,12 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
     while (lo < hi) {
       const uint32_t mid = lo + (uint32_t)(((uint64_t)hi - lo + 1) / 2);
       int c = 0;
-      for (int i = threadIdx.x; i < vocab; i += blockDim.x) c += float_key(row[i] * inv_temp) >= mid;
+      for (int i = threadIdx.x; i < vocab; i += blockDim.x) c += float_key(row[i] / temp) >= mid;
       if (block_sum_int(c) >= k) lo = mid; else hi = mid - 1;
     }
     kth_key = lo;
     int above = 0;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) above += float_key(row[i] * inv_temp) > kth_key;
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) above += float_key(row[i] / temp) > kth_key;
     ties_kept = k - block_sum_int(above);
   }
   // rank among equals needs an index-ordered count: each thread owns a contiguous segment of the row
@@ -186,7 +186,7 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
   int ties_before = 0;           // tokens equal to the k-th value in earlier segments
   if (ties_kept != 0x7fffffff) {
     int mine = 0;
-    for (int i = seg_lo; i < seg_hi; ++i) mine += float_key(row[i] * inv_temp) == kth_key;
+    for (int i = seg_lo; i < seg_hi; ++i) mine += float_key(row[i] / temp) == kth_key;
     scan_i[threadIdx.x] = mine;
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -210,7 +210,7 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
   {
     int tie_rank = ties_before;
     for (int i = seg_lo; i < seg_hi; ++i) {
-      const float x = row[i] * inv_temp;
+      const float x = row[i] / temp;
       if (in_top_k(x, tie_rank)) part += expf(x - xmax);
     }
   }
@@ -229,7 +229,7 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
       float above = 0.f;
       int tie_rank = ties_before;
       for (int i = seg_lo; i < seg_hi; ++i) {
-        const float x = row[i] * inv_temp;
+        const float x = row[i] / temp;
         const bool kept = in_top_k(x, tie_rank);
         if (kept && float_key(x) > mid) above += expf(x - xmax);
       }
@@ -239,7 +239,7 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
     float above = 0.f;
     int tie_rank = ties_before;
     for (int i = seg_lo; i < seg_hi; ++i) {
-      const float x = row[i] * inv_temp;
+      const float x = row[i] / temp;
       const bool kept = in_top_k(x, tie_rank);
       if (kept && float_key(x) > p_key) above += expf(x - xmax);
     }
@@ -251,7 +251,7 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
   if (p_keep < 1.0f) {
     int mine = 0, tie_rank = ties_before;
     for (int i = seg_lo; i < seg_hi; ++i) {
-      const float x = row[i] * inv_temp;
+      const float x = row[i] / temp;
       const bool kept = in_top_k(x, tie_rank);
       mine += kept && float_key(x) == p_key;
     }
@@ -285,7 +285,7 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
   float mine = 0.f;
   {
     int tie_rank = ties_before, p_rank = p_ties_before;
-    for (int i = seg_lo; i < seg_hi; ++i) mine += law(row[i] * inv_temp, tie_rank, p_rank);
+    for (int i = seg_lo; i < seg_hi; ++i) mine += law(row[i] / temp, tie_rank, p_rank);
   }
   const float total = block_sum(mine);
   const float target = u * total;
@@ -297,7 +297,7 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
       float above = 0.f;
       int tie_rank = ties_before, p_rank = p_ties_before;
       for (int i = seg_lo; i < seg_hi; ++i) {
-        const float x = row[i] * inv_temp;
+        const float x = row[i] / temp;
         const float qv = law(x, tie_rank, p_rank);
         if (float_key(x) > mid) above += qv;
       }
@@ -310,7 +310,7 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
   {
     int tie_rank = ties_before, p_rank = p_ties_before;
     for (int i = seg_lo; i < seg_hi; ++i) {
-      const float x = row[i] * inv_temp;
+      const float x = row[i] / temp;
       const float qv = law(x, tie_rank, p_rank);
       const uint32_t key = float_key(x);
       if (key > d_key) above += qv;
@@ -337,7 +337,7 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
   if (ties_mine > 0 && d_before <= want && want < d_before + ties_mine) {   // (one thread)
     int tie_rank = ties_before, p_rank = p_ties_before, rank = d_before;
     for (int i = seg_lo; i < seg_hi; ++i) {
-      const float x = row[i] * inv_temp;
+      const float x = row[i] / temp;
       const float qv = law(x, tie_rank, p_rank);
       if (float_key(x) == d_key && qv > 0.f && rank++ == want) { chosen = i; break; }
     }
@@ -436,24 +436,24 @@ __device__ u64 block_scan_u64(u64 v, u64& total) {
   return before + incl - v;
 }
 
-// f(x, i) for every token of the row, x = logit * inv_temp, in no particular order: 16-byte loads where the row allows.
+// f(x, i) for every token of the row, x = logit / temp, in no particular order: 16-byte loads where the row allows.
 template <typename F>
-__device__ __forceinline__ void for_each_token(const float* __restrict__ row, int vocab, float inv_temp, F f) {
+__device__ __forceinline__ void for_each_token(const float* __restrict__ row, int vocab, float temp, F f) {
   if ((vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {
     const float4* row4 = reinterpret_cast<const float4*>(row);
     for (int i = threadIdx.x; i < vocab / 4; i += blockDim.x) {
       const float4 v = row4[i];
-      f(v.x * inv_temp, 4 * i); f(v.y * inv_temp, 4 * i + 1); f(v.z * inv_temp, 4 * i + 2); f(v.w * inv_temp, 4 * i + 3);
+      f(v.x / temp, 4 * i); f(v.y / temp, 4 * i + 1); f(v.z / temp, 4 * i + 2); f(v.w / temp, 4 * i + 3);
     }
   } else {
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) f(row[i] * inv_temp, i);
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) f(row[i] / temp, i);
   }
 }
 
 // About how many tokens lie in bands 0 .. j below the largest value, for every j, into counts[] (shared): every eighth
 // stretch of the row is counted (a token's place in the vocabulary says nothing about its value), a thread counting in
 // 8-bit fields of two registers.
-__device__ void estimate_band_counts(const float* __restrict__ row, int vocab, float inv_temp, float xmax, int* counts,
+__device__ void estimate_band_counts(const float* __restrict__ row, int vocab, float temp, float xmax, int* counts,
                                      int (*band_counts)[SAMPLE_BANDS]) {
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   u64 near_lo = 0, near_hi = 0;                  // bands 0..7 and 8..15
@@ -463,7 +463,7 @@ __device__ void estimate_band_counts(const float* __restrict__ row, int vocab, f
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (i0 + e < vocab) {
-        const int band = near_band(xmax - row[i0 + e] * inv_temp);
+        const int band = near_band(xmax - row[i0 + e] / temp);
         if (band < 8) near_lo += 1ull << (8 * band); else if (band < SAMPLE_BANDS) near_hi += 1ull << (8 * (band - 8));
       }
     }
@@ -494,12 +494,12 @@ __device__ void estimate_band_counts(const float* __restrict__ row, int vocab, f
 
 // The tokens of bands 0 .. `bands` into cand[] as order keys, in no order; returns how many there are (the same in
 // every thread), of which only the first SAMPLE_CANDIDATES were stored.
-__device__ int collect_bands(const float* __restrict__ row, int vocab, float inv_temp, float xmax, int bands, u64* cand,
+__device__ int collect_bands(const float* __restrict__ row, int vocab, float temp, float xmax, int bands, u64* cand,
                              int* n_cand) {
   if (threadIdx.x == 0) *n_cand = 0;
   __syncthreads();
   const float edge = band_edge(bands);
-  for_each_token(row, vocab, inv_temp, [&](float x, int i) {
+  for_each_token(row, vocab, temp, [&](float x, int i) {
     if (xmax - x < edge) {
       const int at = atomicAdd(n_cand, 1);
       if (at < SAMPLE_CANDIDATES) cand[at] = order_key(x, i);
@@ -533,7 +533,7 @@ __device__ void bitonic_sort(u64* a, int n_pad, bool descending) {
 // bound), and more than the bound lies over the range's lower end. The tokens of the range are then collected and
 // sorted, and the kept ones among them are those whose preceding mass, `above` included, is within the bound. Returns
 // the order key of the last kept token, or 0 when the range cannot be narrowed (thousands of equal values).
-__device__ u64 top_p_cut_wide(const float* __restrict__ row, int vocab, float inv_temp, float xmax, u64 bound, u64* cand,
+__device__ u64 top_p_cut_wide(const float* __restrict__ row, int vocab, float temp, float xmax, u64 bound, u64* cand,
                               int* n_cand) {
   __shared__ int kept_s;
   const int tid = threadIdx.x;
@@ -544,7 +544,7 @@ __device__ u64 top_p_cut_wide(const float* __restrict__ row, int vocab, float in
     if (step == 48 || !(x_mid > x_lo && x_mid < x_hi)) return 0;
     u64 mass = 0;
     int up = 0, down = 0;
-    for_each_token(row, vocab, inv_temp, [&](float x, int) {
+    for_each_token(row, vocab, temp, [&](float x, int) {
       if (x > x_mid && x <= x_hi) { mass += fixed_mass(__expf(x - xmax)); ++up; }
       else if (x > x_lo && x <= x_mid) ++down;
     });
@@ -558,7 +558,7 @@ __device__ u64 top_p_cut_wide(const float* __restrict__ row, int vocab, float in
   }
   if (tid == 0) *n_cand = 0;
   __syncthreads();
-  for_each_token(row, vocab, inv_temp, [&](float x, int i) {
+  for_each_token(row, vocab, temp, [&](float x, int i) {
     if (x > x_lo && x <= x_hi) {
       const int at = atomicAdd(n_cand, 1);
       if (at < SAMPLE_CANDIDATES) cand[at] = order_key(x, i);
@@ -599,21 +599,21 @@ __device__ u64 top_p_cut_wide(const float* __restrict__ row, int vocab, float in
 // tokens lie over the range and the k-th lies inside it; the range's tokens are then collected and sorted, and the
 // (k - above)-th of them is the last kept one. Sets `cut` to its order key (0 when fewer than k tokens weigh anything:
 // all are kept); false when the range cannot be narrowed.
-__device__ bool top_k_cut_wide(const float* __restrict__ row, int vocab, float inv_temp, float xmax, int k, u64* cand,
+__device__ bool top_k_cut_wide(const float* __restrict__ row, int vocab, float temp, float xmax, int k, u64* cand,
                                int* n_cand, u64& cut) {
   const int tid = threadIdx.x;
   float x_hi = xmax, x_lo = xmax - 128.f;        // (what lies further below weighs nothing)
   int above = 0;
   {
     int within = 0;
-    for_each_token(row, vocab, inv_temp, [&](float x, int) { within += x > x_lo; });
+    for_each_token(row, vocab, temp, [&](float x, int) { within += x > x_lo; });
     if (block_sum_int(within) <= k) { cut = 0; return true; }
   }
   for (int step = 0;; ++step) {
     const float x_mid = 0.5f * (x_lo + x_hi);
     if (step == 48 || !(x_mid > x_lo && x_mid < x_hi)) return false;
     int up = 0, down = 0;
-    for_each_token(row, vocab, inv_temp, [&](float x, int) {
+    for_each_token(row, vocab, temp, [&](float x, int) {
       if (x > x_mid && x <= x_hi) ++up;
       else if (x > x_lo && x <= x_mid) ++down;
     });
@@ -626,7 +626,7 @@ __device__ bool top_k_cut_wide(const float* __restrict__ row, int vocab, float i
   }
   if (tid == 0) *n_cand = 0;
   __syncthreads();
-  for_each_token(row, vocab, inv_temp, [&](float x, int i) {
+  for_each_token(row, vocab, temp, [&](float x, int i) {
     if (x > x_lo && x <= x_hi) {
       const int at = atomicAdd(n_cand, 1);
       if (at < SAMPLE_CANDIDATES) cand[at] = order_key(x, i);
@@ -663,8 +663,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     if (tid == 0) out[r] = a.i;
     return;
   }
-  const float inv_temp = 1.0f / temp;
-  const ArgMax top = block_argmax(row, vocab, inv_temp);
+  const ArgMax top = block_argmax(row, vocab, temp);
   const float xmax = top.v;
   const int k = top_k[pr];
   const float p_keep = top_p[pr], p_min = min_p[pr];
@@ -675,7 +674,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
   const bool m_on = p_min > 0.f;
   const bool filtered = k > 0 || p_on || m_on;
   if (filtered && vocab > 255 * SAMPLE_THREADS) {      // (uniform over the block)
-    sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
+    sample_row_general(row, out + r, vocab, temp, top, k, p_keep, p_min, u);
     return;
   }
 
@@ -689,11 +688,11 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
       u64 z_all = 0;
       if (!k_on) {                               // top-p without top-k: the mass of the whole row
         u64 mass = 0;
-        for_each_token(row, vocab, inv_temp, [&](float x, int) { mass += fixed_mass(__expf(x - xmax)); });
+        for_each_token(row, vocab, temp, [&](float x, int) { mass += fixed_mass(__expf(x - xmax)); });
         z_all = block_sum_u64(mass);
       }
       wide = k_on && k > SAMPLE_CANDIDATES;      // no room for the kept set whatever the bands
-      if (!wide) estimate_band_counts(row, vocab, inv_temp, xmax, counts, band_counts);
+      if (!wide) estimate_band_counts(row, vocab, temp, xmax, counts, band_counts);
       // Which bands to collect: the fewest that should hold twice what is needed (k tokens; 256 for top-p alone). The
       // collecting counts exactly; too many, or fewer than k, and another set of bands is tried.
       const int need = k_on ? k : 1;
@@ -707,7 +706,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
           wide = true;
           break;
         }
-        const int count = collect_bands(row, vocab, inv_temp, xmax, bands, cand, &n_cand);
+        const int count = collect_bands(row, vocab, temp, xmax, bands, cand, &n_cand);
         if (count > SAMPLE_CANDIDATES) {
           --bands;
           if (bands <= beyond_at) attempt = 5;    // the next fewer bands held too little: no set of bands will do
@@ -768,22 +767,22 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
         bool found = true;
         u64 z_k = z_all;
         if (k_on) {
-          found = top_k_cut_wide(row, vocab, inv_temp, xmax, k, cand, &n_cand, cut);
+          found = top_k_cut_wide(row, vocab, temp, xmax, k, cand, &n_cand, cut);
           if (found && p_on) {
             u64 mass = 0;
-            for_each_token(row, vocab, inv_temp, [&](float x, int i) {
+            for_each_token(row, vocab, temp, [&](float x, int i) {
               if (order_key(x, i) >= cut) mass += fixed_mass(__expf(x - xmax));
             });
             z_k = block_sum_u64(mass);
           }
         }
         if (found && p_on) {
-          const u64 p_cut = top_p_cut_wide(row, vocab, inv_temp, xmax, (u64)((double)p_keep * (double)z_k), cand, &n_cand);
+          const u64 p_cut = top_p_cut_wide(row, vocab, temp, xmax, (u64)((double)p_keep * (double)z_k), cand, &n_cand);
           found = p_cut != 0;
           cut = max(cut, p_cut);
         }
         if (!found) {                              // thousands of equal values where a cut falls
-          sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
+          sample_row_general(row, out + r, vocab, temp, top, k, p_keep, p_min, u);
           return;
         }
       }
@@ -794,7 +793,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
       while (bands < SAMPLE_BANDS && band_edge(bands) < reach) ++bands;
       wide = true;
       if (bands < SAMPLE_BANDS) {
-        const int count = collect_bands(row, vocab, inv_temp, xmax, bands, cand, &n_cand);
+        const int count = collect_bands(row, vocab, temp, xmax, bands, cand, &n_cand);
         if (count <= SAMPLE_CANDIDATES) {
           int n_pad = WAVE;
           while (n_pad < count) n_pad <<= 1;
@@ -848,15 +847,15 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     // the bound (what precedes a kept token is kept, so the search need not know the filters).
     __syncthreads();                            // `cand` is free from here on
     u64 mass = 0;
-    for_each_token(row, vocab, inv_temp, [&](float x, int i) {
+    for_each_token(row, vocab, temp, [&](float x, int i) {
       const float q = __expf(x - xmax);
       if (order_key(x, i) >= cut && q >= p_min) mass += fixed_mass(q);
     });
     const u64 total = block_sum_u64(mass);
     const u64 target = (u64)((double)u * (double)total);
-    const u64 hit = total > 0 ? top_p_cut_wide(row, vocab, inv_temp, xmax, target, cand, &n_cand) : 0;
+    const u64 hit = total > 0 ? top_p_cut_wide(row, vocab, temp, xmax, target, cand, &n_cand) : 0;
     if (total > 0 && hit == 0) {                 // thousands of equal values around the target
-      sample_row_general(row, out + r, vocab, inv_temp, top, k, p_keep, p_min, u);
+      sample_row_general(row, out + r, vocab, temp, top, k, p_keep, p_min, u);
       return;
     }
     if (tid == 0) out[r] = total > 0 ? (int)(0x7fffffffu - (uint32_t)hit) : top.i;
@@ -878,7 +877,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
       for (int e = 0; e < 4; ++e) x[e] = i0 + e < vocab ? row[i0 + e] : -INFINITY;
     }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) m[e] = i0 + e < vocab ? law(x[e] * inv_temp, i0 + e, all) : 0u;
+    for (int e = 0; e < 4; ++e) m[e] = i0 + e < vocab ? law(x[e] / temp, i0 + e, all) : 0u;
   };
   auto chunk_sums = [&](auto all) {
     for (int c = wave; c < chunks; c += SAMPLE_WAVES) {

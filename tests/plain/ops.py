@@ -208,7 +208,7 @@ class TorchKernels:
             temp = float(temperature[r])
             if temp == 0:
                 continue
-            x = logits[r].float() / temp
+            x = logits[r].float() / torch.full_like(logits[r], temp, dtype=torch.float32)   # (a tensor: a true division)
             keep = torch.ones_like(x, dtype=torch.bool)
             order = x.argsort(descending=True, stable=True)
             if int(top_k[r]) > 0:

@@ -45,11 +45,13 @@ def probs(logits: torch.Tensor, temperature: float, top_k: int = 0, top_p: float
           ) -> torch.Tensor:
     """The law of one row [V] in float64: temperature, then top-k, then top-p over the renormalised rest (the most
     likely token always stays), then min-p against the largest probability after top-k; temperature 0 is one-hot at
-    the first maximum. std/holon_std/sampling/reference.py:13-30."""
+    the first maximum. std/holon_std/sampling/reference.py:13-30. The logits are divided by the temperature in
+    float32, as the reference's sampler divides them (std/holon_std/sampling/sampler.py:137): which values are equal
+    after that decides ties at a filter's edge."""
     x = logits.double()
     if temperature == 0:
         return torch.nn.functional.one_hot(x.argmax(), x.numel()).double()
-    x = x / temperature
+    x = scaled(logits, temperature)
     keep = torch.ones_like(x, dtype=torch.bool)
     order = x.argsort(descending=True, stable=True)
     if top_k > 0:
@@ -63,6 +65,12 @@ def probs(logits: torch.Tensor, temperature: float, top_k: int = 0, top_p: float
     return torch.where(keep, x, float("-inf")).softmax(-1)
 
 
+def scaled(logits: torch.Tensor, temperature: float) -> torch.Tensor:
+    """logits / temperature as a float32 division, in float64 for what follows. The divisor is a tensor of the logits'
+    shape: by a scalar, torch may multiply by the reciprocal instead, which is not the same in the last place."""
+    return (logits.float() / torch.full_like(logits, temperature, dtype=torch.float32)).double()
+
+
 def drawing_order(logits: torch.Tensor, temperature: float, top_k: int = 0, top_p: float = 1.0, min_p: float = 0.0
                   ) -> torch.Tensor | None:
     """The order in which a row's tokens are walked by the draw: vocabulary order (None) when no filter is set, else
@@ -71,7 +79,7 @@ def drawing_order(logits: torch.Tensor, temperature: float, top_k: int = 0, top_
     std/holon_std/sampling/sampler.py:43-54,134-141."""
     if temperature == 0 or not (top_k > 0 or top_p < 1 or min_p > 0):
         return None
-    return (logits.double() / temperature).argsort(descending=True, stable=True)
+    return scaled(logits, temperature).argsort(descending=True, stable=True)
 
 
 def draw(q: torch.Tensor, u: float, order: torch.Tensor | None = None) -> int:

@@ -248,7 +248,8 @@ def test_engine_at_the_wide_sizes_with_everything_on(folder, products):
             H.assert_greedy_follows(plain, prompt, got)
     assert full.cache.tokens_saved > 0 and full.stats()["graphs"] >= 1 and full.runner.graph_replays > 10
     how = {"timed": "pinned", "own": "own"}[products]
-    assert full.stats()["products"] == bare.products() and set(full.kernels.plan.how.values()) == {how}, full.kernels.plan.how
+    assert full.stats()["products"].items() <= bare.products().items()           # (a rival's own form is not met again)
+    assert set(full.kernels.plan.how.values()) == {how}, full.kernels.plan.how
 
 
 def test_long_context_attention_kernels():

@@ -1,7 +1,9 @@
 """The decode attention entry point that allocates nothing (`holon_attention_decode_bf16_static`), called through
 ctypes as a caller without an allocator would: its split partials live in a device array inside the library. It must
 give bit for bit what the entry point with a caller's workspace gives, on two calls in a row (the second smaller, so
-that it runs over what the first left in the array), and refuse what does not fit."""
+that it runs over what the first left in the array), stay within the bfloat16 budget of the plain attention computed in
+float64 (the two entry points share their launch: a fault in it would not show between them), and refuse what does
+not fit."""
 from __future__ import annotations
 
 import ctypes
@@ -9,6 +11,8 @@ import ctypes
 import pytest
 import torch
 
+from tests import helpers as H
+from tests.plain.ops import TorchKernels
 from tests.test_kernels_gpu import _paged_case
 
 pytestmark = pytest.mark.gpu
@@ -49,6 +53,8 @@ def _both(lib, rows, heads, kv_heads, head_dim, splits, seed, window=0):
     assert rc == 0, lib.holon_last_error().decode()
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    plain = TorchKernels().paged_attention(q.double(), pages.double(), table, attn, page, head_dim ** -0.5, window)
+    assert H.op_budget_usage(got, plain, torch.bfloat16, head_dim + longest) <= 1, (rows, heads, kv_heads, head_dim)
     return got, want
 
 
