@@ -53,6 +53,8 @@ struct AttnArgs {
   float* part_o;           // [n_rows, Hq, splits, D]
   float* part_ml;          // [n_rows, Hq, splits, 2]
   int splits, keys_per_split;
+  int out_splits;          // partials a (row, head) leaves: splits / waves of a block (1: the block writes the result)
+  int rows_in_order;       // every row of the step is a decode row and row_ids[i] = query_start[i] = i
   // long prompt portions only: a block runs one of its two ranges (blockIdx.z = 2 row + which), not both
   int unpaired;
 };
@@ -122,12 +124,20 @@ __device__ __forceinline__ bf16x8_t softmax_block(const f32x4_t& s0, const f32x4
 // One wave: NT tiles against keys [key_lo, key_hi] (inclusive, as bounded per row by causality and the window).
 // On return o[t][dsub] holds the unnormalised O^T, m[t] the running max (base-2 scaled), l[t] this lane's share of
 // the sum (to be added over the four lane groups).
-template <int D, int NT>
+// `fresh` (nullable): the key (D values) and then the value (D values) of key number `key_hi`, in LDS, which take the
+// place of what the cache holds there (a decode row's new token, whose stores to the cache may still be under way).
+// `prepare()` runs once the first block's keys have been asked for and before `qf` is first read: arithmetic that
+// makes the queries (a decode row's norm and rotation) then runs while those loads are under way.
+struct Nothing {
+  __device__ __forceinline__ void operator()() const {}
+};
+template <int D, int NT, typename Prepare = Nothing>
 __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __restrict__ trow, int hk,
                                            const bf16x8_t (&qf)[NT][D / 32], const int (&qpos)[NT],
                                            const int (&tile_last)[NT], const int (&tile_first)[NT], int key_lo,
                                            int key_hi,
-                                           f32x4_t (&o)[NT][D / 16], float (&m)[NT], float (&l)[NT]) {
+                                           f32x4_t (&o)[NT][D / 16], float (&m)[NT], float (&l)[NT],
+                                           const bf16_t* fresh = nullptr, Prepare prepare = Prepare()) {
   const int lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
   const int P = a.page_size;
@@ -153,6 +163,7 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
   const int kb_first = (key_lo / 32) * 32;
   bf16x8_t kf0[D / 32], kf1[D / 32];
   load_keys(kb_first, kf0, kf1);
+  prepare();
   for (int kb = kb_first; kb <= key_hi; kb += 32) {
     // values of this block (lane group g needs keys 8g .. 8g+7, for dims dsub*16 + c) and the keys of the next one
     // are requested before this block's products, so that their latency hides behind the matrix cores
@@ -165,6 +176,26 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
     if (kb + 31 > key_hi) {
 #pragma unroll
       for (int ds = 0; ds < D / 16; ++ds) zero_after(vf[ds], kb + 8 * g, key_hi);
+    }
+    if (fresh != nullptr && kb + 31 >= key_hi) {           // the block that holds key_hi: its key and value from LDS
+      const int k0 = kb + 16 * khalf + kin;                // this lane's keys are k0 and k0 + 4
+      if (k0 == key_hi || k0 + 4 == key_hi) {
+#pragma unroll
+        for (int ks = 0; ks < D / 32; ++ks) {
+          const bf16x8_t nk = *reinterpret_cast<const bf16x8_t*>(fresh + ks * 32 + 8 * g);
+          if (k0 == key_hi) kf0[ks] = nk; else kf1[ks] = nk;
+        }
+      }
+      const int j = key_hi - (kb + 8 * g);                 // the value's place among this lane's eight keys, if any
+      if (j >= 0 && j < 8) {
+#pragma unroll
+        for (int ds = 0; ds < D / 16; ++ds) {
+          const __bf16 nv = reinterpret_cast<const __bf16*>(fresh + D)[ds * 16 + c];
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (i == j) vf[ds][i] = nv;
+        }
+      }
     }
     bf16x8_t nf0[D / 32], nf1[D / 32];
     const bool more = kb + 32 <= key_hi;
@@ -750,19 +781,119 @@ __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kerne
   }
 }
 
-// Decode rows: block (split, kv head x head block, row), one wave. Partials go to part_o / part_ml.
+// What the decode kernel needs to take the step's raw q/k/v projection itself (`qkv` [T, (Hq + 2 Hkv) D]) instead of
+// queries that another kernel has normed and rotated and keys that it has stored: per-head RMSNorm weights (both or
+// neither), the rotation table (cos | sin of every position, over the whole head, or none), where each token's key
+// and value go in the cache.
+struct FusedArgs {
+  const bf16_t* qkv;
+  int64_t qkv_stride;
+  const bf16_t* q_weight;
+  const bf16_t* k_weight;
+  float eps;
+  const float* table;          // [max_positions, D]; a decode row's token sits at position len - 1
+  int max_positions;           // (a longer row, which the engine never makes, would read the table's last row)
+  bf16_t* pages;               // the cache, written for the row's new token
+  const int32_t* write_page;   // [T]
+  const int32_t* write_off;    // [T]
+};
+
+// The row's new key and value from the raw projection: RMSNorm over the head and rotation for the key, the value as
+// it is. One wave: lanes 0 .. D/8 - 1 hold eight dims each of the key, the next D/8 lanes of the value. `make` leaves
+// both in LDS (`fresh`: the key's D values, then the value's) and in the lanes' registers; `store` sends them to the
+// cache (the value transposed inside its page). The roundings are those of the norm + rotation + write kernel
+// (elementwise.hip).
 template <int D>
-__global__ void __launch_bounds__(64) attn_decode_kernel(AttnArgs a) {
-  const int lane = threadIdx.x % WAVE;
+struct NewKeyValue {
+  static constexpr int LPH = D / 8;
+  uint4 mine;       // role 0: the key's eight values as stored; role 1: the value's
+  int li, role;
+
+  __device__ __forceinline__ void make(const AttnArgs& a, const FusedArgs& f, int token, int pos, int hk, bf16_t* fresh) {
+    const int lane = threadIdx.x % WAVE;
+    li = lane % LPH;
+    role = lane / LPH;                                   // 0: the key, 1: the value, beyond: nothing to store
+    const int head = a.heads + (role == 1 ? a.kv_heads : 0) + hk;
+    const bf16_t* src = f.qkv + (int64_t)token * f.qkv_stride + (int64_t)head * D + li * 8;
+    const uint4 raw = *reinterpret_cast<const uint4*>(src);
+    const bf16_t* e = reinterpret_cast<const bf16_t*>(&raw);
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = bf16_to_float(e[j]);
+    if (f.k_weight != nullptr) {
+      const uint4 wraw = *reinterpret_cast<const uint4*>(f.k_weight + li * 8);
+      const bf16_t* w = reinterpret_cast<const bf16_t*>(&wraw);
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
+#pragma unroll
+      for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
+      const float inv = 1.0f / sqrtf(ss / (float)D + f.eps);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (float)(__bf16)((v[j] * inv) * bf16_to_float(w[j]));
+    }
+    if (f.table != nullptr) {
+      const float* cs = f.table + (int64_t)pos * D + (li % (LPH / 2)) * 8;
+      float co[8], si[8];
+      *reinterpret_cast<float4*>(co) = *reinterpret_cast<const float4*>(cs);
+      *reinterpret_cast<float4*>(co + 4) = *reinterpret_cast<const float4*>(cs + 4);
+      *reinterpret_cast<float4*>(si) = *reinterpret_cast<const float4*>(cs + D / 2);
+      *reinterpret_cast<float4*>(si + 4) = *reinterpret_cast<const float4*>(cs + D / 2 + 4);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float other = __shfl_xor(v[j], LPH / 2, WAVE);
+        v[j] = li < LPH / 2 ? v[j] * co[j] - other * si[j] : v[j] * co[j] + other * si[j];
+      }
+    }
+    mine = raw;
+    if (role == 0) {
+      __bf16* oe = reinterpret_cast<__bf16*>(&mine);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) oe[j] = (__bf16)v[j];
+    }
+    if (role < 2) *reinterpret_cast<uint4*>(fresh + role * D + li * 8) = mine;
+  }
+
+  __device__ __forceinline__ void store(const AttnArgs& a, const FusedArgs& f, int token, int hk) const {
+    const int P = a.page_size;
+    const int64_t plane = (int64_t)P * D;
+    const int wpage = f.write_page[token], woff = f.write_off[token];
+    if (role == 0) {
+      *reinterpret_cast<uint4*>(f.pages + (((int64_t)wpage * 2) * a.kv_heads + hk) * plane + (int64_t)woff * D + li * 8) = mine;
+    } else if (role == 1) {
+      const bf16_t* e = reinterpret_cast<const bf16_t*>(&mine);
+      bf16_t* dst = f.pages + (((int64_t)wpage * 2 + 1) * a.kv_heads + hk) * plane + woff;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dst[(int64_t)(li * 8 + j) * P] = e[j];
+    }
+  }
+};
+
+// Decode rows: block (split, kv head x head block, row), one wave. Partials go to part_o / part_ml.
+// FUSED: the queries come raw from the step's q/k/v projection and are normed and rotated here (each wave its own
+// copy: a few hundred values), and the wave whose keys end with the row's new token norms and rotates that token's key
+// and keeps it and the value in LDS, from where they take their place among the wave's operands; it stores them into
+// the cache as the last thing it does (a store before the loads would make every later load wait for it), and no
+// other wave reads that place. A decode row's token sits at position len - 1. The kernel that did all this for decode
+// steps is gone.
+// A block's waves take consecutive shares of the row's keys and their partials are combined through LDS in wave order
+// (waves 1.. leave theirs there, wave 0 adds them up); with one block a (row, kv head) the block writes the result
+// itself and no merge kernel follows.
+template <int D, bool FUSED>
+__global__ void __launch_bounds__(512) attn_decode_kernel(AttnArgs a, FusedArgs f) {
+  extern __shared__ __attribute__((aligned(16))) float red[];   // [waves - 1][16 D values, 16 maxima, 16 sums]
+  __shared__ __attribute__((aligned(16))) bf16_t fresh_lds[FUSED ? 2 * D : 8];
+  constexpr int PART = 16 * D + 32;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, waves = blockDim.x / WAVE;
   const int g = lane / 16, c = lane % 16;
   const int ri = blockIdx.z;
-  const int b = a.row_ids[ri];
+  const int b = a.rows_in_order ? ri : a.row_ids[ri];
   const int group = a.heads / a.kv_heads;
   const TileMap tm = tile_map(group);
   const int hk = blockIdx.y / tm.head_blocks, hb = blockIdx.y % tm.head_blocks;
-  const int split = blockIdx.x;
-  const int qs = a.qstart[b], nq = a.qstart[b + 1] - qs, n = a.lens[b];
-  const RowRef rr = row_ref(tm, c, 0, hb, hk, group, qs, nq > 0 ? 1 : 0, n);
+  const int split = blockIdx.x * waves + wave;
+  const int qs = a.rows_in_order ? b : a.qstart[b], n = a.lens[b];
+  const RowRef rr = row_ref(tm, c, 0, hb, hk, group, qs, 1, n);
   // the keys this row can see, cut into `splits` ranges of keys_per_split
   const int qp_row = n - 1;
   const int first = a.window > 0 ? max(0, qp_row - a.window + 1) : 0;
@@ -772,37 +903,154 @@ __global__ void __launch_bounds__(64) attn_decode_kernel(AttnArgs a) {
   const int share = max(32, ((qp_row - base + a.splits) / a.splits + 31) / 32 * 32);
   const int key_lo = base + split * share;
   const int key_hi = min(qp_row, key_lo + share - 1);
-  float* po = a.part_o + (((int64_t)ri * a.heads + rr.head) * a.splits + split) * D + 4 * g;
-  float* pml = a.part_ml + (((int64_t)ri * a.heads + rr.head) * a.splits + split) * 2;
-  if (n <= 0 || key_lo > key_hi) {   // an empty range: a partial that weighs nothing
-    if (rr.valid && g == 0) { pml[0] = -INFINITY; pml[1] = 0.f; }
-    return;
-  }
-  const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
-  bf16x8_t qf[1][D / 32];
-  const bf16_t* qptr = a.q + ((int64_t)rr.token * a.heads + rr.head) * D + 8 * g;
-#pragma unroll
-  for (int ks = 0; ks < D / 32; ++ks) {
-    if (rr.valid) {
-      qf[0][ks] = load8(qptr + ks * 32);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) qf[0][ks][i] = (__bf16)0.f;
-    }
-  }
-  int qpos[1] = {rr.valid ? qp_row : -1}, tile_last[1] = {qp_row}, tile_first[1] = {qp_row};
+  const bool empty = n <= 0 || key_lo > key_hi;           // (uniform over the wave) a partial that weighs nothing
+  const bool writer = FUSED && !empty && key_hi == qp_row;   // its keys end with the row's new token
   f32x4_t o[1][D / 16];
   float m[1] = {-INFINITY}, l[1] = {0.f};
 #pragma unroll
   for (int ds = 0; ds < D / 16; ++ds) o[0][ds] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  attn_tiles<D, 1>(a, trow, hk, qf, qpos, tile_last, tile_first, max(key_lo, first), key_hi, o, m, l);
+  NewKeyValue<D> fresh;
+  if (!empty) {
+    const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
+    bf16x8_t qf[1][D / 32];
+    // FUSED: what makes the queries is asked for now (lane (g, c) holds dims 32 ks + 8 g .. + 7 of head c: the raw
+    // values, the norm's weights, the cosines and sines of the row's position) and turned into `qf` inside attn_tiles,
+    // while the first keys are on their way
+    uint4 qraw[D / 32], wraw[D / 32];
+    float4 cs[D / 64][4];
+    if constexpr (FUSED) {
+      const bf16_t* qptr = f.qkv + (int64_t)rr.token * f.qkv_stride + (int64_t)rr.head * D + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < D / 32; ++ks) {
+        qraw[ks] = uint4{0u, 0u, 0u, 0u};
+        if (rr.valid) qraw[ks] = *reinterpret_cast<const uint4*>(qptr + ks * 32);
+        if (f.q_weight != nullptr) wraw[ks] = *reinterpret_cast<const uint4*>(f.q_weight + ks * 32 + 8 * g);
+      }
+      if (f.table != nullptr) {
+        const float* t0 = f.table + (int64_t)min(qp_row, f.max_positions - 1) * D + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < D / 64; ++ks) {
+          cs[ks][0] = *reinterpret_cast<const float4*>(t0 + ks * 32);
+          cs[ks][1] = *reinterpret_cast<const float4*>(t0 + ks * 32 + 4);
+          cs[ks][2] = *reinterpret_cast<const float4*>(t0 + D / 2 + ks * 32);
+          cs[ks][3] = *reinterpret_cast<const float4*>(t0 + D / 2 + ks * 32 + 4);
+        }
+      }
+      if (writer) {                      // one wave of the block at most; what it leaves in LDS only it reads
+        fresh.make(a, f, qs, min(qp_row, f.max_positions - 1), hk, fresh_lds);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
+    } else {
+      const bf16_t* qptr = a.q + ((int64_t)rr.token * a.heads + rr.head) * D + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < D / 32; ++ks) {
+        if (rr.valid) {
+          qf[0][ks] = load8(qptr + ks * 32);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) qf[0][ks][i] = (__bf16)0.f;
+        }
+      }
+    }
+    auto make_queries = [&]() {
+      if constexpr (FUSED) {
+        float qv[D / 32][8];
+        float ss = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < D / 32; ++ks) {
+          const bf16_t* e = reinterpret_cast<const bf16_t*>(&qraw[ks]);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            qv[ks][j] = bf16_to_float(e[j]);
+            ss += qv[ks][j] * qv[ks][j];
+          }
+        }
+        if (f.q_weight != nullptr) {     // the sum of squares over the four lane groups, then round((x inv) w)
+          ss += __shfl_xor(ss, 16, WAVE);
+          ss += __shfl_xor(ss, 32, WAVE);
+          const float inv = 1.0f / sqrtf(ss / (float)D + f.eps);
+#pragma unroll
+          for (int ks = 0; ks < D / 32; ++ks) {
+            const bf16_t* w = reinterpret_cast<const bf16_t*>(&wraw[ks]);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) qv[ks][j] = (float)(__bf16)((qv[ks][j] * inv) * bf16_to_float(w[j]));
+          }
+        }
+        if (f.table != nullptr) {        // dim i turns with dim i + D/2: fragment ks + D/64 of the same lane
+#pragma unroll
+          for (int ks = 0; ks < D / 64; ++ks) {
+            const float* co = reinterpret_cast<const float*>(&cs[ks][0]);
+            const float* si = reinterpret_cast<const float*>(&cs[ks][2]);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float lo = qv[ks][j], hi = qv[ks + D / 64][j];
+              qv[ks][j] = lo * co[j] - hi * si[j];
+              qv[ks + D / 64][j] = hi * co[j] + lo * si[j];
+            }
+          }
+        }
+#pragma unroll
+        for (int ks = 0; ks < D / 32; ++ks)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) qf[0][ks][j] = (__bf16)qv[ks][j];
+      }
+    };
+    int qpos[1] = {rr.valid ? qp_row : -1}, tile_last[1] = {qp_row}, tile_first[1] = {qp_row};
+    attn_tiles<D, 1>(a, trow, hk, qf, qpos, tile_last, tile_first, max(key_lo, first), key_hi, o, m, l,
+                     writer ? fresh_lds : nullptr, make_queries);
+  }
   float lt = l[0];
   lt += __shfl_xor(lt, 16, WAVE);
   lt += __shfl_xor(lt, 32, WAVE);
-  if (!rr.valid) return;
+  float mt = m[0];
+  if (waves > 1) {                       // the block's partials, added up in wave order by wave 0
+    if (wave > 0) {
+      float* mine = red + (int64_t)(wave - 1) * PART;
 #pragma unroll
-  for (int ds = 0; ds < D / 16; ++ds) *reinterpret_cast<f32x4_t*>(po + ds * 16) = o[0][ds];
-  if (g == 0) { pml[0] = m[0]; pml[1] = lt; }
+      for (int ds = 0; ds < D / 16; ++ds) *reinterpret_cast<f32x4_t*>(mine + (ds * WAVE + lane) * 4) = o[0][ds];
+      if (g == 0) { mine[16 * D + c] = mt; mine[16 * D + 16 + c] = lt; }
+    }
+    __syncthreads();
+    if (wave == 0) {
+      for (int w = 1; w < waves; ++w) {
+        const float* theirs = red + (int64_t)(w - 1) * PART;
+        const float mw = theirs[16 * D + c], lw = theirs[16 * D + 16 + c];
+        const float m_new = fmaxf(mt, mw);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(mt - m_use), beta = __builtin_amdgcn_exp2f(mw - m_use);
+        lt = lt * alpha + lw * beta;
+#pragma unroll
+        for (int ds = 0; ds < D / 16; ++ds)
+          o[0][ds] = o[0][ds] * alpha + *reinterpret_cast<const f32x4_t*>(theirs + (ds * WAVE + lane) * 4) * beta;
+        mt = m_new;
+      }
+    }
+  }
+  if (wave == 0 && rr.valid) {
+    if (a.out_splits == 1) {             // the row's whole result: normalised and rounded here
+      const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+      bf16_t* op = a.out + ((int64_t)rr.token * a.heads + rr.head) * D + 4 * g;
+#pragma unroll
+      for (int ds = 0; ds < D / 16; ++ds) {
+        ushort4 w;
+        w.x = float_to_bf16(o[0][ds][0] * inv);
+        w.y = float_to_bf16(o[0][ds][1] * inv);
+        w.z = float_to_bf16(o[0][ds][2] * inv);
+        w.w = float_to_bf16(o[0][ds][3] * inv);
+        *reinterpret_cast<ushort4*>(op + ds * 16) = w;
+      }
+    } else {
+      const int64_t cell = ((int64_t)ri * a.heads + rr.head) * a.out_splits + blockIdx.x;
+      float* po = a.part_o + cell * D + 4 * g;
+#pragma unroll
+      for (int ds = 0; ds < D / 16; ++ds) *reinterpret_cast<f32x4_t*>(po + ds * 16) = o[0][ds];
+      if (g == 0) { a.part_ml[cell * 2] = mt; a.part_ml[cell * 2 + 1] = lt; }
+    }
+  }
+  if constexpr (FUSED) {
+    if (writer) fresh.store(a, f, qs, hk);
+  }
 }
 
 // out[row, head, :] = sum_i 2^(m_i - M) o_i / sum_i 2^(m_i - M) l_i over the splits (at most 64). One block of four
@@ -934,13 +1182,19 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
 static int decode_launch(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
                          const int32_t* slots, const int32_t* lens, const int32_t* query_start, const int32_t* row_ids,
                          int n_rows, int max_len, int heads, int kv_heads, int head_dim, int page_size, float scale,
-                         int window, float* part_o, float* part_ml, int splits, int keys_per_split, void* stream) {
+                         int window, float* part_o, float* part_ml, int splits, int keys_per_split, void* stream,
+                         const FusedArgs* fused = nullptr, int waves = 1, int rows_in_order = 0) {
   HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
               "attention: bad sizes");
-  HOLON_CHECK(splits > 0 && splits <= 64 && keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml,
-              "attention decode: splits %d of %d keys (a multiple of 32) need a workspace", splits, keys_per_split);
+  HOLON_CHECK(splits > 0 && splits <= 64 && keys_per_split > 0 && keys_per_split % 32 == 0,
+              "attention decode: %d splits of %d keys (1 to 64 splits of a multiple of 32 keys)", splits, keys_per_split);
+  HOLON_CHECK(waves >= 1 && waves <= 8 && splits % waves == 0 && (waves - 1) * (16 * head_dim + 32) * 4 <= 64 * 1024,
+              "attention decode: %d waves a block for %d splits of head_dim %d (1 to 8, a divisor of the splits, "
+              "partials within 64 KB of LDS)", waves, splits, head_dim);
+  HOLON_CHECK(splits == waves || (part_o && part_ml), "attention decode: %d splits over blocks need a workspace",
+              splits / waves);
   const int span = window > 0 ? (window < max_len ? window + 31 : max_len) : max_len;
   HOLON_CHECK((int64_t)splits * keys_per_split >= span, "attention decode: %d splits of %d keys do not cover %d keys",
               splits, keys_per_split, span);
@@ -951,13 +1205,25 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
   a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size;
   a.scale_log2 = scale * 1.4426950408889634f; a.window = window;
   a.part_o = part_o; a.part_ml = part_ml; a.splits = splits; a.keys_per_split = keys_per_split;
+  a.out_splits = splits / waves; a.rows_in_order = rows_in_order;
   const TileMap tm = tile_map(heads / kv_heads);
-  dim3 grid(splits, kv_heads * tm.head_blocks, n_rows);
+  dim3 grid(a.out_splits, kv_heads * tm.head_blocks, n_rows);
   hipStream_t s = (hipStream_t)stream;
-  if (head_dim == 64) attn_decode_kernel<64><<<grid, 64, 0, s>>>(a);
-  else if (head_dim == 128) attn_decode_kernel<128><<<grid, 64, 0, s>>>(a);
-  else attn_decode_kernel<256><<<grid, 64, 0, s>>>(a);
+  const int threads = waves * WAVE;
+  const size_t lds = (size_t)(waves - 1) * (16 * head_dim + 32) * sizeof(float);
+  if (fused != nullptr) {
+    if (head_dim == 64) attn_decode_kernel<64, true><<<grid, threads, lds, s>>>(a, *fused);
+    else if (head_dim == 128) attn_decode_kernel<128, true><<<grid, threads, lds, s>>>(a, *fused);
+    else attn_decode_kernel<256, true><<<grid, threads, lds, s>>>(a, *fused);
+  } else {
+    const FusedArgs none{};
+    if (head_dim == 64) attn_decode_kernel<64, false><<<grid, threads, lds, s>>>(a, none);
+    else if (head_dim == 128) attn_decode_kernel<128, false><<<grid, threads, lds, s>>>(a, none);
+    else attn_decode_kernel<256, false><<<grid, threads, lds, s>>>(a, none);
+  }
   HOLON_LAUNCH_OK();
+  if (a.out_splits == 1) return 0;       // every block has written its row's result
+  splits = a.out_splits;
   dim3 mgrid(n_rows, heads);
   if (head_dim == 64)
     attn_merge_kernel<64><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits);
@@ -977,6 +1243,49 @@ extern "C" int holon_attention_decode_bf16(const void* q, void* out, const void*
                                            void* stream) {
   return decode_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len, heads,
                        kv_heads, head_dim, page_size, scale, window, part_o, part_ml, splits, keys_per_split, stream);
+}
+
+// The same with `waves` waves a block (1 to 8, a divisor of `splits`): a block's waves combine their partials through
+// LDS, so a (row, head) leaves splits / waves partials (part_o [n_rows, heads, splits / waves, head_dim], part_ml
+// likewise) and, when that is one, none at all: the block writes the result and the workspace may be NULL.
+// rows_in_order: every row of the step is a decode row, row_ids[i] = i and query_start[i] = i (neither is then read).
+extern "C" int holon_attention_decode_waves_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                                 int table_stride, const int32_t* slots, const int32_t* lens,
+                                                 const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                                 int max_len, int heads, int kv_heads, int head_dim, int page_size,
+                                                 float scale, int window, float* part_o, float* part_ml, int splits,
+                                                 int keys_per_split, int waves, int rows_in_order, void* stream) {
+  return decode_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len, heads,
+                       kv_heads, head_dim, page_size, scale, window, part_o, part_ml, splits, keys_per_split, stream,
+                       nullptr, waves, rows_in_order);
+}
+
+// Decode rows straight from the step's raw q/k/v projection: per-head norm, rotation and the cache write of each
+// row's new token happen inside the attention kernel. `qkv` [T, (heads + 2 kv_heads) head_dim]; q_weight / k_weight
+// (both or neither) the per-head RMSNorm weights; rope_table [max_positions, head_dim] (cos | sin) or NULL. A row's
+// token is taken to sit at position len - 1 (what a decode row is).
+extern "C" int holon_attention_decode_fused_bf16(const void* qkv, void* out, void* pages, const int32_t* table,
+                                                 int table_stride, const int32_t* slots, const int32_t* lens,
+                                                 const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                                 int max_len, int heads, int kv_heads, int head_dim, int page_size,
+                                                 float scale, int window, const void* q_weight, const void* k_weight,
+                                                 float eps, const float* rope_table, int max_positions,
+                                                 const int32_t* write_page, const int32_t* write_off, float* part_o,
+                                                 float* part_ml, int splits, int keys_per_split, int waves,
+                                                 int rows_in_order, void* stream) {
+  HOLON_CHECK((q_weight == nullptr) == (k_weight == nullptr), "attention decode (fused): q and k norm weights come together");
+  HOLON_CHECK(qkv && pages && write_page && write_off, "attention decode (fused): the projection, the cache and write "
+              "targets are needed");
+  HOLON_CHECK(rope_table == nullptr || max_positions >= 1, "attention decode (fused): a rotation table of %d positions",
+              max_positions);
+  FusedArgs f{};
+  f.qkv = (const bf16_t*)qkv; f.qkv_stride = (int64_t)(heads + 2 * kv_heads) * head_dim;
+  f.q_weight = (const bf16_t*)q_weight; f.k_weight = (const bf16_t*)k_weight; f.eps = eps;
+  f.table = rope_table; f.max_positions = max_positions; f.pages = (bf16_t*)pages;
+  f.write_page = write_page; f.write_off = write_off;
+  return decode_launch(nullptr, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len,
+                       heads, kv_heads, head_dim, page_size, scale, window, part_o, part_ml, splits, keys_per_split,
+                       stream, &f, waves, rows_in_order);
 }
 
 // ---- decode attention for callers that cannot allocate ------------------------------------------------------------

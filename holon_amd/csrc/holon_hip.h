@@ -53,6 +53,28 @@ int holon_attention_decode_bf16(const void* q, void* out, const void* pages, con
                                 const int32_t* row_ids, int n_rows, int max_len, int heads, int kv_heads, int head_dim,
                                 int page_size, float scale, int window, float* part_o, float* part_ml, int splits,
                                 int keys_per_split, void* stream);
+// The same with `waves` waves a block (1 to 8, a divisor of `splits`), whose partials are combined through LDS: a
+// (row, head) leaves splits / waves partials (the workspace's third dimension), and when that is one the block writes
+// the result itself (the workspace may then be NULL, and no merge runs). rows_in_order: every row of the step is a
+// decode row with row_ids[i] = i and query_start[i] = i (neither array is then read).
+int holon_attention_decode_waves_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                      int table_stride, const int32_t* slots, const int32_t* lens,
+                                      const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
+                                      int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
+                                      float* part_o, float* part_ml, int splits, int keys_per_split, int waves,
+                                      int rows_in_order, void* stream);
+// The same from the step's raw q/k/v projection `qkv` [T, (heads + 2 kv_heads) head_dim]: per-head RMSNorm (q_weight
+// and k_weight, both or neither), rotation (rope_table [max_positions, head_dim] = cos | sin, or NULL) and the cache
+// write of every row's new token (write_page, write_off by token; its position is the row's len - 1) happen inside
+// the attention kernel.
+int holon_attention_decode_fused_bf16(const void* qkv, void* out, void* pages, const int32_t* table, int table_stride,
+                                      const int32_t* slots, const int32_t* lens, const int32_t* query_start,
+                                      const int32_t* row_ids, int n_rows, int max_len, int heads, int kv_heads,
+                                      int head_dim, int page_size, float scale, int window, const void* q_weight,
+                                      const void* k_weight, float eps, const float* rope_table,
+                                      int max_positions, const int32_t* write_page, const int32_t* write_off,
+                                      float* part_o, float* part_ml, int splits, int keys_per_split, int waves,
+                                      int rows_in_order, void* stream);
 // The same decode attention for callers that cannot allocate device memory (code under HIP graph capture, tight serving
 // loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. The split partials that
 // holon_attention_decode_bf16 takes as a workspace live in a device array inside the library instead, of

@@ -83,7 +83,7 @@ class StepRunner:
         for _, rows, contents in dirty:
             arrays += [rows, contents]
         facts = dict(fixed=fixed, dirty=[(g, len(rows)) for g, rows, _ in dirty],
-                     total=total, n_rows=len(slots), n_decode=len(decode), n_chunk=len(chunk),
+                     total=total, n_rows=len(slots), n_decode=len(decode), n_chunk=len(chunk), in_order=total == n,
                      max_decode_len=int(lens[decode].max()) if len(decode) else 0,
                      max_chunk_query=int(counts[chunk].max()) if len(chunk) else 0,
                      max_chunk_len=int(lens[chunk].max()) if len(chunk) else 0)
@@ -133,7 +133,8 @@ class StepRunner:
                  for i, g in enumerate(cache.groups)}
         attn = AttnRows(slots=dev[3], lens=dev[5], query_start=dev[6], decode_rows=dev[7], chunk_rows=dev[8],
                         n_decode=facts["n_decode"], n_chunk=facts["n_chunk"], max_decode_len=facts["max_decode_len"],
-                        max_chunk_query=facts["max_chunk_query"], max_chunk_len=facts["max_chunk_len"])
+                        max_chunk_query=facts["max_chunk_query"], max_chunk_len=facts["max_chunk_len"],
+                        in_order=facts["in_order"])
         return Step(kernels=self.kernels, n_tokens=facts["total"], n_rows=facts["n_rows"], token_ids=dev[0],
                     positions=dev[1], token_row=dev[2], slots=dev[3], starts=dev[4], rows=attn, paged=paged,
                     h_slots=slots, h_starts=starts, h_counts=counts, token_take=(dev[9], self.last_token))

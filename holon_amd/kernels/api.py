@@ -26,7 +26,8 @@ class AttnRows:
     """The rows of a step, as attention sees them. Row b reads block table row `slots[b]`, holds `lens[b]` tokens
     including this step's, and owns query tokens `query_start[b]:query_start[b+1]`, the last of its sequence
     ("bottom-right causal": query i of the row sits at position lens[b] - n_query[b] + i). Rows with one query token
-    are listed in `decode_rows`, the others in `chunk_rows` (row indices, int32, device)."""
+    are listed in `decode_rows`, the others in `chunk_rows` (row indices, int32, device). `in_order` says that the
+    step is decode rows alone, listed as they lie (a kernel then need not read the lists)."""
 
     slots: torch.Tensor                  # [B] int32
     lens: torch.Tensor                   # [B] int32
@@ -38,6 +39,7 @@ class AttnRows:
     max_decode_len: int                  # host bounds for launch shapes
     max_chunk_query: int
     max_chunk_len: int
+    in_order: bool = False               # every row is a decode row, and decode_rows[i] = query_start[i] = i
 
 
 class Kernels(Protocol):
@@ -135,6 +137,15 @@ class Kernels(Protocol):
                         page_size: int, scale: float, window: int) -> torch.Tensor:
         """softmax(q k^T * scale) v per row over its cached tokens, causal; with window W > 0 a query at position p
         sees keys p-W+1 .. p. q [T, Hq, D] -> [T, Hq, D]. This step's keys are already in the cache."""
+
+    def qkv_attention(self, qkv: torch.Tensor, heads: int, kv_heads: int, head_dim: int,
+                      q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float,
+                      rope_table: torch.Tensor | None, positions: torch.Tensor, pages: torch.Tensor | None,
+                      table: torch.Tensor, write_page: torch.Tensor, write_off: torch.Tensor, rows: AttnRows,
+                      page_size: int, scale: float, window: int, writes: bool = True) -> torch.Tensor:
+        """`paged_attention(qk_norm_rope_write(qkv, ...), pages, table, rows, ...)` as one operation, with that
+        composition's roundings; a kernel set may run it in fewer kernels (a step of decode rows alone). `writes`
+        False: the keys and values are not stored (a run that reads another run's cache)."""
 
     def argmax(self, logits: torch.Tensor) -> torch.Tensor:
         """logits [R, V] float32 -> [R] int32, the first maximal index of each row."""

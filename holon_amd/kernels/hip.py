@@ -69,6 +69,10 @@ class HipKernels:
                                              _P],
             "holon_attention_decode_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P,
                                             _I, _I, _P],
+            "holon_attention_decode_waves_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
+                                                  _P, _P, _I, _I, _I, _I, _P],
+            "holon_attention_decode_fused_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
+                                                  _P, _P, _F, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P],
             "holon_gemm_skinny_supported": [_I, _I, _I],
             "holon_gemm_skinny_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
             "holon_tile_weight_bf16": [_P, _P, _I, _I, _P, _P],
@@ -443,11 +447,12 @@ class HipKernels:
         residual = torch.zeros((x.shape[0], n), dtype=torch.bfloat16, device=x.device)
         ones = torch.ones(n, dtype=torch.bfloat16, device=x.device)
         pairs = self._alike(weight, tiled)
+        rival = self._MID_FORMS[self._time_mid_forms(x, weight)]      # the vendor library's best form (kept only if it wins)
         took = {
             "parts": self._graph_time(self._in_turn(
                 pairs, lambda w, t: self.add_rmsnorm(self._rows_parts(x, w, t, splits), residual, ones, 1e-6))),
             "vendor": self._graph_time(self._in_turn(
-                pairs, lambda w, _t: self.add_rmsnorm(self._vendor_product(x, w), residual, ones, 1e-6)))}
+                pairs, lambda w, _t: self.add_rmsnorm(rival(x, w), residual, ones, 1e-6)))}
         return "parts" if took["parts"] < 0.97 * took["vendor"] else "vendor"
 
     def sum_parts(self, parts, dtype=torch.bfloat16):
@@ -464,8 +469,8 @@ class HipKernels:
     def _time_rows(self, rows, weight, tiled, gated) -> str:
         x = torch.randn(rows, weight.shape[1], device=weight.device).to(torch.bfloat16)
         pairs = self._alike(weight, tiled)
-        vendor = (lambda w, _t: self.silu_mul(self._vendor_product(x, w))) if gated \
-            else (lambda w, _t: self._vendor_product(x, w))
+        rival = self._MID_FORMS[self._time_mid_forms(x, weight)]      # the vendor library's best form (kept only if it wins)
+        vendor = (lambda w, _t: self.silu_mul(rival(x, w))) if gated else (lambda w, _t: rival(x, w))
         took = {"rows": self._graph_time(self._in_turn(pairs, lambda w, t: self._rows_product(x, w, t, gated))),
                 "vendor": self._graph_time(self._in_turn(pairs, vendor))}
         return "rows" if took["rows"] < took["vendor"] else "vendor"
@@ -591,12 +596,12 @@ class HipKernels:
                            self._stream())
             if rows.n_decode:
                 span = rows.max_decode_len if not window else min(rows.max_decode_len, window + 31)
-                splits, per = self.decode_splits(rows.n_decode * hkv * ((hq // hkv + 15) // 16), span)
-                part_o = torch.empty((rows.n_decode * hq * splits * d,), dtype=torch.float32, device=q.device)
-                part_ml = torch.empty((rows.n_decode * hq * splits * 2,), dtype=torch.float32, device=q.device)
-                self._call(self.lib.holon_attention_decode_bf16, *common, rows.decode_rows.data_ptr(), rows.n_decode,
-                           rows.max_decode_len, hq, hkv, d, page_size, float(scale), int(window), part_o.data_ptr(),
-                           part_ml.data_ptr(), splits, per, self._stream())
+                splits, per, waves = self.decode_splits(rows.n_decode * hkv * ((hq // hkv + 15) // 16), span, d)
+                part_o, part_ml = self._decode_parts(rows.n_decode * hq * (splits // waves), d, q.device)
+                self._call(self.lib.holon_attention_decode_waves_bf16, *common, rows.decode_rows.data_ptr(),
+                           rows.n_decode, rows.max_decode_len, hq, hkv, d, page_size, float(scale), int(window),
+                           _ptr(part_o), _ptr(part_ml), splits, per, waves, int(rows.in_order and rows.n_decode == t),
+                           self._stream())
             return out
         self._call(self.lib.holon_attention_generic, q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(),
                    table.shape[1], rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr(), b, t, hq,
@@ -604,14 +609,82 @@ class HipKernels:
                    self._stream())
         return out
 
+    def qkv_attention(self, qkv, heads, kv_heads, head_dim, q_weight, k_weight, eps, rope_table, positions, pages,
+                      table, write_page, write_off, rows: AttnRows, page_size, scale, window, writes=True):
+        """`paged_attention(qk_norm_rope_write(qkv, ...), ...)`. A step of decode rows alone over the matrix-core
+        kernels runs as one kernel less: the attention kernel takes the raw projection, norms and rotates the queries
+        itself and puts each row's new key and value into the cache before it reads them."""
+        t = qkv.shape[0]
+        if not (qkv.dtype == torch.bfloat16 and writes and rows.n_chunk == 0 and rows.n_decode == t
+                and (rope_table is None or rope_table.shape[1] == head_dim)
+                and self.lib.holon_attention_mfma_supported(head_dim, page_size, _DT[torch.bfloat16])):
+            q = self.qk_norm_rope_write(qkv, heads, kv_heads, head_dim, q_weight, k_weight, eps, rope_table, positions,
+                                        pages if writes else None, write_page, write_off, page_size)
+            return self.paged_attention(q, pages, table, rows, page_size, scale, window)
+        self._check(qkv, "qkv", torch.bfloat16)
+        self._check(pages, "attention pages", torch.bfloat16)
+        self._check(table, "block table", torch.int32)
+        if qkv.shape[1] != (heads + 2 * kv_heads) * head_dim:
+            raise KernelError(f"qkv width {qkv.shape[1]} is not ({heads} + 2*{kv_heads}) * {head_dim}")
+        if pages.shape[1:] != (2, kv_heads, page_size * head_dim):
+            raise KernelError(f"pages {tuple(pages.shape)} do not fit {kv_heads} heads of {head_dim}, page {page_size}")
+        for w in (q_weight, k_weight):
+            if w is not None:
+                self._check(w, "q/k norm weight", torch.bfloat16)
+                if w.shape != (head_dim,):
+                    raise KernelError(f"q/k norm weight {tuple(w.shape)} does not fit head_dim {head_dim}")
+        if (q_weight is None) != (k_weight is None):
+            raise KernelError("q and k norm weights come together")
+        if rope_table is not None:
+            self._check(rope_table, "rope table", torch.float32)
+        for ix, what in ((write_page, "write_page"), (write_off, "write_off")):
+            self._check(ix, what, torch.int32)
+            if ix.shape[0] < t:
+                raise KernelError(f"{what}: {ix.shape[0]} entries for {t} tokens")
+        out = torch.empty((t, heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+        span = rows.max_decode_len if not window else min(rows.max_decode_len, window + 31)
+        splits, per, waves = self.decode_splits(rows.n_decode * kv_heads * ((heads // kv_heads + 15) // 16), span,
+                                                head_dim)
+        part_o, part_ml = self._decode_parts(rows.n_decode * heads * (splits // waves), head_dim, qkv.device)
+        self._call(self.lib.holon_attention_decode_fused_bf16, qkv.data_ptr(), out.data_ptr(), pages.data_ptr(),
+                   table.data_ptr(), table.shape[1], rows.slots.data_ptr(), rows.lens.data_ptr(),
+                   rows.query_start.data_ptr(), rows.decode_rows.data_ptr(), rows.n_decode, rows.max_decode_len, heads,
+                   kv_heads, head_dim, page_size, float(scale), int(window), _ptr(q_weight), _ptr(k_weight), float(eps),
+                   _ptr(rope_table), rope_table.shape[0] if rope_table is not None else 0, write_page.data_ptr(),
+                   write_off.data_ptr(), _ptr(part_o), _ptr(part_ml), splits, per, waves, int(rows.in_order),
+                   self._stream())
+        return out
+
     @staticmethod
-    def decode_splits(waves_per_split: int, span: int, target_waves: int = 2048, min_keys: int = 64) -> tuple[int, int]:
-        """How a decode row's keys are cut over waves: (splits, keys per split, a multiple of 32), enough waves to
-        fill the GPU but at least `min_keys` keys each."""
-        want = max(1, min(64, target_waves // max(1, waves_per_split)))
+    def _decode_parts(cells: int, head_dim: int, device):
+        """The split partials' workspace: (values [cells, head_dim], maxima and sums [cells, 2]); none where every
+        block writes its row's result."""
+        if cells == 0:
+            return None, None
+        return (torch.empty((cells * head_dim,), dtype=torch.float32, device=device),
+                torch.empty((cells * 2,), dtype=torch.float32, device=device))
+
+    @staticmethod
+    def decode_splits(pairs: int, span: int, head_dim: int = 128, target_waves: int = 2048, min_keys: int = 64,
+                      blocks: int | None = None) -> tuple[int, int, int]:
+        """How a decode row's keys are cut over waves: (splits, keys per split, waves a block). `pairs`: (row, kv head)
+        tiles in the launch. Enough waves to fill the GPU but at least `min_keys` keys each (a multiple of 32); the
+        waves of a block combine their partials through LDS, so as many of a row's splits share a block as leave
+        `blocks` blocks in the launch and fit LDS (at most 8): a (row, head) then leaves splits / waves partials for
+        the merge, and with one block a row none (the block writes the result, no merge runs). The last return value
+        times the number of partials is the splits. Measured at context 4,096 (attention + merge, us a layer): one row
+        18.3 with 256 blocks against 19.6 with 512; eight rows 37.3 with 512 against 38.6 with 256."""
+        if blocks is None:
+            blocks = 256 if pairs <= 16 else 512
+        want = max(1, min(64, target_waves // max(1, pairs)))
         per = max(min_keys, -(-span // want))
         per = -(-per // 32) * 32
-        return max(1, -(-span // per)), per
+        splits = max(1, -(-span // per))
+        cap = max(1, min(8, (64 * 1024 // 4) // (16 * head_dim + 32) + 1))
+        outer = min(splits, max(1, -(-blocks // max(1, pairs))))
+        waves = min(cap, -(-splits // outer))
+        outer = -(-splits // waves)
+        return outer * waves, per, waves
 
     def argmax(self, logits):
         self._check(logits, "argmax logits", torch.float32)

@@ -74,10 +74,12 @@ class GQA(Part):
         pages = site.pages.view(-1, 2, hkv, view.page_size * d)
         qkv = self.qkv(x)
         if self._fused is not None:
-            q = k.qk_norm_rope_write(
+            out = k.qkv_attention(
                 qkv, hq, hkv, d, self.q_norm.weight if self.q_norm is not None else None,
                 self.k_norm.weight if self.k_norm is not None else None, self._fused["eps"], self._fused["table"],
-                step.positions, pages if site.writes else None, view.write_page, view.write_off, view.page_size)
+                step.positions, pages, view.table, view.write_page, view.write_off, step.rows, view.page_size,
+                self.scale, self.window, writes=site.writes)
+            return self.o_proj(out.view(t, hq * d), residual=residual)
         else:
             q = qkv[:, : hq * d].contiguous().view(t, hq, d)
             kk = qkv[:, hq * d: (hq + hkv) * d].contiguous().view(t, hkv, d) if site.writes else None

@@ -191,6 +191,12 @@ class TorchKernels:
         order = lp.argsort(dim=-1, descending=True, stable=True)[:, :k]
         return lp.gather(-1, tokens.long()[:, None])[:, 0], order.to(torch.int32), lp.gather(-1, order)
 
+    def qkv_attention(self, qkv, heads, kv_heads, head_dim, q_weight, k_weight, eps, rope_table, positions, pages,
+                      table, write_page, write_off, rows, page_size, scale, window, writes=True):
+        q = self.qk_norm_rope_write(qkv, heads, kv_heads, head_dim, q_weight, k_weight, eps, rope_table, positions,
+                                    pages if writes else None, write_page, write_off, page_size)
+        return self.paged_attention(q, pages, table, rows, page_size, scale, window)
+
     def scatter_rows(self, dst, idx, src):
         dst[idx.long()] = src.view(idx.shape[0], dst.shape[1])
 
