@@ -7,11 +7,15 @@
 
 One JSON line: decoded tokens a second at the given batch (default 8) with every request near a context of 4,096 tokens
 (the far end of a 2,048-token prompt and 2,048 generated tokens: the requests are given prompts that leave just the
-timed steps, `config.decode_prompt_len`), plus the prefill of one 2,048-token prompt, the decode step's memory
-roofline, decode at batch 1 and 64 with their step times and roofline fractions (`points`), and the time to the first
-token of the 2,048-token prompt and the median time between two tokens of a request (`latency`, as the reference's
-driver reports them: bench/driver.py:102-134). A step is one decode step of the engine: scheduling, the model, sampling and
-the commit. The engine is one process on one GPU; for --gpus > 1 a line says so and the exit code is 2.
+timed steps, `config.decode_prompt_len`), plus the prefill of one 2,048-token prompt (`prefill.ms` is the best of three
+prompts, `prefill.ms_median` their median), the decode step's memory roofline, and `points`: decode at batch 1, 16, 32
+and 64 at the same context and at batch 8 at a context of 32,768 (tokens a second, ms a step, the gigabytes a step
+must read, the fraction of the memory roofline), and prompts of 512 and 8,192 tokens (tokens a second, best and median
+ms, TFLOP, the fraction of the matrix peak; the longer one takes two steps under the step budget of 4,096 tokens).
+`latency` holds the time to the first token of the 2,048-token prompt and the median time between two tokens of a
+request, as the reference's driver reports them (bench/driver.py:102-134); `products` what every matrix product with
+a choice of kernels took. A step is one decode step of the engine: scheduling, the model, sampling and the commit.
+The engine is one process on one GPU; for --gpus > 1 a line says so and the exit code is 2.
 
 --workload runs a whole job through the engine instead and prints its own line: `mixed` is 32 requests of 128 to 4,096
 prompt tokens at the Qwen3-32B shape, portions of 512 tokens beside decode rows, 256 greedy tokens each; `long` is 8
@@ -31,6 +35,9 @@ QWEN3_8B = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 36, "hid
             "vocab_size": 151936, "rope_theta": 1e6, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
             "max_position_embeddings": 40960}
 CONTEXT, PROMPT = 4096, 2048
+LONG_CONTEXT = 32768            # the context of the long decode point (batch 8)
+POINT_BATCHES = (1, 16, 32, 64)
+POINT_PROMPTS = (512, 8192)
 QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
 QWEN3_4B = dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, tie_word_embeddings=True)
 
@@ -98,7 +105,7 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"],
                     help="fewer layers than the configuration has (recorded in config)")
     ap.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
-    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-points", action="store_true", help="skip the further decode and prefill points")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--workload", choices=("decode", "mixed", "long"), default="decode")
     ap.add_argument("--products", choices=("own", "vendor", "timed"), default="timed",
@@ -122,22 +129,24 @@ def main(argv: list[str] | None = None) -> int:
     if kernel_build.find_library() is None:
         kernel_build.build()
     cfg_json = dict(QWEN3_8B, num_hidden_layers=a.layers)
-    max_batch = max(a.batch, 1 if a.no_points else 64)
+    max_batch = max(a.batch, 1 if a.no_points else max(POINT_BATCHES))
+    longest = CONTEXT if a.no_points else max(LONG_CONTEXT, max(POINT_PROMPTS))
     engine = Engine.from_random(cfg_json, seed=0, cfg=EngineConfig(
         model="random:qwen3-8b", device="cuda:0", dtype=a.dtype, page_size=16, max_seqs=max_batch,
-        max_model_len=CONTEXT + 16, max_step_tokens=4096, cache_tokens=max_batch * (CONTEXT + 16),
+        max_model_len=longest + 16, max_step_tokens=4096,
+        cache_tokens=max(max_batch * (CONTEXT + 16), 0 if a.no_points else 8 * (LONG_CONTEXT + 16)),
         graphs=not a.no_graphs, products=a.products))
     spec, c = engine.spec, cfg_json
     item = 2 if a.dtype == "bfloat16" else 4
     g = torch.Generator().manual_seed(0)
     greedy = lambda n: SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True)
 
-    def decode(batch: int, steps: int, warmup: int) -> tuple[float, float, float, int]:
+    def decode(batch: int, steps: int, warmup: int, context: int = CONTEXT) -> tuple[float, float, float, int]:
         """(ms per decode step, mean context, median ms between two steps' ends, prompt length) for `batch` requests
-        whose contexts end at CONTEXT. The requests go on for two steps after the timed ones, so that the host's work
+        whose contexts end at `context`. The requests go on for two steps after the timed ones, so that the host's work
         for finished requests (not part of a decode step) falls outside the timed region."""
         after = 2
-        start = CONTEXT - steps - warmup - 1 - after
+        start = context - steps - warmup - 1 - after
         for _ in range(batch):
             engine.add(torch.randint(0, c["vocab_size"], (start,), generator=g).tolist(),
                        greedy(steps + warmup + 1 + after))
@@ -159,15 +168,17 @@ def main(argv: list[str] | None = None) -> int:
         return ms, start + 1 + warmup + steps / 2, gaps[len(gaps) // 2] * 1e3, start
 
     def prefill(tokens: int) -> tuple[float, float]:
-        """(best, median) ms from adding a prompt of `tokens` to its first generated token on the host."""
+        """(best, median) ms from adding a prompt of `tokens` to its first generated token on the host: one step, or as
+        many as the step budget cuts the prompt into."""
         times = []
         for _ in range(3):                     # another prompt each time: nothing of it is in the prefix cache
             ids = torch.randint(0, c["vocab_size"], (tokens,), generator=g).tolist()
             engine.add(ids, greedy(1))
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            engine.step()
-            engine.drain()                     # the step's one token on the host: the request is finished
+            while engine.has_work():
+                engine.step()
+            engine.drain()                     # the last step's one token on the host: the request is finished
             torch.cuda.synchronize()
             times.append((time.perf_counter() - t0) * 1e3)
             assert not engine.has_work()
@@ -178,19 +189,34 @@ def main(argv: list[str] | None = None) -> int:
     layer_params = h * (hq + 2 * hkv) * d + hq * d * h + 3 * h * inter
     weight_bytes = (layers * (layer_params + 2 * h + 2 * d) + h + h * v) * item      # every weight a decode step reads
     kv_token_bytes = layers * 2 * hkv * d * item
+    def prompt_flops(tokens: int) -> float:
+        """Products of every layer over `tokens` rows, causal attention (half of the square), the head on one row."""
+        return layers * (2 * tokens * layer_params + 2 * hq * d * tokens * tokens) + 2 * h * v
+
     pre_ms, ttft_ms = prefill(PROMPT)
-    pre_flops = layers * (2 * PROMPT * layer_params + 2 * hq * d * PROMPT * PROMPT) + 2 * h * v
+    pre_flops = prompt_flops(PROMPT)
     ms, ctx, tpot_ms, decode_prompt = decode(a.batch, a.steps, a.warmup)
     step_bytes = weight_bytes + a.batch * ctx * kv_token_bytes
     achieved = step_bytes / (ms * 1e-3) / 1e9
     points = {}
     if not a.no_points:
-        for b in (1, 64):
-            pms, pctx, _, _ = decode(b, a.steps, a.warmup)
-            points[f"decode_b{b}"] = round(b / (pms * 1e-3), 1)
-            points[f"decode_b{b}_ms"] = round(pms, 4)
-            points[f"decode_b{b}_gb"] = round((weight_bytes + b * pctx * kv_token_bytes) / 1e9, 2)
-            points[f"decode_b{b}_frac"] = round((weight_bytes + b * pctx * kv_token_bytes) / (pms * 1e-3) / 1e9 / HBM_GBS, 4)
+        def decode_point(name: str, b: int, context: int) -> None:
+            pms, pctx, _, _ = decode(b, a.steps, a.warmup, context)
+            gb = (weight_bytes + b * pctx * kv_token_bytes) / 1e9
+            points[name] = round(b / (pms * 1e-3), 1)
+            points[f"{name}_ms"] = round(pms, 4)
+            points[f"{name}_gb"] = round(gb, 2)
+            points[f"{name}_frac"] = round(gb / (pms * 1e-3) / HBM_GBS, 4)
+        for b in POINT_BATCHES:
+            decode_point(f"decode_b{b}", b, CONTEXT)
+        decode_point(f"decode_b8_ctx{LONG_CONTEXT}", 8, LONG_CONTEXT)
+        for tokens in POINT_PROMPTS:
+            best, median = prefill(tokens)
+            points[f"prefill_{tokens}"] = round(tokens / (best * 1e-3), 1)
+            points[f"prefill_{tokens}_ms"] = round(best, 3)
+            points[f"prefill_{tokens}_ms_median"] = round(median, 3)
+            points[f"prefill_{tokens}_tflop"] = round(prompt_flops(tokens) / 1e12, 2)
+            points[f"prefill_{tokens}_frac"] = round(prompt_flops(tokens) / (best * 1e-3) / PEAK_FLOPS[a.dtype], 4)
     line = {
         "metric": f"decode tok/s at batch {a.batch} (context 4,096), Qwen3-8B shape", "value": round(a.batch / (ms * 1e-3), 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
@@ -203,6 +229,7 @@ def main(argv: list[str] | None = None) -> int:
                    "parallelism": "single GPU", "graphs": not a.no_graphs, "mean_context": round(ctx, 1),
                    "products": a.products},
         "prefill": {"value": round(PROMPT / (pre_ms * 1e-3), 1), "tokens": PROMPT, "ms": round(pre_ms, 3),
+                    "ms_is": "best of 3 prompts", "ms_median": round(ttft_ms, 3),
                     "frac": round(pre_flops / (pre_ms * 1e-3) / PEAK_FLOPS[a.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},
