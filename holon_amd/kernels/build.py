@@ -110,5 +110,35 @@ def build(verbose: bool = True, force: bool = True) -> pathlib.Path:
     return target
 
 
+def source_library(source: str | pathlib.Path) -> pathlib.Path | None:
+    """The library built from one source file of a part's own (`lib<stem>.so` beside it, else in the per-user folder),
+    if it is there and not older than the source."""
+    source = pathlib.Path(source).resolve()
+    for cand in (source.with_name(f"lib{source.stem}.so"), fallback_dir() / f"lib{source.stem}.so"):
+        if cand.is_file() and cand.stat().st_mtime >= source.stat().st_mtime:
+            return cand
+    return None
+
+
+def build_source(source: str | pathlib.Path, verbose: bool = True) -> pathlib.Path:
+    """Compile one HIP source that a part brings with it into a library of its own, with this package's flags and
+    headers (`holon_amd/csrc` is on the include path: `common.h` may be used)."""
+    source = pathlib.Path(source).resolve()
+    target = source.with_name(f"lib{source.stem}.so")
+    if not _writable(target.parent):
+        fallback_dir().mkdir(parents=True, exist_ok=True)
+        target = fallback_dir() / target.name
+    tmp = target.parent / f"{target.name}.tmp{os.getpid()}"
+    t0 = time.time()
+    proc = subprocess.run([hipcc(), *HIP_FLAGS, "-shared", f"-I{CSRC}", str(source), "-o", str(tmp)],
+                          capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {source}:\n{proc.stderr[-4000:]}")
+    os.replace(tmp, target)
+    if verbose:
+        print(f"holon_amd: built {target} in {time.time() - t0:.0f} s", file=sys.stderr, flush=True)
+    return target
+
+
 if __name__ == "__main__":
     build()

@@ -13,6 +13,7 @@ import torch
 
 from . import build as _build
 from .api import AttnRows
+from .registry import kernel_op
 from ..config.products import ProductPlan, row_bucket
 
 _P, _I, _L, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
@@ -115,6 +116,38 @@ class HipKernels:
         if time is not None and (not self.plan.resolving or torch.cuda.is_current_stream_capturing()):
             time = None
         return self.plan.choose(kind, tuple(weight.shape), row_bucket(rows), time)
+
+    # -- operations that parts bring with them ----------------------------------------------------------------------
+    _part_libs: dict[str, ctypes.CDLL] = {}       # libraries built from parts' own sources, by source path
+
+    def __getattr__(self, name: str):
+        """An operation registered with `holon_amd.kernels.registry.register_kernel`: its HIP form when it has one
+        (the symbol from this library, or from the library built from the operation's own source), else its plain
+        form."""
+        op = kernel_op(name) if not name.startswith("_") else None
+        if op is None:
+            raise AttributeError(f"{type(self).__name__} has no operation {name!r}")
+        if op.symbol is None:
+            return op.plain
+        lib = self.lib
+        if op.source is not None:
+            key = str(op.source)
+            lib = self._part_libs.get(key)
+            if lib is None:
+                path = _build.source_library(op.source) or _build.build_source(op.source)
+                try:
+                    lib = self._part_libs[key] = ctypes.CDLL(str(path))
+                except OSError as e:
+                    raise KernelError(f"cannot load {path}: {e}") from e
+        fn = getattr(lib, op.symbol)
+        fn.argtypes, fn.restype = [*op.argtypes, _P], _I
+
+        def launch(*args) -> None:
+            rc = fn(*args, self._stream())
+            if rc != 0:
+                detail = self.lib.holon_last_error().decode() if op.source is None else f"returned {rc}"
+                raise KernelError(f"{op.symbol}: {detail}")
+        return lambda *args, **kwargs: op.call(launch, *args, **kwargs)
 
     # -- plumbing -------------------------------------------------------------------------------------------------
     def _call(self, fn, *args) -> None:

@@ -155,14 +155,68 @@ class Part:
         there; the scheduler asks every part of the model and takes the smallest answer. Default: all of them."""
         return count
 
+    def absorb_norm(self, norm: "Part") -> bool:
+        """A mixer or feed-forward whose first product can take the norm in front of it into its own kernel folds the
+        norm's weight into its weights now and answers True; it is from then on handed the norm deferred
+        (`norm.defer(...)`) instead of the norm's result. Default: it cannot."""
+        return False
+
+    def extra_tensors(self) -> list[torch.Tensor]:
+        """Device tensors this part holds beside its declared parameters (copies in another layout, tables): what
+        `nbytes` counts on top of them."""
+        return []
+
     def nbytes(self) -> int:
         total = 0
         for part in self.walk():
-            for name in part._decls:
-                t = getattr(part, name)
-                if t is not None:
-                    total += t.numel() * t.element_size()
-            tiled = getattr(part, "tiled", None)
-            if tiled is not None:
-                total += tiled.numel() * tiled.element_size()
+            held = [getattr(part, name) for name in part._decls] + list(part.extra_tensors())
+            total += sum(t.numel() * t.element_size() for t in held if t is not None)
         return total
+
+
+class NormPart(Part):
+    """What the model and the blocks ask of a norm. A norm implements `forward`; the rest has defaults that run it as
+    a kernel of its own. A norm that fused kernels can take over describes itself in `fusion` and may hand out its
+    result deferred (`defer`)."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        return self.forward(x)
+
+    def add(self, x: "torch.Tensor | PartialSums", residual: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        """(norm(residual + x), residual + x); the sum, rounded to the residual's dtype, replaces `residual` in place."""
+        residual.add_(x.value() if isinstance(x, PartialSums) else x)
+        return self.forward(residual), residual
+
+    def fusion(self) -> dict | None:
+        """What a fused kernel needs to do this norm itself ({"norm": kind, "eps": ..., "weight": ...}); None: no
+        kernel takes it over, it always runs by itself."""
+        return None
+
+    defer = None              # a norm that can be folded into the product that reads it offers
+                              # defer(h, stats, delta) -> an object with value() (see norms.Normed)
+
+
+class EmbedPart(Part):
+    """What the model asks of the part that turns token ids into rows of the residual stream. A part implements
+    `rows(ids)`; `forward` adds what the step function may ask for beside it."""
+
+    def rows(self, ids: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def forward(self, ids: torch.Tensor, take: tuple[torch.Tensor, torch.Tensor] | None = None,
+                want_stats: bool = False):
+        """ids [T] int32 -> rows [T, hidden]. `take` = (take_slot [T], last_token [slots]): where take_slot[t] >= 0
+        the token is last_token[take_slot[t]], one that the step before drew and left on the device. With
+        `want_stats` the answer is (rows, statistics of the rows for a norm that follows, or None): a part whose
+        kernel leaves none answers None."""
+        if take is not None:
+            slot, last = take
+            ids = torch.where(slot >= 0, last[slot.clamp(min=0).long()], ids)
+        out = self.rows(ids)
+        return (out, None) if want_stats else out
+
+    def __call__(self, *args, **kwargs):
+        return self.forward(*args, **kwargs)

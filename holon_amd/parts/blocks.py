@@ -26,8 +26,8 @@ class PreNorm(Part):
     def finalize(self) -> None:
         """A mixer or feed-forward that can fold the norm in front of it into its own first product does so now (its
         weights are loaded and merged); it is then handed the norm deferred (`Normed`) instead of its result."""
-        self._mixer_defers = bool(getattr(self.mixer, "absorb_norm", None)) and self.mixer.absorb_norm(self.input_norm)
-        self._ffn_defers = bool(getattr(self.ffn, "absorb_norm", None)) and self.ffn.absorb_norm(self.post_norm)
+        self._mixer_defers = self.input_norm.defer is not None and bool(self.mixer.absorb_norm(self.input_norm))
+        self._ffn_defers = self.post_norm.defer is not None and bool(self.ffn.absorb_norm(self.post_norm))
 
     _mixer_defers = _ffn_defers = False
 

@@ -4,16 +4,19 @@ from __future__ import annotations
 import torch
 
 from ..registry import register_part
-from .base import Build, Part
+from .base import Build, EmbedPart, Part
 
 
 @register_part("embed", "table")
-class Embedding(Part):
+class Embedding(EmbedPart):
     graph_safe = True
 
     def __init__(self, build: Build, *, vocab: int, hidden: int) -> None:
         super().__init__(build)
         self.declare("weight", (vocab, hidden))
+
+    def rows(self, ids: torch.Tensor) -> torch.Tensor:
+        return self.kernels.embedding(ids, self.weight)
 
     def forward(self, ids: torch.Tensor, take: tuple[torch.Tensor, torch.Tensor] | None = None,
                 want_stats: bool = False):
@@ -44,6 +47,9 @@ class LMHead(Part):
     def finalize(self) -> None:
         if self.build.decode_copy and self._weight() is not None:
             self.tiled = self.kernels.tile_weight(self._weight())
+
+    def extra_tensors(self) -> list[torch.Tensor]:
+        return [self.tiled] if self.tiled is not None else []
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         return self.kernels.linear(h, self._weight(), torch.float32, self.tiled)

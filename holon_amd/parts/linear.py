@@ -22,12 +22,15 @@ class Linear(Part):
         if self.weight is not None and self.build.decode_copy:
             self.tiled = self.kernels.tile_weight(self.weight)
 
+    def extra_tensors(self) -> list[torch.Tensor]:
+        return [self.tiled] if self.tiled is not None else []
+
     def absorb(self, norm: Part) -> bool:
         """Fold the weight of the norm in front of this projection into the tiled copy, so that steps of few rows
         need no kernel for the norm: the product runs over the un-normed rows and scales each by the norm's factor
         (`forward` with a `Normed`). The tiled copy then serves only such input. False when this norm or this weight
         cannot be folded; nothing changes then."""
-        spec = norm.fusion() if hasattr(norm, "fusion") else None
+        spec = norm.fusion()
         if not self.build.decode_copy or self.weight is None or spec is None or spec.get("norm") != "rmsnorm" \
                 or spec["weight"] is None:
             return False

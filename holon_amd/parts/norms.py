@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 
 from ..registry import register_part
-from .base import Build, PartialSums, Part
+from .base import Build, NormPart, PartialSums
 
 
 def _term(x: "torch.Tensor | PartialSums") -> torch.Tensor:
@@ -47,7 +47,7 @@ class Normed:
 
 
 @register_part("norm", "rmsnorm")
-class RMSNorm(Part):
+class RMSNorm(NormPart):
     """y = x * rsqrt(mean(x^2) + eps) * weight over the last `dim` values, float32 inside, rounded once."""
 
     graph_safe = True

@@ -9,7 +9,7 @@ from typing import Any
 
 from .spec import ModelSpec, PartRef
 
-FAMILIES = ("mixer", "ffn", "norm", "position", "block", "embed", "head")
+FAMILIES = ("mixer", "ffn", "norm", "position", "block", "embed", "head")     # the built-in parts' families
 
 
 class RegistryError(KeyError):
@@ -62,26 +62,31 @@ def resolve(config_json: Mapping[str, Any], generation: Mapping[str, Any] | None
 
 
 def register_part(family: str, kind: str) -> Callable[[type], type]:
-    """Class decorator: `@register_part("mixer", "gqa")`."""
-    if family not in _PARTS:
-        raise RegistryError(f"no part family {family!r}; families: {FAMILIES}")
+    """Class decorator: `@register_part("mixer", "gqa")`. A family is any name: the first part of a new one (a
+    router, another kind of state) opens it."""
+    if not family or not isinstance(family, str):
+        raise RegistryError(f"a part family is a name, not {family!r}")
 
     def add(cls: type) -> type:
-        if kind in _PARTS[family]:
+        kinds = _PARTS.setdefault(family, {})
+        if kind in kinds:
             raise RegistryError(f"{family} {kind!r} is registered twice")
-        _PARTS[family][kind] = cls
+        kinds[kind] = cls
         return cls
     return add
 
 
 def unregister_part(family: str, kind: str) -> None:
-    _PARTS[family].pop(kind, None)
+    _PARTS.get(family, {}).pop(kind, None)
+    if family not in FAMILIES and not _PARTS.get(family, True):
+        del _PARTS[family]
 
 
 def part_class(ref: PartRef) -> type:
     _load_builtin()
     if ref.family not in _PARTS or ref.kind not in _PARTS[ref.family]:
-        raise RegistryError(f"no {ref.family} named {ref.kind!r}; registered: {sorted(_PARTS.get(ref.family, {}))}")
+        raise RegistryError(f"no {ref.family} named {ref.kind!r}; registered: {sorted(_PARTS.get(ref.family, {}))}"
+                            + ("" if ref.family in _PARTS else f" (families: {sorted(_PARTS)})"))
     return _PARTS[ref.family][ref.kind]
 
 

@@ -46,6 +46,14 @@ class TorchKernels:
     split_products = 0       # a test may set a number of shares: steps of 17 to 128 rows then get their products that
                              # are added to the residual stream as partial sums over that many shares of K
 
+    def __getattr__(self, name):
+        """An operation a part registered for itself (`holon_amd.kernels.registry`): its plain form."""
+        from holon_amd.kernels.registry import kernel_op
+        op = kernel_op(name) if not name.startswith("_") else None
+        if op is None:
+            raise AttributeError(f"TorchKernels has no operation {name!r}")
+        return op.plain
+
     def embedding(self, ids, table, take=None, want_stats=False):
         if take is not None:
             take_slot, last_token = take

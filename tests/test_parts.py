@@ -551,3 +551,144 @@ def test_toy_architecture_through_the_engine_with_a_portion_grid_and_graphs_aske
     finally:
         unregister_part("mixer", "test-grid-mean")
         unregister_architecture("ToyGridModel")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_mixer_that_brings_a_kernel_of_its_own(device, dtype):
+    """A toy mixer under tests/ registers the operation it needs beside itself: the plain form, and a HIP symbol with
+    its argument types and its own source file, which is compiled into a library of its own. Every kernel set then
+    answers `kernels.decay_scan(...)`: the plain twin runs the plain form, the HIP kernels the symbol. The toy
+    architecture generates through the engine (prompt portions under a small step budget, then decode steps, replayed
+    from graphs on the GPU) and its greedy tokens equal a whole-sequence computation written out here. No file of
+    the framework names the operation."""
+    from holon_amd.config import EngineConfig, SamplingParams
+    from holon_amd.engine.engine import Engine
+    from holon_amd.kernels.registry import kernel_ops, register_kernel, unregister_kernel
+    from holon_amd.registry import register_architecture, unregister_architecture
+    from tests.toy_parts import DecayScan, ToyScanConfig, decay_scan_op, toy_scan_recipe
+    register_kernel(decay_scan_op())
+    register_part("mixer", "test-decay-scan")(DecayScan)
+    register_architecture("ToyScanModel", ToyScanConfig, toy_scan_recipe)
+    try:
+        assert "decay_scan" in kernel_ops()
+        with pytest.raises(KeyError, match="twice"):
+            register_kernel(decay_scan_op())
+        config = {"architectures": ["ToyScanModel"], "width": 64, "tokens": 97, "depth": 2, "decay": 0.75, "eps": 1e-5}
+        kernels = _kernels(device)
+        engine = Engine.from_random(config, 5, EngineConfig(
+            model="random:toy-scan", device=device, dtype=dtype, page_size=4, max_seqs=4, max_model_len=96,
+            max_step_tokens=16, graphs=True, overlap=True), kernels=kernels)
+        assert engine.runner.use_graphs == (device == "cuda") and not engine.runner.not_graph_safe
+        with pytest.raises(AttributeError, match="no operation"):
+            kernels.an_operation_nobody_registered
+        w = _weights_of(engine.model)
+        dt = getattr(torch, dtype)
+
+        def logits(ids):
+            h = w["embed.weight"].to(dt)[torch.tensor(ids)]
+            for layer in (0, 1):
+                p = f"layers.{layer}."
+                x = plain.rms_norm(h, w[p + "input_norm.weight"].to(dt), 1e-5)
+                s, rows = torch.zeros(64), []
+                for t in range(len(ids)):
+                    s = 0.75 * s + x[t].float()
+                    rows.append(s.to(dt))
+                h = h + plain.linear(torch.stack(rows), w[p + "mixer.proj.weight"].to(dt))
+                x = plain.rms_norm(h, w[p + "post_norm.weight"].to(dt), 1e-5)
+                gu = w[p + "ffn.gate_up.weight"].to(dt)
+                h = h + plain.swiglu(x, gu[:128], gu[128:], w[p + "ffn.down_proj.weight"].to(dt))
+            return plain.linear(plain.rms_norm(h, w["norm.weight"].to(dt), 1e-5), w["embed.weight"].to(dt)).float()
+
+        def greedy_follows(prompt, got):
+            ids = list(prompt)
+            for token in got:
+                last = logits(ids)[-1]
+                top = last.topk(2).values
+                if float(top[0] - top[1]) > (1e-4 if dtype == "float32" else 0.05) * float(last.std()):
+                    assert token == int(last.argmax()), (len(ids), token, int(last.argmax()))
+                ids.append(token)
+        prompts = [H.random_ids(n, 97, 30 + n) for n in (37, 5, 21, 9)]
+        got = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+        for prompt, tokens in zip(prompts, got):
+            assert len(tokens) == 12
+            greedy_follows(prompt, tokens)
+        if device == "cuda":
+            from tests.toy_parts import DECAY_SCAN_SOURCE
+            assert str(DECAY_SCAN_SOURCE) in kernels._part_libs and engine.runner.graph_replays > 5
+    finally:
+        unregister_architecture("ToyScanModel")
+        unregister_part("mixer", "test-decay-scan")
+        unregister_kernel("decay_scan")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_norm_and_an_embedding_that_implement_only_their_base_class(device, dtype):
+    """Another norm (no weight: x centred, over its root mean square) and another embedding (the table's rows times a
+    constant) written as the base classes ask: `NormPart.forward`, `EmbedPart.rows`. What the model and the blocks
+    call beside these (the residual add in front of a norm, tokens taken from the device, row statistics, deferral,
+    fusion into other kernels) comes from the base classes' defaults: nothing is folded or fused, every step gives the
+    plain computation. A part of a family the framework does not know opens it."""
+    from holon_amd.parts import EmbedPart, NormPart
+    from holon_amd.registry import RegistryError, part_class
+
+    class Centred(NormPart):
+        graph_safe = True
+
+        def __init__(self, build, *, eps, dim):
+            super().__init__(build)
+            self.eps = eps
+
+        def forward(self, x):
+            x32 = x.float() - x.float().mean(-1, keepdim=True)
+            return (x32 * torch.rsqrt(x32.pow(2).mean(-1, keepdim=True) + self.eps)).to(x.dtype)
+
+    class ScaledTable(EmbedPart):
+        graph_safe = True
+
+        def __init__(self, build, *, vocab, hidden, scale):
+            super().__init__(build)
+            self.scale = scale
+            self.declare("weight", (vocab, hidden))
+
+        def rows(self, ids):
+            return (self.weight[ids.long()].float() * self.scale).to(self.weight.dtype)
+
+    register_part("norm", "test-centred")(Centred)
+    register_part("embed", "test-scaled-table")(ScaledTable)
+    register_part("test-family", "thing")(Centred)
+    try:
+        assert part_class(PartRef("test-family", "thing")) is Centred
+        with pytest.raises(RegistryError, match="test-family"):
+            part_class(PartRef("test-family", "other"))
+        hq, hkv, d, eps = 4, 2, 16, 1e-5
+        norm = PartRef("norm", "test-centred", eps=eps)
+        layer = LayerSpec(block=PartRef("block", "prenorm"), mixer=_gqa(hq, hkv, d), ffn=PartRef("ffn", "swiglu", inter=96),
+                          norm=norm)
+        spec = ModelSpec(hidden=64, vocab=97, layers=(layer, layer), order=in_order(2),
+                         embed=PartRef("embed", "test-scaled-table", scale=1.5), norm=norm,
+                         head=PartRef("head", "linear", tied=False), rules=())
+        model, w, cache, runner = _model(spec, device, dtype, 21, page_size=4, cache_tokens=96)
+        assert not model.blocks[0]._mixer_defers and not model.blocks[0]._ffn_defers        # nothing to fold
+        ids = H.random_ids(45, 97, 22)
+        pos = torch.arange(len(ids))
+
+        def centred(x):
+            x32 = x.float() - x.float().mean(-1, keepdim=True)
+            return (x32 * torch.rsqrt(x32.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype)
+
+        def logits(dt):
+            h = (w["embed.weight"].to(dt)[torch.tensor(ids)].float() * 1.5).to(dt)
+            for layer_at in (0, 1):
+                p = f"layers.{layer_at}."
+                h = h + _plain_attention(centred(h), pos, w, p + "mixer.", hq, hkv, d, 1e-6, 1e4)[0]
+                h = h + _plain_ffn(centred(h), w, p + "ffn.")
+            return plain.linear(centred(h), w["lm_head.weight"].to(dt)).float()
+        want, floor = logits(torch.float32), logits(torch.bfloat16)
+        for cuts, also in (([45], ()), ([13] + [1] * 32, ()), ([3, 2, 17, 9, 14], (H.random_ids(13, 97, 9),))):
+            _check_logits(_run_cut(cache, runner, ids, cuts, also), want, floor, dtype, f"base-class parts, cuts {cuts[:3]}")
+    finally:
+        unregister_part("norm", "test-centred")
+        unregister_part("embed", "test-scaled-table")
+        unregister_part("test-family", "thing")

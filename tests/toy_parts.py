@@ -141,3 +141,90 @@ def toy_recipe(c: ToyConfig) -> ModelSpec:
     return ModelSpec(hidden=c.width, vocab=c.tokens, layers=(layer,) * c.depth, order=in_order(c.depth),
                      embed=PartRef("embed", "table"), norm=norm, head=PartRef("head", "linear", tied=True),
                      rules=(WeightRule("toy.{rest}", "{rest}"),))
+
+
+# -- a toy mixer that brings a kernel of its own ---------------------------------------------------------------------
+DECAY_SCAN_SOURCE = __import__("pathlib").Path(__file__).resolve().parent / "kernels" / "decay_scan.hip"
+
+
+def decay_scan_plain(x, state, slots, starts, query_start, n_rows, decay):
+    """y[t] = s_t, s_t = decay * s_(t-1) + x[t] along each row's tokens; `state[slot]` (float32) holds a row's s between
+    steps and is updated in place; a row that starts at position 0 starts from zero."""
+    y = torch.empty_like(x)
+    qs, slot_of, start_of = query_start.tolist(), slots.tolist(), starts.tolist()
+    for b in range(n_rows):
+        s = torch.zeros_like(state[slot_of[b]]) if start_of[b] == 0 else state[slot_of[b]].clone()
+        for t in range(qs[b], qs[b + 1]):
+            s = decay * s + x[t].float()
+            y[t] = s.to(x.dtype)
+        state[slot_of[b]] = s
+    return y
+
+
+def _decay_scan_hip(launch, x, state, slots, starts, query_start, n_rows, decay):
+    if not (x.is_cuda and x.is_contiguous() and state.dtype == torch.float32 and state.shape[1] == x.shape[1]):
+        raise ValueError("decay_scan: contiguous rows on the GPU and float32 state of their width")
+    y = torch.empty_like(x)
+    launch(x.data_ptr(), y.data_ptr(), state.data_ptr(), slots.data_ptr(), starts.data_ptr(), query_start.data_ptr(),
+           n_rows, x.shape[1], float(decay), {torch.float32: 0, torch.bfloat16: 1}[x.dtype])
+    return y
+
+
+def decay_scan_op():
+    """The operation as the toy mixer registers it: plain form, HIP symbol, argument types, and the source it is
+    built from (a file under tests/, compiled into a library of its own)."""
+    import ctypes
+
+    from holon_amd.kernels.registry import KernelOp
+    p, i, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    return KernelOp(name="decay_scan", plain=decay_scan_plain, symbol="toy_decay_scan",
+                    argtypes=[p, p, p, p, p, p, i, i, f, i], call=_decay_scan_hip, source=DECAY_SCAN_SOURCE)
+
+
+class DecayScan(Part):
+    """A toy mixer whose arithmetic is a kernel it registers itself (`decay_scan`): a decaying running sum of the
+    inputs, kept per request in its slot, then a projection. It reads nothing on the host, so steps over it may be
+    replayed from graphs."""
+
+    graph_safe = True
+
+    def __init__(self, build: Build, *, hidden: int, layer: int, decay: float) -> None:
+        super().__init__(build)
+        self.hidden, self.decay = hidden, float(decay)
+        self.attach("proj", Linear(build, inp=hidden, out=hidden))
+
+    def state(self):
+        return [SlotState("s", (self.hidden,), torch.float32)]
+
+    def forward(self, x, step, site):
+        y = self.kernels.decay_scan(x, site.slot_state["s"], step.slots, step.starts, step.query_start, step.n_rows,
+                                    self.decay)
+        return self.proj(y)
+
+    __call__ = forward
+
+
+@dataclasses.dataclass(frozen=True)
+class ToyScanConfig:
+    width: int
+    tokens: int
+    depth: int
+    decay: float
+    eps: float
+    eos_token_ids: tuple[int, ...] = ()
+
+    @classmethod
+    def from_dict(cls, c, generation=None) -> "ToyScanConfig":
+        return cls(width=c["width"], tokens=c["tokens"], depth=c["depth"], decay=c["decay"], eps=c["eps"])
+
+    def to_dict(self) -> dict:
+        return {"architectures": ["ToyScanModel"], **{k: getattr(self, k) for k in ("width", "tokens", "depth", "decay", "eps")}}
+
+
+def toy_scan_recipe(c: ToyScanConfig) -> ModelSpec:
+    norm = PartRef("norm", "rmsnorm", eps=c.eps)
+    layer = LayerSpec(block=PartRef("block", "prenorm"), mixer=PartRef("mixer", "test-decay-scan", decay=c.decay),
+                      ffn=PartRef("ffn", "swiglu", inter=2 * c.width), norm=norm)
+    return ModelSpec(hidden=c.width, vocab=c.tokens, layers=(layer,) * c.depth, order=in_order(c.depth),
+                     embed=PartRef("embed", "table"), norm=norm, head=PartRef("head", "linear", tied=True),
+                     rules=(WeightRule("toy.{rest}", "{rest}"),))
