@@ -12,25 +12,26 @@ from typing import Any
 DTYPES = ("bfloat16", "float32")
 
 
-def _setting(default: object, help: str) -> Any:
-    return dataclasses.field(default=default, metadata={"help": help})
+def _setting(default: object, text: str) -> Any:
+    """A field with the line the command line shows for it."""
+    return dataclasses.field(default=default, metadata={"help": text})
 
 
 @dataclasses.dataclass
 class EngineConfig:
     model: str = dataclasses.field(metadata={"help": "model folder (config.json and *.safetensors)"})
-    device: str = _setting("cuda", "torch device to serve on")
+    device: str = _setting("cuda", "the GPU the engine runs on, as torch names it")
     dtype: str = _setting("bfloat16", "activation, weight and cache dtype: bfloat16, or float32 (every product, sum "
                                       "and stored value in true 32-bit)")
-    page_size: int = _setting(16, "tokens per page of paged state")
-    max_seqs: int = _setting(64, "sequences served at once")
-    max_model_len: int = _setting(8192, "prompt + generated tokens per request; pools always hold one")
-    max_step_tokens: int = _setting(4096, "tokens one step computes at most")
-    chunk_with_decode: int = _setting(0, "prefill tokens a step with decode rows may also carry (0: none)")
-    memory_fraction: float = _setting(0.9, "of the memory left after weights, for activations and state")
-    state_memory: int | None = _setting(None, "bytes for state pools; default: from memory_fraction")
+    page_size: int = _setting(16, "how many tokens one cache page holds")
+    max_seqs: int = _setting(64, "the most requests that run side by side (slots)")
+    max_model_len: int = _setting(8192, "the longest a request may grow, prompt and generated tokens together; the cache is never smaller than one such request")
+    max_step_tokens: int = _setting(4096, "the token budget of one step (prompt portions and decode rows together)")
+    chunk_with_decode: int = _setting(0, "how many prompt tokens may ride along in a step that also decodes (0: such steps decode only)")
+    memory_fraction: float = _setting(0.9, "the share of the GPU memory still free once the weights are loaded that steps and the cache may use")
+    state_memory: int | None = _setting(None, "the cache's size in bytes, instead of deriving it from memory_fraction")
     cache_tokens: int | None = _setting(None, "tokens of paged state per pool (overrides state_memory)")
-    prefix_cache: bool = _setting(True, "reuse cached prompt blocks across requests")
+    prefix_cache: bool = _setting(True, "let a request start from the pages of an earlier request with the same first tokens")
     overlap: bool = _setting(True, "schedule and launch the next step while the last one runs")
     graphs: bool = _setting(True, "replay decode steps from HIP graphs, per batch-size bucket")
     decode_weight_copy: bool = _setting(True, "keep a second copy of every projection in the tile layout that steps of "
@@ -43,11 +44,12 @@ class EngineConfig:
                                                "separated list)")
 
     def __post_init__(self) -> None:
-        for name in ("page_size", "max_seqs", "max_model_len", "max_step_tokens"):
-            if getattr(self, name) < 1:
-                raise ValueError(f"EngineConfig.{name} must be >= 1")
-        if self.chunk_with_decode < 0:
-            raise ValueError("EngineConfig.chunk_with_decode must be >= 0")
+        too_small = [name for name, least in (("page_size", 1), ("max_seqs", 1), ("max_model_len", 1),
+                                              ("max_step_tokens", 1), ("chunk_with_decode", 0))
+                     if getattr(self, name) < least]
+        if too_small:
+            raise ValueError(f"EngineConfig: {', '.join(too_small)} below the least value allowed (0 for "
+                             "chunk_with_decode, 1 for the others)")
         if self.dtype not in DTYPES:
             raise ValueError(f"EngineConfig.dtype must be one of {DTYPES}, got {self.dtype!r}")
         if self.chunk_with_decode and self.max_step_tokens < self.max_seqs + self.chunk_with_decode:

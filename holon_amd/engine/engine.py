@@ -174,7 +174,7 @@ class Engine:
         if rid is None:
             rid = str(next(self._ids))
         if rid in self._live:
-            raise ValueError(f"request id {rid!r} is already in flight")
+            raise ValueError(f"there is a live request with the id {rid!r} already")
         seed = secrets.randbits(63) if params.seed is None else params.seed
         seqs = [Seq(rid=rid, tokens=list(token_ids), index=i,
                     params=dataclasses.replace(params, seed=sequence_seed(seed, i),
@@ -247,7 +247,7 @@ class Engine:
     def generate(self, prompts: list[list[int]], params: SamplingParams | None = None) -> list[list[int]]:
         """Run the prompts to their end; the generated token ids of each, in the prompts' order."""
         if params is not None and params.n != 1:
-            raise ValueError("generate() returns one sequence per prompt; step() streams n > 1")
+            raise ValueError("generate() gives back one list of tokens a prompt: for n > 1 add the prompts and read step()'s deltas")
         streams: dict[str, list[int]] = {self.add(p, params): [] for p in prompts}
         unfinished = len(streams)
         while unfinished:
@@ -276,7 +276,7 @@ class Engine:
             rows = self.sched.schedule()
         if rows is None:
             if self.has_work():
-                raise RuntimeError("the scheduler made no progress with requests pending")
+                raise RuntimeError("requests are waiting but the scheduler found nothing to run")
             return deltas
         launched = self._launch(rows)
         deltas += self.drain()
