@@ -106,6 +106,8 @@ def main(argv: list[str] | None = None) -> int:
                     help="fewer layers than the configuration has (recorded in config)")
     ap.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip the further decode and prefill points")
+    ap.add_argument("--context", type=int, default=CONTEXT, help="the context the timed decode steps end at")
+    ap.add_argument("--prompt", type=int, default=PROMPT, help="tokens of the timed prompt")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--workload", choices=("decode", "mixed", "long"), default="decode")
     ap.add_argument("--products", choices=("own", "vendor", "timed"), default="timed",
@@ -130,11 +132,12 @@ def main(argv: list[str] | None = None) -> int:
         kernel_build.build()
     cfg_json = dict(QWEN3_8B, num_hidden_layers=a.layers)
     max_batch = max(a.batch, 1 if a.no_points else max(POINT_BATCHES))
-    longest = CONTEXT if a.no_points else max(LONG_CONTEXT, max(POINT_PROMPTS))
+    longest = max(a.context, a.prompt, 0 if a.no_points else max(LONG_CONTEXT, max(POINT_PROMPTS)))
     engine = Engine.from_random(cfg_json, seed=0, cfg=EngineConfig(
         model="random:qwen3-8b", device="cuda:0", dtype=a.dtype, page_size=16, max_seqs=max_batch,
         max_model_len=longest + 16, max_step_tokens=4096,
-        cache_tokens=max(max_batch * (CONTEXT + 16), 0 if a.no_points else 8 * (LONG_CONTEXT + 16)),
+        cache_tokens=max(max_batch * (CONTEXT + 16), a.batch * (a.context + 16), a.prompt + 16,
+                         0 if a.no_points else 8 * (LONG_CONTEXT + 16)),
         graphs=not a.no_graphs, products=a.products))
     spec, c = engine.spec, cfg_json
     item = 2 if a.dtype == "bfloat16" else 4
@@ -193,9 +196,9 @@ def main(argv: list[str] | None = None) -> int:
         """Products of every layer over `tokens` rows, causal attention (half of the square), the head on one row."""
         return layers * (2 * tokens * layer_params + 2 * hq * d * tokens * tokens) + 2 * h * v
 
-    pre_ms, ttft_ms = prefill(PROMPT)
-    pre_flops = prompt_flops(PROMPT)
-    ms, ctx, tpot_ms, decode_prompt = decode(a.batch, a.steps, a.warmup)
+    pre_ms, ttft_ms = prefill(a.prompt)
+    pre_flops = prompt_flops(a.prompt)
+    ms, ctx, tpot_ms, decode_prompt = decode(a.batch, a.steps, a.warmup, a.context)
     step_bytes = weight_bytes + a.batch * ctx * kv_token_bytes
     achieved = step_bytes / (ms * 1e-3) / 1e9
     points = {}
@@ -218,24 +221,24 @@ def main(argv: list[str] | None = None) -> int:
             points[f"prefill_{tokens}_tflop"] = round(prompt_flops(tokens) / 1e12, 2)
             points[f"prefill_{tokens}_frac"] = round(prompt_flops(tokens) / (best * 1e-3) / PEAK_FLOPS[a.dtype], 4)
     line = {
-        "metric": f"decode tok/s at batch {a.batch} (context 4,096), Qwen3-8B shape", "value": round(a.batch / (ms * 1e-3), 1),
+        "metric": f"decode tok/s at batch {a.batch} (context {a.context:,}), Qwen3-8B shape", "value": round(a.batch / (ms * 1e-3), 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
         "data": "synthetic (random weights, uniform random token ids)",
         "config": {"model": "Qwen3-8B shape", "layers": layers, "layers_of_config": QWEN3_8B["num_hidden_layers"],
                    "hidden": h, "heads": hq, "kv_heads": hkv, "head_dim": d, "intermediate": inter, "vocab": v,
-                   "tied": False, "global_batch": a.batch, "seq_len": CONTEXT, "prefill_tokens": PROMPT,
+                   "tied": False, "global_batch": a.batch, "seq_len": a.context, "prefill_tokens": a.prompt,
                    "decode_prompt_len": decode_prompt, "page_size": 16,
                    "parallelism": "single GPU", "graphs": not a.no_graphs, "mean_context": round(ctx, 1),
                    "products": a.products},
-        "prefill": {"value": round(PROMPT / (pre_ms * 1e-3), 1), "tokens": PROMPT, "ms": round(pre_ms, 3),
+        "prefill": {"value": round(a.prompt / (pre_ms * 1e-3), 1), "tokens": a.prompt, "ms": round(pre_ms, 3),
                     "ms_is": "best of 3 prompts", "ms_median": round(ttft_ms, 3),
                     "frac": round(pre_flops / (pre_ms * 1e-3) / PEAK_FLOPS[a.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},
         "points": points,
         "products": engine.products(),
-        "latency": {"ttft_ms_p50": round(ttft_ms, 3), "ttft_tokens": PROMPT, "tpot_ms_p50": round(tpot_ms, 4),
+        "latency": {"ttft_ms_p50": round(ttft_ms, 3), "ttft_tokens": a.prompt, "tpot_ms_p50": round(tpot_ms, 4),
                     "tpot_batch": a.batch},
     }
     if engine.stats()["prefix_tokens_saved"]:

@@ -781,6 +781,295 @@ __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kerne
   }
 }
 
+#ifndef PAIR_VALU_PER_MFMA
+#define PAIR_VALU_PER_MFMA 16   // vector instructions the scheduler is asked to put between two matrix products
+#endif
+// The same with two tiles of 32 rows a wave (a block: 256 rows, 64 positions of a group of four heads). A stage's
+// keys and values are read from the cache into LDS once for twice the rows (the staged kernels are bound by what the
+// blocks of a launch read through L2: every block reads every key before its rows), a wave reads them from LDS once
+// for both tiles, and the two tiles are independent work in one instruction stream: one tile's exponentials are issued
+// between the other tile's matrix products. Stages that both tiles see whole run without masks (`MASK` false); the
+// stages at the diagonal, with a window, and the last one run the masked form.
+template <bool MASK>
+__device__ __forceinline__ void scores_to_probs(const f32x16_t& sc, int kb, int h, int qpos, int first,
+                                                float scale_log2, float m, float& m_new, float& psum, bf16x8_t& pb0,
+                                                bf16x8_t& pb1) {
+  float sv[16];
+#pragma unroll
+  for (int idx = 0; idx < 16; ++idx) sv[idx] = sc[idx];
+  if constexpr (MASK) {
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) {
+      const int i = idx / 4, r = idx % 4;
+      const int key = kb + 16 * (i / 2) + 8 * h + 4 * (i % 2) + r;
+      if (!(key <= qpos && key >= first)) sv[idx] = -INFINITY;
+    }
+  }
+  float mx = fmaxf(fmaxf(sv[0], sv[1]), sv[2]);
+#pragma unroll
+  for (int idx = 3; idx + 1 < 16; idx += 2) mx = fmaxf(fmaxf(mx, sv[idx]), sv[idx + 1]);
+  mx = fmaxf(mx, sv[15]);
+  {                                          // the other half of the keys is in lane l ^ 32
+    const auto halves = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+    mx = fmaxf(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
+  }
+  m_new = fmaxf(m, mx * scale_log2);
+  const float m_use = m_new == -INFINITY ? 0.f : m_new;
+  psum = 0.f;
+#pragma unroll
+  for (int idx = 0; idx < 16; ++idx) {
+    const float p = __builtin_amdgcn_exp2f(fmaf(sv[idx], scale_log2, -m_use));
+    psum += p;
+    if (idx < 8) pb0[idx] = (__bf16)p; else pb1[idx - 8] = (__bf16)p;
+  }
+}
+
+template <int D>
+__global__ void __launch_bounds__(256, 1) attn_prefill_pair_kernel(AttnArgs a) {
+  constexpr int KP = D + 8;    // pitch of a key row in LDS (elements)
+  constexpr int VP = 40;       // pitch of a value row: 32 keys + 8
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][32 * KP];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][D * VP];
+  constexpr int PG = 4096;
+  __shared__ int32_t pg_lds[PG];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, tid = threadIdx.x;
+  const int h = lane / 32, c = lane % 32;
+  const int b = a.row_ids[a.unpaired ? blockIdx.z / 2 : blockIdx.z];
+  const int group = a.heads / a.kv_heads;      // <= 32 (the host checks)
+  const TileMap32 tm = tile_map32(group);
+  const int hk = blockIdx.y;
+  const int qs = a.qstart[b], nq = a.qstart[b + 1] - qs, n = a.lens[b];
+  const int n_tiles = (nq + tm.pos_per_tile - 1) / tm.pos_per_tile;
+  constexpr int TPB = 8;                       // tiles a block owns per range: two a wave, side by side
+  const int n_ranges = (n_tiles + TPB - 1) / TPB;
+  if (n <= 0 || (int)blockIdx.x >= (n_ranges + 1) / 2) return;   // uniform over the block
+  const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
+  const int P = a.page_size;
+  const int64_t plane = (int64_t)P * D;
+  const int64_t page_stride = 2 * (int64_t)a.kv_heads * plane;
+  const bf16_t* kbase = a.pages + (int64_t)hk * plane;
+  const bf16_t* vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
+  const int max_page = min(a.table_stride, PG) - 1;
+  for (int i = tid; i < min(PG, a.table_stride); i += 256) pg_lds[i] = trow[i];
+  constexpr int KCH = D / 8;
+  constexpr int ROUNDS = D / 64;
+  static_assert(D == 64 || D == 128, "the LDS kernels copy one or two chunks of each kind per thread");
+  constexpr bool HALVES = ROUNDS == 2;         // (what a thread copies per stage: as in attn_prefill_wide_kernel)
+  int k_half[ROUNDS], k_off[ROUNDS], k_dst[ROUNDS], v_half[ROUNDS], v_off[ROUNDS], v_dst[ROUNDS];
+#pragma unroll
+  for (int i = 0; i < ROUNDS; ++i) {
+    const int q = tid + 256 * i;
+    const int j = q / KCH, col = (q % KCH) * 8;
+    const int row = 8 * (2 * (j / 16) + (j % 8) / 4) + 4 * ((j % 16) / 8) + j % 4;
+    k_half[i] = j / 16;
+    k_off[i] = (j % 16) * D + col;
+    k_dst[i] = row * KP + col;
+    const int vd = HALVES ? tid / 2 : tid / 4, vkc = HALVES ? 2 * i + tid % 2 : tid % 4;
+    v_half[i] = vkc / 2;
+    v_off[i] = vd * P + 8 * (vkc % 2);
+    v_dst[i] = vd * VP + vkc * 8;
+  }
+  const int pi = c / tm.rows_per_pos, hi = c % tm.rows_per_pos;
+
+  const int pass_lo = a.unpaired ? 1 - (int)(blockIdx.z % 2) : 0, pass_hi = a.unpaired ? pass_lo + 1 : 2;
+  for (int pass = pass_lo; pass < pass_hi; ++pass) {
+    const int range = pass == 0 ? (int)blockIdx.x : n_ranges - 1 - (int)blockIdx.x;
+    if (pass == 1 && range <= (int)blockIdx.x) break;
+    const int p_lo = range * TPB * tm.pos_per_tile;
+    const int p_hi = min(nq, p_lo + TPB * tm.pos_per_tile) - 1;
+    const int key_hi = n - nq + p_hi;                          // over the whole block (all waves walk the same stages)
+    const int key_lo = a.window > 0 ? max(0, n - nq + p_lo - a.window + 1) : 0;
+    bool valid[2];
+    int token[2], qpos[2], tile_last[2], tile_first[2];
+    const int head = hk * group + hi;
+    bf16x8_t qf[2][D / 16];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int p0 = (range * TPB + wave * 2 + t) * tm.pos_per_tile;
+      const int qi = p0 + pi;
+      valid[t] = pi < tm.pos_per_tile && qi < nq && hi < group;
+      token[t] = qs + qi;
+      qpos[t] = valid[t] ? n - nq + qi : -1;
+      tile_last[t] = p0 < nq ? n - nq + min(nq, p0 + tm.pos_per_tile) - 1 : -1;
+      tile_first[t] = n - nq + p0;
+      const bf16_t* qp = a.q + ((int64_t)token[t] * a.heads + head) * D + 8 * h;
+#pragma unroll
+      for (int ds = 0; ds < D / 16; ++ds) {
+        if (valid[t]) {
+          qf[t][ds] = load8(qp + ds * 16);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) qf[t][ds][i] = (__bf16)0.f;
+        }
+      }
+    }
+    f32x16_t o[2][D / 32];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[t][db][i] = 0.f;
+    float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+
+    struct Regs { bf16x8_t k[ROUNDS], v[ROUNDS]; };
+    Regs r0, r1;
+    const int kb_last = (key_hi / 32) * 32;
+    auto fetch = [&](int kb_want, Regs& r) {
+      const int kb = min(kb_want, kb_last);
+      const int i0 = min(kb / P, max_page), i1 = min((kb + 16) / P, max_page);
+      const int64_t pg0 = (int64_t)__builtin_amdgcn_readfirstlane(pg_lds[i0]) * page_stride;
+      const int64_t pg1 = (int64_t)__builtin_amdgcn_readfirstlane(pg_lds[i1]) * page_stride;
+      const int off0 = kb % P, off1 = (kb + 16) % P;
+      const bf16_t* kh[2] = {kbase + pg0 + (int64_t)off0 * D, kbase + pg1 + (int64_t)off1 * D};
+      const bf16_t* vh[2] = {vbase + pg0 + off0, vbase + pg1 + off1};
+#pragma unroll
+      for (int i = 0; i < ROUNDS; ++i) {
+        if constexpr (HALVES) {
+          r.k[i] = load8(kh[i] + (uint32_t)k_off[i]);
+          r.v[i] = load8(vh[i] + (uint32_t)v_off[i]);
+        } else {
+          r.k[i] = load8((k_half[i] ? kh[1] : kh[0]) + (uint32_t)k_off[i]);
+          r.v[i] = load8((v_half[i] ? vh[1] : vh[0]) + (uint32_t)v_off[i]);
+        }
+      }
+    };
+    auto stash = [&](int buf, const Regs& r) {
+#pragma unroll
+      for (int i = 0; i < ROUNDS; ++i) {
+        *reinterpret_cast<bf16x8_t*>(&k_lds[buf][k_dst[i]]) = r.k[i];
+        *reinterpret_cast<bf16x8_t*>(&v_lds[buf][v_dst[i]]) = r.v[i];
+      }
+    };
+    // what follows a tile's probabilities: the rescale of its sums when some row's max moved, then its sum
+    auto settle = [&](int t, float m_new, float psum) {
+      if (__any(m_new != m[t])) {
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m[t] - m_use);
+        l[t] *= alpha;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db) o[t][db] *= alpha;
+        m[t] = m_new;
+      }
+      l[t] += psum;
+    };
+    // One stage. `masked`: some row of the wave's tiles does not see the whole stage (the diagonal, a window);
+    // `last`: the stage holds the row's last key and may reach past it; nothing is staged behind it.
+    auto stage = [&](auto masked, auto last, int kb, int buf, Regs& next) {
+      constexpr bool MASK = decltype(masked)::value, LAST = decltype(last)::value;
+      const bool on0 = !MASK || kb <= tile_last[0], on1 = !MASK || kb <= tile_last[1];   // (uniform over the wave)
+      if (on0 || on1) {
+        bf16x8_t kf[D / 16];
+#pragma unroll
+        for (int ds = 0; ds < D / 16; ++ds)
+          kf[ds] = *reinterpret_cast<const bf16x8_t*>(&k_lds[buf][c * KP + ds * 16 + 8 * h]);
+        f32x16_t sc0, sc1;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { sc0[i] = 0.f; sc1[i] = 0.f; }
+#pragma unroll
+        for (int ds = 0; ds < D / 16; ++ds) sc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds], qf[0][ds], sc0, 0, 0, 0);
+#pragma unroll
+        for (int ds = 0; ds < D / 16; ++ds) sc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds], qf[1][ds], sc1, 0, 0, 0);
+        bf16x8_t vf[D / 32][2];
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db) {
+          vf[db][0] = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(db * 32 + c) * VP + 8 * h]);
+          vf[db][1] = *reinterpret_cast<const bf16x8_t*>(&v_lds[buf][(db * 32 + c) * VP + 16 + 8 * h]);
+          if constexpr (LAST) {
+            zero_after(vf[db][0], kb + 8 * h, key_hi);
+            zero_after(vf[db][1], kb + 16 + 8 * h, key_hi);
+          }
+        }
+        float m_new, psum;
+        bf16x8_t pb0, pb1;
+        if (on0) {
+          scores_to_probs<MASK>(sc0, kb, h, qpos[0], a.window > 0 ? qpos[0] - a.window + 1 : 0, a.scale_log2, m[0],
+                                m_new, psum, pb0, pb1);
+          if constexpr (!MASK) {     // the second tile's score products, one at a time between the first tile's exponentials
+            __builtin_amdgcn_sched_group_barrier(0x008, D / 16, 0);
+#pragma unroll
+            for (int i = 0; i < D / 16; ++i) {
+              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+              __builtin_amdgcn_sched_group_barrier(0x002, PAIR_VALU_PER_MFMA, 0);
+            }
+          }
+          settle(0, m_new, psum);
+#pragma unroll
+          for (int db = 0; db < D / 32; ++db) {
+            o[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][0], pb0, o[0][db], 0, 0, 0);
+            o[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][1], pb1, o[0][db], 0, 0, 0);
+          }
+        }
+        if (on1) {
+          scores_to_probs<MASK>(sc1, kb, h, qpos[1], a.window > 0 ? qpos[1] - a.window + 1 : 0, a.scale_log2, m[1],
+                                m_new, psum, pb0, pb1);
+          if constexpr (!MASK) {     // the first tile's value products between the second tile's exponentials
+#pragma unroll
+            for (int i = 0; i < D / 16; ++i) {
+              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+              __builtin_amdgcn_sched_group_barrier(0x002, PAIR_VALU_PER_MFMA, 0);
+            }
+          }
+          settle(1, m_new, psum);
+#pragma unroll
+          for (int db = 0; db < D / 32; ++db) {
+            o[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][0], pb0, o[1][db], 0, 0, 0);
+            o[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][1], pb1, o[1][db], 0, 0, 0);
+          }
+        }
+      }
+      if constexpr (!LAST) {
+        stash(buf ^ 1, next);
+        fetch(kb + 96, next);
+        lds_barrier();
+      }
+    };
+    // a stage is unmasked when every row of both tiles sees all of it: it ends at or before the first tile's first
+    // position, and there is no window
+    auto step = [&](auto last, int kb, int buf, Regs& next) {
+      if (a.window <= 0 && kb + 31 <= tile_first[0]) stage(std::false_type{}, last, kb, buf, next);
+      else stage(std::true_type{}, last, kb, buf, next);
+    };
+    const int kb_first = (key_lo / 32) * 32;
+    lds_barrier();               // the previous pass has finished reading both buffers
+    fetch(kb_first, r0);
+    fetch(kb_first + 32, r1);
+    stash(0, r0);
+    fetch(kb_first + 64, r0);
+    lds_barrier();
+    int kb = kb_first;
+    for (; kb + 32 < kb_last; kb += 64) {        // pairs of stages that both lie before the last one
+      step(std::false_type{}, kb, 0, r1);
+      step(std::false_type{}, kb + 32, 1, r0);
+    }
+    if (kb < kb_last) {
+      step(std::false_type{}, kb, 0, r1);
+      stage(std::true_type{}, std::true_type{}, kb + 32, 1, r0);
+    } else {
+      stage(std::true_type{}, std::true_type{}, kb, 0, r1);
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const float lt = l[t] + __shfl_xor(l[t], 32, WAVE);
+      if (valid[t]) {
+        const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+        bf16_t* op = a.out + ((int64_t)token[t] * a.heads + head) * D + 4 * h;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            ushort4 w;
+            w.x = float_to_bf16(o[t][db][4 * i + 0] * inv);
+            w.y = float_to_bf16(o[t][db][4 * i + 1] * inv);
+            w.z = float_to_bf16(o[t][db][4 * i + 2] * inv);
+            w.w = float_to_bf16(o[t][db][4 * i + 3] * inv);
+            *reinterpret_cast<ushort4*>(op + db * 32 + 8 * i) = w;
+          }
+      }
+    }
+  }
+}
+
 // What the decode kernel needs to take the step's raw q/k/v projection itself (`qkv` [T, (Hq + 2 Hkv) D]) instead of
 // queries that another kernel has normed and rotated and keys that it has stored: per-head RMSNorm weights (both or
 // neither), the rotation table (cos | sin of every position, over the whole head, or none), where each token's key
@@ -1113,6 +1402,26 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict
   }
 }
 
+#ifndef PAIR_VALU_PER_MFMA
+#define PAIR_VALU_PER_MFMA 16
+#endif
+#ifndef PAIR_UNPAIR_BELOW
+#define PAIR_UNPAIR_BELOW 512
+#endif
+// Long prompt portions of groups of up to 32 heads: two tiles of 32 rows a wave from PAIR_FROM_KEYS keys on (measured,
+// 32 heads over 8 kv heads of 128, portions of 4,096 tokens, us a layer, one tile against two: behind 4,096 tokens 616
+// and 636, behind 12,288 tokens 1,366 and 1,279, behind 28,672 tokens 2,625 and 2,441; whole prompts of 2,048 and
+// 4,096 tokens 78 and 101, 208 and 298: short rows have too few blocks of 256 rows to fill the GPU).
+// holon_attention_prefill_form: 0 never, 1 by that rule, 2 always (tests run both forms at the same sizes); returns
+// what was set before; a negative argument only asks.
+constexpr int PAIR_FROM_KEYS = 12288;
+static int g_prefill_pair = 1;
+extern "C" int holon_attention_prefill_form(int form) {
+  const int was = g_prefill_pair;
+  if (form >= 0 && form <= 2) g_prefill_pair = form;
+  return was;
+}
+
 static bool mfma_serves(int head_dim, int page_size) {
   return (head_dim == 64 || head_dim == 128 || head_dim == 256) && page_size % 16 == 0;
 }
@@ -1148,7 +1457,14 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
     hipStream_t ls = (hipStream_t)stream;
     const TileMap32 tm32 = tile_map32(heads / kv_heads);
     const int ranges32 = ((max_query + tm32.pos_per_tile - 1) / tm32.pos_per_tile + 3) / 4;
-    if (heads / kv_heads <= 32) {   // tiles of 32 rows (measured faster at every length: 2,048 tokens 89 against 95 us,
+    const int ranges_pair = ((max_query + tm32.pos_per_tile - 1) / tm32.pos_per_tile + 7) / 8;
+    if (heads / kv_heads <= 32 && (g_prefill_pair == 2 || (g_prefill_pair == 1 && max_len >= PAIR_FROM_KEYS))) {
+      // two tiles of 32 rows a wave
+      a.unpaired = (int64_t)((ranges_pair + 1) / 2) * kv_heads * n_rows < PAIR_UNPAIR_BELOW ? 1 : 0;
+      dim3 lgrid((ranges_pair + 1) / 2, kv_heads, a.unpaired ? 2 * n_rows : n_rows);
+      if (head_dim == 64) attn_prefill_pair_kernel<64><<<lgrid, 256, 0, ls>>>(a);
+      else attn_prefill_pair_kernel<128><<<lgrid, 256, 0, ls>>>(a);
+    } else if (heads / kv_heads <= 32) {   // tiles of 32 rows (measured faster at every length: 2,048 tokens 89 against 95 us,
                                     // 32,768 tokens 11.1 against 13.3 ms); larger groups keep tiles of 16
       // fewer than two paired blocks a compute unit: the ranges of a pair as blocks of their own, so that a second
       // wave on every SIMD hides the first one's waits

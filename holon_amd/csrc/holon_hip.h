@@ -45,6 +45,9 @@ int holon_attention_prefill_bf16(const void* q, void* out, const void* pages, co
                                  const int32_t* slots, const int32_t* lens, const int32_t* query_start,
                                  const int32_t* row_ids, int n_rows, int max_query, int max_len, int heads,
                                  int kv_heads, int head_dim, int page_size, float scale, int window, void* stream);
+// Which kernel long prompt portions of groups of up to 32 heads take: 0 one tile of 32 rows a wave, 2 two tiles a wave,
+// 1 (the default) two from 12,288 keys on. Returns the setting before; a negative argument changes nothing.
+int holon_attention_prefill_form(int form);
 // One query token per row; the keys are split over `splits` waves of `keys_per_split` keys (a multiple of 32) whose
 // partial results (part_o [n_rows, heads, splits, head_dim], part_ml [n_rows, heads, splits, 2], float32) are merged
 // in split order.

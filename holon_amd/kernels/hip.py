@@ -70,6 +70,7 @@ class HipKernels:
                                              _P],
             "holon_attention_decode_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P,
                                             _I, _I, _P],
+            "holon_attention_prefill_form": [_I],
             "holon_attention_decode_waves_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
                                                   _P, _P, _I, _I, _I, _I, _P],
             "holon_attention_decode_fused_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
@@ -156,7 +157,7 @@ class HipKernels:
 
     @staticmethod
     def _stream() -> int:
-        return torch.cuda.current_stream().cuda_stream
+        return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
 
     @staticmethod
     def _check(t: torch.Tensor, what: str, dtype: torch.dtype | None = None) -> None:

@@ -3,6 +3,8 @@
     python -m holon_amd.trace_summary DB                 every kernel of the run, summed by name
     python -m holon_amd.trace_summary DB --step decode   one decode step (the one before the last embedding kernel)
     python -m holon_amd.trace_summary DB --step prefill  the third step of the run (bench.py's last timed prompt step)
+    ... --classes                                        after the kernels, the step's time by class of kernel:
+                                                         attention, matrix products, elementwise, sampling, other
 
 A step is what lies between two embedding kernels: every step of the engine starts with one. The database is the
 `*_results.db` file that rocprofv3 writes (SQLite: `rocpd_kernel_dispatch` joined with `rocpd_info_kernel_symbol`).
@@ -41,6 +43,33 @@ def dispatches(path: str) -> list[tuple]:
     return [(n, st, en, gx // max(wx, 1), gy, gz) for n, st, en, gx, gy, gz, wx in rows]
 
 
+CLASSES = (("attention", ("attn_",)), ("matrix products", ("gemm_", "Cijk_", "Custom_Cijk_", "hipBLASLt")),
+           ("elementwise", ("rmsnorm", "silu_mul", "qk_norm_rope", "v_write", "kv_write", "embedding", "sum_parts",
+                            "row_sumsq", "scatter_rows")),
+           ("sampling", ("argmax", "sample_kernel", "store_tokens", "logprobs")))
+
+
+def kernel_class(name: str) -> str:
+    for label, marks in CLASSES:
+        if any(mark in name for mark in marks):
+            return label
+    return "other (copies, library elementwise)"
+
+
+def by_class(rows: list[tuple]) -> str:
+    """The step's kernel time by class of kernel, as a share of the time from its first start to its last end (what
+    no kernel covers is the gaps between kernels)."""
+    span = (rows[-1][2] - rows[0][1]) / 1e3
+    took: dict[str, float] = collections.OrderedDict()
+    for name, st, en, *_ in rows:
+        took[kernel_class(name)] = took.get(kernel_class(name), 0.0) + (en - st) / 1e3
+    out = [f"{'us':>10} {'of step':>8}  class"]
+    for label, us in sorted(took.items(), key=lambda kv: -kv[1]):
+        out.append(f"{us:10.1f} {100 * us / span:7.1f}%  {label}")
+    out.append(f"{span - sum(took.values()):10.1f} {100 * (span - sum(took.values())) / span:7.1f}%  between kernels")
+    return "\n".join(out)
+
+
 def summarise(rows: list[tuple], title: str, top: int, with_grid: bool) -> str:
     agg: dict[str, list] = collections.OrderedDict()
     total = 0.0
@@ -64,6 +93,7 @@ def main(argv=None) -> int:
     ap.add_argument("--step", choices=("decode", "prefill"), help="one step instead of the whole run")
     ap.add_argument("--index", type=int, default=2, help="which step of the run --step prefill takes (default: the third)")
     ap.add_argument("--top", type=int, default=16)
+    ap.add_argument("--classes", action="store_true", help="also the time by class of kernel")
     args = ap.parse_args(argv)
     rows = dispatches(args.db)
     if not rows:
@@ -74,14 +104,18 @@ def main(argv=None) -> int:
         if len(starts) < 3:
             print("fewer than three steps in this trace")
             return 1
-        print(summarise(rows[starts[-3]:starts[-2]], "one decode step", args.top, True))
+        rows = rows[starts[-3]:starts[-2]]
+        print(summarise(rows, "one decode step", args.top, True))
     elif args.step == "prefill":
         if len(starts) < args.index + 2:
             print(f"fewer than {args.index + 2} steps in this trace")
             return 1
-        print(summarise(rows[starts[args.index]:starts[args.index + 1]], "one prompt step", args.top, True))
+        rows = rows[starts[args.index]:starts[args.index + 1]]
+        print(summarise(rows, "one prompt step", args.top, True))
     else:
         print(summarise(rows, "whole run", args.top, False))
+    if args.classes:
+        print(by_class(rows))
     return 0
 
 

@@ -278,8 +278,8 @@ def test_decode_attention_from_the_raw_projection(hip, geometry, norm, rope):
 @pytest.mark.parametrize("geometry", [(32, 8, 128), (16, 8, 64), (8, 1, 128), (7, 7, 64), (6, 2, 64), (5, 1, 128),
                                       (24, 1, 64), (32, 1, 128), (40, 1, 128), (66, 1, 64), (80, 2, 64)])
 def test_long_prompt_portions_two_tiles_a_wave(hip, geometry):
-    """Portions long enough for the kernels that stage keys and values through LDS (tiles of 32 rows for groups of up
-    to 32 heads, tiles of 16 rows, one or two a wave, for larger groups): one row of 4,500 tokens from position 0, two
+    """Portions long enough for the kernels that stage keys and values through LDS (tiles of 32 rows, one or two a
+    wave, for groups of up to 32 heads; tiles of 16 rows, one or two a wave, for larger groups): one row of 4,500 tokens from position 0, two
     rows continuing earlier tokens (so the keys start before the queries), and a window. Groups of 1, 3, 5, 24, 32
     (tiles that hold one position or several, whole or in part), 40 and 66 heads."""
     heads, kv_heads, head_dim = geometry
@@ -288,17 +288,23 @@ def test_long_prompt_portions_two_tiles_a_wave(hip, geometry):
         q, pages, table, attn = _paged_case(rows, heads, kv_heads, head_dim, 16, bf, seed=len(rows) + window)
         scale = head_dim ** -0.5
         want = PLAIN.paged_attention(q.double(), pages.double(), table, attn, 16, scale, window)
-        got = hip.paged_attention(q, pages, table, attn, 16, scale, window)
-        # rows that see few keys are averages of few values and much larger than rows that see thousands: each
-        # stretch of rows is held to the budget of its own size and of the keys it sees
-        at = 0
-        for start, n in rows:
-            for lo, hi in ((0, 64), (64, 512), (512, n)):
-                part = slice(at + lo, at + min(hi, n))
-                span = head_dim + (min(window, start + hi) if window else start + min(hi, n))
-                assert H.op_budget_usage(got[part], want[part], bf, span) <= 1, (geometry, rows, window, lo)
-            at += n
-        assert torch.equal(got, hip.paged_attention(q, pages, table, attn, 16, scale, window))
+        for form in (0, 2):                      # one tile of 32 rows a wave, and two (groups of up to 32 heads)
+            before = hip.lib.holon_attention_prefill_form(form)
+            try:
+                got = hip.paged_attention(q, pages, table, attn, 16, scale, window)
+                again = hip.paged_attention(q, pages, table, attn, 16, scale, window)
+            finally:
+                hip.lib.holon_attention_prefill_form(before)
+            # rows that see few keys are averages of few values and much larger than rows that see thousands: each
+            # stretch of rows is held to the budget of its own size and of the keys it sees
+            at = 0
+            for start, n in rows:
+                for lo, hi in ((0, 64), (64, 512), (512, n)):
+                    part = slice(at + lo, at + min(hi, n))
+                    span = head_dim + (min(window, start + hi) if window else start + min(hi, n))
+                    assert H.op_budget_usage(got[part], want[part], bf, span) <= 1, (geometry, rows, window, lo, form)
+                at += n
+            assert torch.equal(got, again)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

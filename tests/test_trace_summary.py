@@ -36,3 +36,21 @@ def test_steps_are_cut_between_embedding_kernels(tmp_path, capsys):
     assert trace_summary.main([path]) == 0
     assert "whole run: 16 kernels" in capsys.readouterr().out
     assert trace_summary.main([path, "--step", "prefill", "--index", "9"]) == 1
+
+
+def test_a_step_by_class_of_kernel(tmp_path, capsys):
+    """`--classes`: the step's kernel time under attention, matrix products, elementwise, sampling and the rest, each as
+    a share of the step from first start to last end; the remainder is the gaps between kernels."""
+    step = [("_Z16embedding_kernelItEvPKi(args)", 5), ("_Z18attn_decode_kernelILi128ELb1EEv8AttnArgs.kd", 30),
+            ("_Z17attn_merge_kernelILi128EEvPKf.kd", 10), ("_Z18gemm_skinny_kernelILi1ELi16E.kd", 40),
+            ("Cijk_Alik_Bljk_BBS_BH_Bias_HA_S_SAV_UserArgs_MT128x256x64", 20), ("_Z18rmsnorm_row_kernelItLb1E.kd", 4),
+            ("_Z13argmax_kernelPKfPii.kd", 6), ("__amd_rocclr_copyBuffer.kd", 3)]
+    path = str(tmp_path / "c_results.db")
+    _database(path, step * 4)
+    assert trace_summary.main([path, "--step", "decode", "--classes"]) == 0
+    lines = capsys.readouterr().out.splitlines()
+    table = {" ".join(line.split()[2:]): float(line.split()[0]) for line in lines[lines.index(next(
+        l for l in lines if l.strip().startswith("us"))) + 1:]}
+    assert table == {"matrix products": 60.0, "attention": 40.0, "elementwise": 9.0, "sampling": 6.0,
+                     "other (copies, library elementwise)": 3.0, "between kernels": 3.5}
+    assert trace_summary.kernel_class("_ZN12_GLOBAL__N_116gemm_rows_kernelILi4E") == "matrix products"
