@@ -149,10 +149,18 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
   const int khalf = krow / 16, kin = krow % 16;
   const int max_page = a.table_stride - 1;
 
+  // The block table's entries for a block of 32 keys: the page of its first 16 keys and of its last 16. They are
+  // looked up two blocks ahead and kept in registers, so that no load of keys or values waits for a lookup issued
+  // just before it: a wave's loads return in the order they were issued, and waiting for the newest one (a lookup)
+  // would wait for every load of keys and values still under way.
+  auto lookup = [&](int kb, int (&e)[2]) {
+    e[0] = trow[min(kb / P, max_page)];
+    e[1] = trow[min((kb + 16) / P, max_page)];
+  };
   // Keys of block kb for this lane: two fragments per 32 dims (the lane's key, and the key 4 further on).
-  auto load_keys = [&](int kb, bf16x8_t (&f0)[D / 32], bf16x8_t (&f1)[D / 32]) {
+  auto load_keys = [&](int kb, const int (&e)[2], bf16x8_t (&f0)[D / 32], bf16x8_t (&f1)[D / 32]) {
     const int half_key = kb + 16 * khalf;
-    const int64_t pg = (int64_t)trow[min(half_key / P, max_page)] * page_stride;
+    const int64_t pg = (int64_t)(khalf ? e[1] : e[0]) * page_stride;
     const bf16_t* krowp = kbase + pg + (int64_t)(half_key % P + kin) * D + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < D / 32; ++ks) {
@@ -161,14 +169,17 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
     }
   };
   const int kb_first = (key_lo / 32) * 32;
+  int e_cur[2], e_next[2];
+  lookup(kb_first, e_cur);
+  lookup(kb_first + 32, e_next);
   bf16x8_t kf0[D / 32], kf1[D / 32];
-  load_keys(kb_first, kf0, kf1);
+  load_keys(kb_first, e_cur, kf0, kf1);
   prepare();
   for (int kb = kb_first; kb <= key_hi; kb += 32) {
     // values of this block (lane group g needs keys 8g .. 8g+7, for dims dsub*16 + c) and the keys of the next one
     // are requested before this block's products, so that their latency hides behind the matrix cores
     const int vkey = kb + (g >= 2 ? 16 : 0);
-    const bf16_t* vrowp = vbase + (int64_t)trow[min(vkey / P, max_page)] * page_stride + (int64_t)c * P + vkey % P +
+    const bf16_t* vrowp = vbase + (int64_t)(g >= 2 ? e_cur[1] : e_cur[0]) * page_stride + (int64_t)c * P + vkey % P +
                           8 * (g % 2);
     bf16x8_t vf[D / 16];
 #pragma unroll
@@ -199,7 +210,11 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
     }
     bf16x8_t nf0[D / 32], nf1[D / 32];
     const bool more = kb + 32 <= key_hi;
-    if (more) load_keys(kb + 32, nf0, nf1);
+    int e_after[2] = {0, 0};
+    if (more) {
+      load_keys(kb + 32, e_next, nf0, nf1);
+      lookup(kb + 64, e_after);                  // (an entry past the row's keys is clamped into the table and unused)
+    }
     bf16x8_t pb[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -230,6 +245,8 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
         kf0[ks] = nf0[ks];
         kf1[ks] = nf1[ks];
       }
+      e_cur[0] = e_next[0]; e_cur[1] = e_next[1];
+      e_next[0] = e_after[0]; e_next[1] = e_after[1];
     }
   }
 }
