@@ -60,8 +60,9 @@ class StepRunner:
 
     # -- inputs ---------------------------------------------------------------------------------------------------
     def _arrays(self, slots: np.ndarray, starts: np.ndarray, counts: np.ndarray, tokens: np.ndarray,
-                take: np.ndarray) -> tuple[list[np.ndarray], dict]:
-        """The int32 arrays of a step, in a fixed order, and the host-side facts about them."""
+                take: np.ndarray, wanted: np.ndarray | None = None) -> tuple[list[np.ndarray], dict]:
+        """The int32 arrays of a step, in a fixed order, and the host-side facts about them. `wanted` (the flat places
+        whose logits are asked for) rides behind the cache groups' write targets when given."""
         cache = self.cache
         total, n = int(counts.sum()), len(slots)
         if total == n:                             # one token a row: the step's shape is the batch's
@@ -78,6 +79,8 @@ class StepRunner:
         for g in cache.groups:
             page, off = cache.write_targets(g.gid, slots[token_row], positions)
             arrays += [page, off]
+        if wanted is not None:
+            arrays.append(wanted)
         fixed = len(arrays)
         dirty = cache.take_dirty()                  # block-table rows that changed: they ride the same copy
         for _, rows, contents in dirty:
@@ -183,60 +186,76 @@ class StepRunner:
     def prepare(self, rows: list[StepRow]) -> tuple[Step, np.ndarray]:
         """Device inputs of a step, and the flat indices of the tokens whose logits are wanted (in row order, then in
         the order of each row's `want`)."""
-        slots, starts, counts, tokens, wanted, take = self._check(rows)
-        arrays, facts = self._arrays(slots, starts, counts, tokens, take)
+        step, wanted, _ = self._prepare(self._check(rows))
+        return step, wanted
+
+    def _prepare(self, checked: tuple) -> tuple[Step, np.ndarray, torch.Tensor | None]:
+        """The same from rows already checked; the last value is the wanted places on the device when only some of
+        the step's tokens are wanted (they ride in the inputs' copy)."""
+        slots, starts, counts, tokens, wanted, take = checked
+        some = 0 < len(wanted) and not _all_in_order(wanted, len(tokens))
+        arrays, facts = self._arrays(slots, starts, counts, tokens, take, wanted if some else None)
         dev = self._to_device(arrays)
         self._table_rows(dev[facts["fixed"]:], facts)
-        return self._step(dev, facts, slots, starts, counts), wanted
+        return self._step(dev, facts, slots, starts, counts), wanted, dev[facts["fixed"] - 1] if some else None
 
     # -- the step -------------------------------------------------------------------------------------------------
-    def _forward(self, step: Step, wanted: np.ndarray | None) -> torch.Tensor | None:
-        """The model on a step; `wanted` None: logits of every token."""
+    def _forward(self, step: Step, wanted: np.ndarray | None, wanted_dev: torch.Tensor | None = None
+                 ) -> torch.Tensor | None:
+        """The model on a step; `wanted` None: logits of every token. `wanted_dev`: the same places on the device."""
         h, delta = self.model.trunk(step)
         if wanted is not None and not len(wanted):
             return None
-        if wanted is None or (len(wanted) == step.n_tokens and (wanted == np.arange(step.n_tokens)).all()):
+        if wanted is None or _all_in_order(wanted, step.n_tokens):
             return self.model.head(h, delta)
-        idx = torch.from_numpy(wanted).to(self.device)
+        idx = wanted_dev if wanted_dev is not None else torch.from_numpy(wanted).to(self.device)
         return self.model.head(h.index_select(0, idx), delta.index_select(0, idx) if delta is not None else None)
 
     @torch.no_grad()
     def run(self, rows: list[StepRow]) -> torch.Tensor | None:
         """Run the rows' tokens through the model; returns float32 logits [wanted, vocab] (None when nothing is
         wanted: then the head does not run). Afterwards the cache holds the rows' tokens."""
+        checked = self._check(rows)
         if self.use_graphs and len(rows) <= BUCKETS[-1] and all(len(r.tokens) == 1 and r.want == [0] for r in rows):
-            logits = self._run_graphed(rows)
+            logits = self._run_graphed(checked)
         else:
-            step, wanted = self.prepare(rows)
+            step, wanted, wanted_dev = self._prepare(checked)
             self.last_slots, self.last_lens = step.slots, step.lens
-            logits = self._forward(step, wanted)
+            logits = self._forward(step, wanted, wanted_dev)
         for r in rows:
             self.cache.advance(r.slot, r.start + len(r.tokens))
         self.steps += 1
         return logits
 
     # -- graphs ---------------------------------------------------------------------------------------------------
-    def _run_graphed(self, rows: list[StepRow]) -> torch.Tensor:
-        slots, starts, counts, tokens, _, take = self._check(rows)
-        n = len(rows)
+    def _padded(self, checked: tuple, pad: int) -> tuple:
+        """The step with `pad` more rows on the padding slot behind its own: one token at position 0 of the null page."""
+        slots, starts, counts, tokens, wanted, take = checked
+        if not pad:
+            return checked
+        return (np.concatenate((slots, np.full(pad, self.cache.padding_slot, dtype=np.int64))),
+                np.concatenate((starts, np.zeros(pad, dtype=np.int64))),
+                np.concatenate((counts, np.ones(pad, dtype=np.int64))),
+                np.concatenate((tokens, np.zeros(pad, dtype=np.int64))), wanted,
+                np.concatenate((take, np.full(pad, -1, dtype=np.int64))))
+
+    def _arena(self, arrays: list[np.ndarray], facts: dict) -> torch.Tensor:
+        """Room at a fixed address for a step's inputs and, behind them, for every block-table row."""
+        size = sum(a.size for a in arrays[: facts["fixed"]])
+        size += sum(gr.table.size + gr.table.shape[0] for gr in self.cache.groups)
+        return torch.zeros(size, dtype=torch.int32, device=self.device)
+
+    def _run_graphed(self, checked: tuple) -> torch.Tensor:
+        n = len(checked[0])
         bucket = next(b for b in BUCKETS if b >= n)
-        longest = int((starts + counts).max())
-        len_bucket = max(LEN_BUCKET_MIN, 1 << (longest - 1).bit_length())
-        pad = bucket - n
-        if pad:                                    # rows on the padding slot: one token at position 0 of the null page
-            slots = np.concatenate((slots, np.full(pad, self.cache.padding_slot, dtype=np.int64)))
-            starts = np.concatenate((starts, np.zeros(pad, dtype=np.int64)))
-            counts = np.concatenate((counts, np.ones(pad, dtype=np.int64)))
-            tokens = np.concatenate((tokens, np.zeros(pad, dtype=np.int64)))
-            take = np.concatenate((take, np.full(pad, -1, dtype=np.int64)))
+        slots, starts, counts, tokens, _, take = self._padded(checked, bucket - n)
+        len_bucket = _len_bucket(int((starts + counts).max()))
         arrays, facts = self._arrays(slots, starts, counts, tokens, take)
         facts["max_decode_len"] = len_bucket       # launch shapes are the bucket's, whatever the rows' lengths
         key = (bucket, len_bucket)
         g = self.graphs.get(key)
-        if g is None:                              # the step's inputs at a fixed address, then room for every table row
-            size = sum(a.size for a in arrays[: facts["fixed"]])
-            size += sum(gr.table.size + gr.table.shape[0] for gr in self.cache.groups)
-            arena = torch.zeros(size, dtype=torch.int32, device=self.device)
+        if g is None:
+            arena = self._arena(arrays, facts)
             dev = self._to_device(arrays, arena)
             g = _Graph(arena=arena, step=self._step(dev, facts, slots, starts, counts))
             self.graphs[key] = g
@@ -257,3 +276,11 @@ class StepRunner:
         g.graph.replay()
         self.graph_replays += 1
         return g.logits[:n]
+
+
+def _len_bucket(longest: int) -> int:
+    return max(LEN_BUCKET_MIN, 1 << (max(longest, 1) - 1).bit_length())
+
+
+def _all_in_order(wanted: np.ndarray, n_tokens: int) -> bool:
+    return len(wanted) == n_tokens and bool((wanted == np.arange(n_tokens)).all())
