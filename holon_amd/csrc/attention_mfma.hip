@@ -841,6 +841,230 @@ __device__ __forceinline__ void scores_to_probs(const f32x16_t& sc, int kb, int 
   }
 }
 
+// The same for head_dim 128 with a stage's keys and values copied from the cache into LDS by the memory pipeline
+// itself (global_load_lds: 16 bytes a lane, a wave's 64 lanes into one contiguous kilobyte of LDS), two stages ahead
+// of the one being multiplied, into three buffers in turn: no registers hold a stage on its way, and no instruction
+// writes LDS. A wave's kilobyte has to be contiguous, so rows cannot be padded apart; instead each 16-byte piece
+// sits at place `piece ^ (row % 16)` of its key's 256-byte row (values: each half of the stage's keys apart, a dim's 16
+// keys a row of 32 bytes, place `piece ^ (row / 8 % 2)`), which a lane's source address arranges and a lane's read
+// undoes: 16 lanes that read the same piece of 16 consecutive rows then touch every bank once, as with padded rows.
+// Every copy instruction reads one page, so its lanes share a scalar base and their own offsets never change.
+// The compiler does not know these loads (it would wait for all of them before every read of LDS): they are issued
+// from inline assembly, and the one wait per stage that they need (all but the newest stage's four loads a lane) is
+// written by hand in front of the stage's barrier. Nothing else loads from memory inside the loop.
+// (the source: a base every lane shares, in scalar registers, plus a byte offset of the lane's own)
+__device__ __forceinline__ void load_to_lds16(const void* base, uint32_t lane_bytes, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               : : "v"(lane_bytes), "s"(base), "s"(lds_wave_base) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_loads_but() {          // until at most N of this wave's loads are under way
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+__global__ void __launch_bounds__(256, 2) attn_prefill_dma_kernel(AttnArgs a) {
+  constexpr int D = 128;
+  constexpr int K_BYTES = 32 * D * 2, V_BYTES = D * 32 * 2, STAGE_BYTES = K_BYTES + V_BYTES;   // 8 KB + 8 KB
+  __shared__ __attribute__((aligned(1024))) unsigned char stage_lds[3][STAGE_BYTES];
+  constexpr int PG = 4096;
+  __shared__ int32_t pg_lds[PG];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, tid = threadIdx.x;
+  const int h = lane / 32, c = lane % 32;
+  const int b = a.row_ids[a.unpaired ? blockIdx.z / 2 : blockIdx.z];
+  const int group = a.heads / a.kv_heads;      // <= 32 (the host checks)
+  const TileMap32 tm = tile_map32(group);
+  const int hk = blockIdx.y;
+  const int qs = a.qstart[b], nq = a.qstart[b + 1] - qs, n = a.lens[b];
+  const int n_tiles = (nq + tm.pos_per_tile - 1) / tm.pos_per_tile;
+  const int n_ranges = (n_tiles + 3) / 4;      // a block owns four tiles per range, one a wave
+  if (n <= 0 || (int)blockIdx.x >= (n_ranges + 1) / 2) return;   // uniform over the block
+  const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
+  const int P = a.page_size;
+  const int64_t plane = (int64_t)P * D;
+  const int64_t page_stride = 2 * (int64_t)a.kv_heads * plane;
+  const bf16_t* kbase = a.pages + (int64_t)hk * plane;
+  const bf16_t* vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
+  const int max_page = min(a.table_stride, PG) - 1;
+  for (int i = tid; i < min(PG, a.table_stride); i += 256) pg_lds[i] = trow[i];
+  // What this lane copies per stage: two pieces of keys and two of values (instruction q = 2 * wave + i of eight;
+  // waves 0 and 1 copy the stage's first 16 keys, which lie in one page, waves 2 and 3 its last 16).
+  // Keys: kilobyte q holds rows 4 q .. 4 q + 3; row 8 i' + 4 h' + r holds key 16 (i' / 2) + 8 h' + 4 (i' % 2) + r of
+  // the stage (the order the score product's result wants), so rows 0-15 are the first half. Values: kilobyte q holds
+  // dims 32 (q % 4) .. + 31 of half q / 4, two pieces a dim: keys 0-7 and 8-15 of the half.
+  const int second = __builtin_amdgcn_readfirstlane(wave / 2);   // which half this wave copies
+  uint32_t k_src[2], v_src[2];                 // byte offsets from the half's first key / from the half's first value
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = 2 * wave + i;
+    const int row = 4 * q + lane / 16, piece = (lane % 16) ^ (row % 16);
+    const int key = 16 * ((row / 8) / 2) + 8 * ((row % 8) / 4) + 4 * ((row / 8) % 2) + row % 4;
+    k_src[i] = (uint32_t)(((key % 16) * D + piece * 8) * 2);
+    const int dim = 32 * (q % 4) + lane / 2, vpiece = (lane % 2) ^ ((dim / 8) % 2);
+    v_src[i] = (uint32_t)((dim * P + 8 * vpiece) * 2);
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&stage_lds[0][0];
+  // where this lane reads: keys, row c, piece 2 ds + h; values, half t, row 32 db + c, piece h
+  uint32_t k_at[D / 16], v_at[2];
+#pragma unroll
+  for (int ds = 0; ds < D / 16; ++ds) k_at[ds] = (uint32_t)(c * (D * 2) + 16 * ((2 * ds + h) ^ (c % 16)));
+#pragma unroll
+  for (int t = 0; t < 2; ++t) v_at[t] = (uint32_t)(K_BYTES + t * (V_BYTES / 2) + c * 32 + 16 * (h ^ ((c / 8) % 2)));
+  const int pi = c / tm.rows_per_pos, hi = c % tm.rows_per_pos;
+
+  const int pass_lo = a.unpaired ? 1 - (int)(blockIdx.z % 2) : 0, pass_hi = a.unpaired ? pass_lo + 1 : 2;
+  for (int pass = pass_lo; pass < pass_hi; ++pass) {
+    const int range = pass == 0 ? (int)blockIdx.x : n_ranges - 1 - (int)blockIdx.x;
+    if (pass == 1 && range <= (int)blockIdx.x) break;
+    const int p_lo = range * 4 * tm.pos_per_tile;
+    const int p_hi = min(nq, p_lo + 4 * tm.pos_per_tile) - 1;
+    const int key_hi = n - nq + p_hi;                          // over the whole block (all waves walk the same stages)
+    const int key_lo = a.window > 0 ? max(0, n - nq + p_lo - a.window + 1) : 0;
+    const int p0 = (range * 4 + wave) * tm.pos_per_tile;       // this wave's tile
+    const int qi = p0 + pi;
+    const bool valid = pi < tm.pos_per_tile && qi < nq && hi < group;
+    const int token = qs + qi, head = hk * group + hi;
+    const int qpos = valid ? n - nq + qi : -1;
+    const int tile_last = p0 < nq ? n - nq + min(nq, p0 + tm.pos_per_tile) - 1 : -1;
+    const int tile_first = n - nq + p0;
+    bf16x8_t qf[D / 16];
+    {
+      const bf16_t* qp = a.q + ((int64_t)token * a.heads + head) * D + 8 * h;
+#pragma unroll
+      for (int ds = 0; ds < D / 16; ++ds) {
+        if (valid) {
+          qf[ds] = load8(qp + ds * 16);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) qf[ds][i] = (__bf16)0.f;
+        }
+      }
+    }
+    f32x16_t o[D / 32];
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    const int kb_last = (key_hi / 32) * 32;
+    // four loads a lane: the stage at kb (a stage past the end copies the last one again) into buffer `buf`
+    auto copy_stage = [&](int kb_want, int buf) {
+      const int kb = min(kb_want, kb_last) + 16 * second;       // this wave's half of the stage: 16 keys of one page
+      const int64_t pg = (int64_t)__builtin_amdgcn_readfirstlane(pg_lds[min(kb / P, max_page)]) * page_stride;
+      const int off = kb % P;
+      const bf16_t* kh = kbase + pg + (int64_t)off * D;
+      const bf16_t* vh = vbase + pg + off;
+      const uint32_t to = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)buf * STAGE_BYTES + (uint32_t)wave * 2048);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        load_to_lds16(kh, k_src[i], to + 1024 * i);
+        load_to_lds16(vh, v_src[i], to + K_BYTES + 1024 * i);
+      }
+    };
+    auto stage = [&](auto last, int kb, int buf) {
+      if (kb <= tile_last) {
+        const unsigned char* at = &stage_lds[buf][0];
+        f32x16_t sc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+        bf16x8_t kf[D / 16];
+#pragma unroll
+        for (int ds = 0; ds < D / 16; ++ds) kf[ds] = *reinterpret_cast<const bf16x8_t*>(at + k_at[ds]);
+#pragma unroll
+        for (int ds = 0; ds < D / 16; ++ds) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds], qf[ds], sc, 0, 0, 0);
+        bf16x8_t vf[D / 32][2];
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db) {
+          vf[db][0] = *reinterpret_cast<const bf16x8_t*>(at + v_at[0] + db * 1024);
+          vf[db][1] = *reinterpret_cast<const bf16x8_t*>(at + v_at[1] + db * 1024);
+          if constexpr (decltype(last)::value) {
+            zero_after(vf[db][0], kb + 8 * h, key_hi);
+            zero_after(vf[db][1], kb + 16 + 8 * h, key_hi);
+          }
+        }
+        const int first = a.window > 0 ? qpos - a.window + 1 : 0;
+        const bool whole = kb + 31 <= tile_first && (a.window <= 0 || kb >= tile_last - a.window + 1);
+        // value idx = 4i + r of this lane is key kb + 16*(i/2) + 8h + 4*(i%2) + r against query column c
+        float sv[16];
+#pragma unroll
+        for (int idx = 0; idx < 16; ++idx) sv[idx] = sc[idx];
+        if (!whole) {
+#pragma unroll
+          for (int idx = 0; idx < 16; ++idx) {
+            const int i = idx / 4, r = idx % 4;
+            const int key = kb + 16 * (i / 2) + 8 * h + 4 * (i % 2) + r;
+            if (!(key <= qpos && key >= first)) sv[idx] = -INFINITY;
+          }
+        }
+        float mx = sv[0];
+#pragma unroll
+        for (int idx = 1; idx < 16; ++idx) mx = fmaxf(mx, sv[idx]);
+        {                                          // the other half of the keys is in lane l ^ 32
+          const auto halves = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+          mx = fmaxf(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
+        }
+        const float m_new = fmaxf(m, mx * a.scale_log2);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        bf16x8_t pb0, pb1;
+        float psum = 0.f;
+#pragma unroll
+        for (int idx = 0; idx < 16; ++idx) {
+          const float p = __builtin_amdgcn_exp2f(fmaf(sv[idx], a.scale_log2, -m_use));
+          psum += p;
+          if (idx < 8) pb0[idx] = (__bf16)p; else pb1[idx - 8] = (__bf16)p;
+        }
+        if (__any(m_new != m)) {
+          const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+          l *= alpha;
+#pragma unroll
+          for (int db = 0; db < D / 32; ++db) o[db] *= alpha;
+          m = m_new;
+        }
+        l += psum;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db) {
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][0], pb0, o[db], 0, 0, 0);
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][1], pb1, o[db], 0, 0, 0);
+        }
+      }
+    };
+    const int kb_first = (key_lo / 32) * 32;
+    wait_loads_but<0>();         // (a stage past the end of the pass before may still be on its way into a buffer)
+    lds_barrier();               // the previous pass has finished reading the buffers; the table is in LDS
+    copy_stage(kb_first, 0);
+    copy_stage(kb_first + 32, 1);
+    wait_loads_but<4>();
+    lds_barrier();
+    int buf = 0;
+    for (int kb = kb_first; kb < kb_last; kb += 32) {          // every stage before the last one
+      copy_stage(kb + 64, buf >= 1 ? buf - 1 : 2);             // (buf + 2) % 3: read last a stage ago
+      stage(std::false_type{}, kb, buf);
+      wait_loads_but<4>();                                     // the next stage has landed (this wave's share of it)
+      lds_barrier();
+      buf = buf == 2 ? 0 : buf + 1;
+    }
+    stage(std::true_type{}, kb_last, buf);
+    float lt = l + __shfl_xor(l, 32, WAVE);
+    if (valid) {
+      const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+      bf16_t* op = a.out + ((int64_t)token * a.heads + head) * D + 4 * h;
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          ushort4 w;
+          w.x = float_to_bf16(o[db][4 * i + 0] * inv);
+          w.y = float_to_bf16(o[db][4 * i + 1] * inv);
+          w.z = float_to_bf16(o[db][4 * i + 2] * inv);
+          w.w = float_to_bf16(o[db][4 * i + 3] * inv);
+          *reinterpret_cast<ushort4*>(op + db * 32 + 8 * i) = w;
+        }
+    }
+  }
+  wait_loads_but<0>();           // nothing of this wave is on its way into LDS when the block ends
+}
+
 template <int D>
 __global__ void __launch_bounds__(256, 1) attn_prefill_pair_kernel(AttnArgs a) {
   constexpr int KP = D + 8;    // pitch of a key row in LDS (elements)
@@ -1439,6 +1663,15 @@ extern "C" int holon_attention_prefill_form(int form) {
   return was;
 }
 
+// Whether tiles of 32 rows at head_dim 128 have their stages copied into LDS by the memory pipeline (1, the default) or
+// through registers (0; tests run both); returns what was set before; a negative argument only asks.
+static int g_prefill_dma = 1;
+extern "C" int holon_attention_prefill_copies(int direct) {
+  const int was = g_prefill_dma;
+  if (direct == 0 || direct == 1) g_prefill_dma = direct;
+  return was;
+}
+
 static bool mfma_serves(int head_dim, int page_size) {
   return (head_dim == 64 || head_dim == 128 || head_dim == 256) && page_size % 16 == 0;
 }
@@ -1488,6 +1721,7 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
       a.unpaired = (int64_t)((ranges32 + 1) / 2) * kv_heads * n_rows < UNPAIR_BELOW ? 1 : 0;
       dim3 lgrid((ranges32 + 1) / 2, kv_heads, a.unpaired ? 2 * n_rows : n_rows);
       if (head_dim == 64) attn_prefill_wide_kernel<64><<<lgrid, 256, 0, ls>>>(a);
+      else if (g_prefill_dma) attn_prefill_dma_kernel<<<lgrid, 256, 0, ls>>>(a);
       else attn_prefill_wide_kernel<128><<<lgrid, 256, 0, ls>>>(a);
     } else if (blocks2 >= 512) {
       dim3 lgrid((ranges2 + 1) / 2, kv_heads * tm.head_blocks, n_rows);

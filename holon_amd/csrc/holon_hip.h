@@ -48,6 +48,9 @@ int holon_attention_prefill_bf16(const void* q, void* out, const void* pages, co
 // Which kernel long prompt portions of groups of up to 32 heads take: 0 one tile of 32 rows a wave, 2 two tiles a wave,
 // 1 (the default) two from 12,288 keys on. Returns the setting before; a negative argument changes nothing.
 int holon_attention_prefill_form(int form);
+// 1 (default): long portions at head_dim 128 copy their stages into LDS without passing registers; 0: through registers.
+// Returns the setting before; a negative argument only asks.
+int holon_attention_prefill_copies(int direct);
 // One query token per row; the keys are split over `splits` waves of `keys_per_split` keys (a multiple of 32) whose
 // partial results (part_o [n_rows, heads, splits, head_dim], part_ml [n_rows, heads, splits, 2], float32) are merged
 // in split order.

@@ -71,6 +71,7 @@ class HipKernels:
             "holon_attention_decode_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P,
                                             _I, _I, _P],
             "holon_attention_prefill_form": [_I],
+            "holon_attention_prefill_copies": [_I],
             "holon_attention_decode_waves_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
                                                   _P, _P, _I, _I, _I, _I, _P],
             "holon_attention_decode_fused_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,

@@ -288,13 +288,17 @@ def test_long_prompt_portions_two_tiles_a_wave(hip, geometry):
         q, pages, table, attn = _paged_case(rows, heads, kv_heads, head_dim, 16, bf, seed=len(rows) + window)
         scale = head_dim ** -0.5
         want = PLAIN.paged_attention(q.double(), pages.double(), table, attn, 16, scale, window)
-        for form in (0, 2):                      # one tile of 32 rows a wave, and two (groups of up to 32 heads)
+        # one tile of 32 rows a wave, its stages copied into LDS by the memory pipeline (head_dim 128) or through
+        # registers, and two tiles a wave (groups of up to 32 heads)
+        for form, direct in ((0, 1), (0, 0), (2, 1)):
             before = hip.lib.holon_attention_prefill_form(form)
+            copies = hip.lib.holon_attention_prefill_copies(direct)
             try:
                 got = hip.paged_attention(q, pages, table, attn, 16, scale, window)
                 again = hip.paged_attention(q, pages, table, attn, 16, scale, window)
             finally:
                 hip.lib.holon_attention_prefill_form(before)
+                hip.lib.holon_attention_prefill_copies(copies)
             # rows that see few keys are averages of few values and much larger than rows that see thousands: each
             # stretch of rows is held to the budget of its own size and of the keys it sees
             at = 0
@@ -302,7 +306,7 @@ def test_long_prompt_portions_two_tiles_a_wave(hip, geometry):
                 for lo, hi in ((0, 64), (64, 512), (512, n)):
                     part = slice(at + lo, at + min(hi, n))
                     span = head_dim + (min(window, start + hi) if window else start + min(hi, n))
-                    assert H.op_budget_usage(got[part], want[part], bf, span) <= 1, (geometry, rows, window, lo, form)
+                    assert H.op_budget_usage(got[part], want[part], bf, span) <= 1, (geometry, rows, window, lo, form, direct)
                 at += n
             assert torch.equal(got, again)
 
