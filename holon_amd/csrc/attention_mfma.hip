@@ -863,12 +863,82 @@ __device__ __forceinline__ void wait_loads_but() {          // until at most N o
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+// A block's staging of 32-key stages at head_dim 128 through three LDS buffers: what each lane copies, where it reads.
+struct StagedCopies {
+  static constexpr int D = 128;
+  static constexpr int K_BYTES = 32 * D * 2, V_BYTES = D * 32 * 2, STAGE_BYTES = K_BYTES + V_BYTES;   // 8 KB + 8 KB
+  static constexpr int BUFFERS = 3, PG = 4096;
+  const unsigned char* lds;      // BUFFERS * STAGE_BYTES, aligned to 1,024
+  const int32_t* pg;             // the row's block table, in LDS
+  const bf16_t* kbase;
+  const bf16_t* vbase;
+  int64_t page_stride;
+  int P, max_page, second, wave;
+  uint32_t lds0, k_src[2], v_src[2], k_at[D / 16], v_at[2];
+
+  // What this lane copies per stage: two pieces of keys and two of values (instruction q = 2 * wave + i of eight;
+  // waves 0 and 1 copy the stage's first 16 keys, which lie in one page, waves 2 and 3 its last 16).
+  // Keys: kilobyte q holds rows 4 q .. 4 q + 3; row 8 i' + 4 h' + r holds key 16 (i' / 2) + 8 h' + 4 (i' % 2) + r of
+  // the stage (the order the score product's result wants), so rows 0-15 are the first half. Values: kilobyte q holds
+  // dims 32 (q % 4) .. + 31 of half q / 4, two pieces a dim: keys 0-7 and 8-15 of the half.
+  // Where it reads: keys, row c, piece 2 ds + h; values, half t, row 32 db + c, piece h (lane = 32 h + c).
+  __device__ __forceinline__ void init(const unsigned char* stage_lds, const int32_t* pg_lds, const AttnArgs& a, int hk) {
+    lds = stage_lds;
+    pg = pg_lds;
+    P = a.page_size;
+    const int64_t plane = (int64_t)P * D;
+    page_stride = 2 * (int64_t)a.kv_heads * plane;
+    kbase = a.pages + (int64_t)hk * plane;
+    vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
+    max_page = min(a.table_stride, PG) - 1;
+    const int lane = threadIdx.x % WAVE, h = lane / 32, c = lane % 32;
+    wave = threadIdx.x / WAVE;
+    second = __builtin_amdgcn_readfirstlane(wave / 2);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int q = 2 * wave + i;
+      const int row = 4 * q + lane / 16, piece = (lane % 16) ^ (row % 16);
+      const int key = 16 * ((row / 8) / 2) + 8 * ((row % 8) / 4) + 4 * ((row / 8) % 2) + row % 4;
+      k_src[i] = (uint32_t)(((key % 16) * D + piece * 8) * 2);
+      const int dim = 32 * (q % 4) + lane / 2, vpiece = (lane % 2) ^ ((dim / 8) % 2);
+      v_src[i] = (uint32_t)((dim * P + 8 * vpiece) * 2);
+    }
+    lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)stage_lds;
+#pragma unroll
+    for (int ds = 0; ds < D / 16; ++ds) k_at[ds] = (uint32_t)(c * (D * 2) + 16 * ((2 * ds + h) ^ (c % 16)));
+#pragma unroll
+    for (int t = 0; t < 2; ++t) v_at[t] = (uint32_t)(K_BYTES + t * (V_BYTES / 2) + c * 32 + 16 * (h ^ ((c / 8) % 2)));
+  }
+  // four loads a lane: the stage at kb (a stage past kb_last copies the last one again) into buffer `buf`
+  __device__ __forceinline__ void copy(int kb_want, int kb_last, int buf) const {
+    const int kb = min(kb_want, kb_last) + 16 * second;         // this wave's half of the stage: 16 keys of one page
+    const int64_t at = (int64_t)__builtin_amdgcn_readfirstlane(pg[min(kb / P, max_page)]) * page_stride;
+    const int off = kb % P;
+    const bf16_t* kh = kbase + at + (int64_t)off * D;
+    const bf16_t* vh = vbase + at + off;
+    const uint32_t to = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)buf * STAGE_BYTES + (uint32_t)wave * 2048);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      load_to_lds16(kh, k_src[i], to + 1024 * i);
+      load_to_lds16(vh, v_src[i], to + K_BYTES + 1024 * i);
+    }
+  }
+  static constexpr int LOADS = 4;                               // of a lane, per stage
+  __device__ __forceinline__ bf16x8_t key(int buf, int ds) const {
+    return *reinterpret_cast<const bf16x8_t*>(lds + buf * STAGE_BYTES + k_at[ds]);
+  }
+  __device__ __forceinline__ bf16x8_t value(int buf, int db, int t) const {
+    return *reinterpret_cast<const bf16x8_t*>(lds + buf * STAGE_BYTES + v_at[t] + db * 1024);
+  }
+  static __device__ __forceinline__ int after(int buf) { return buf == BUFFERS - 1 ? 0 : buf + 1; }
+  static __device__ __forceinline__ int before(int buf) { return buf == 0 ? BUFFERS - 1 : buf - 1; }
+};
+
 __global__ void __launch_bounds__(256, 2) attn_prefill_dma_kernel(AttnArgs a) {
-  constexpr int D = 128;
-  constexpr int K_BYTES = 32 * D * 2, V_BYTES = D * 32 * 2, STAGE_BYTES = K_BYTES + V_BYTES;   // 8 KB + 8 KB
-  __shared__ __attribute__((aligned(1024))) unsigned char stage_lds[3][STAGE_BYTES];
-  constexpr int PG = 4096;
-  __shared__ int32_t pg_lds[PG];
+  using SC = StagedCopies;
+  constexpr int D = SC::D;
+  __shared__ __attribute__((aligned(1024))) unsigned char stage_lds[SC::BUFFERS * SC::STAGE_BYTES];
+  __shared__ int32_t pg_lds[SC::PG];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, tid = threadIdx.x;
   const int h = lane / 32, c = lane % 32;
   const int b = a.row_ids[a.unpaired ? blockIdx.z / 2 : blockIdx.z];
@@ -880,36 +950,9 @@ __global__ void __launch_bounds__(256, 2) attn_prefill_dma_kernel(AttnArgs a) {
   const int n_ranges = (n_tiles + 3) / 4;      // a block owns four tiles per range, one a wave
   if (n <= 0 || (int)blockIdx.x >= (n_ranges + 1) / 2) return;   // uniform over the block
   const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
-  const int P = a.page_size;
-  const int64_t plane = (int64_t)P * D;
-  const int64_t page_stride = 2 * (int64_t)a.kv_heads * plane;
-  const bf16_t* kbase = a.pages + (int64_t)hk * plane;
-  const bf16_t* vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
-  const int max_page = min(a.table_stride, PG) - 1;
-  for (int i = tid; i < min(PG, a.table_stride); i += 256) pg_lds[i] = trow[i];
-  // What this lane copies per stage: two pieces of keys and two of values (instruction q = 2 * wave + i of eight;
-  // waves 0 and 1 copy the stage's first 16 keys, which lie in one page, waves 2 and 3 its last 16).
-  // Keys: kilobyte q holds rows 4 q .. 4 q + 3; row 8 i' + 4 h' + r holds key 16 (i' / 2) + 8 h' + 4 (i' % 2) + r of
-  // the stage (the order the score product's result wants), so rows 0-15 are the first half. Values: kilobyte q holds
-  // dims 32 (q % 4) .. + 31 of half q / 4, two pieces a dim: keys 0-7 and 8-15 of the half.
-  const int second = __builtin_amdgcn_readfirstlane(wave / 2);   // which half this wave copies
-  uint32_t k_src[2], v_src[2];                 // byte offsets from the half's first key / from the half's first value
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int q = 2 * wave + i;
-    const int row = 4 * q + lane / 16, piece = (lane % 16) ^ (row % 16);
-    const int key = 16 * ((row / 8) / 2) + 8 * ((row % 8) / 4) + 4 * ((row / 8) % 2) + row % 4;
-    k_src[i] = (uint32_t)(((key % 16) * D + piece * 8) * 2);
-    const int dim = 32 * (q % 4) + lane / 2, vpiece = (lane % 2) ^ ((dim / 8) % 2);
-    v_src[i] = (uint32_t)((dim * P + 8 * vpiece) * 2);
-  }
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&stage_lds[0][0];
-  // where this lane reads: keys, row c, piece 2 ds + h; values, half t, row 32 db + c, piece h
-  uint32_t k_at[D / 16], v_at[2];
-#pragma unroll
-  for (int ds = 0; ds < D / 16; ++ds) k_at[ds] = (uint32_t)(c * (D * 2) + 16 * ((2 * ds + h) ^ (c % 16)));
-#pragma unroll
-  for (int t = 0; t < 2; ++t) v_at[t] = (uint32_t)(K_BYTES + t * (V_BYTES / 2) + c * 32 + 16 * (h ^ ((c / 8) % 2)));
+  for (int i = tid; i < min(SC::PG, a.table_stride); i += 256) pg_lds[i] = trow[i];
+  SC sc_;
+  sc_.init(stage_lds, pg_lds, a, hk);
   const int pi = c / tm.rows_per_pos, hi = c % tm.rows_per_pos;
 
   const int pass_lo = a.unpaired ? 1 - (int)(blockIdx.z % 2) : 0, pass_hi = a.unpaired ? pass_lo + 1 : 2;
@@ -948,44 +991,30 @@ __global__ void __launch_bounds__(256, 2) attn_prefill_dma_kernel(AttnArgs a) {
     float m = -INFINITY, l = 0.f;
 
     const int kb_last = (key_hi / 32) * 32;
-    // four loads a lane: the stage at kb (a stage past the end copies the last one again) into buffer `buf`
-    auto copy_stage = [&](int kb_want, int buf) {
-      const int kb = min(kb_want, kb_last) + 16 * second;       // this wave's half of the stage: 16 keys of one page
-      const int64_t pg = (int64_t)__builtin_amdgcn_readfirstlane(pg_lds[min(kb / P, max_page)]) * page_stride;
-      const int off = kb % P;
-      const bf16_t* kh = kbase + pg + (int64_t)off * D;
-      const bf16_t* vh = vbase + pg + off;
-      const uint32_t to = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)buf * STAGE_BYTES + (uint32_t)wave * 2048);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        load_to_lds16(kh, k_src[i], to + 1024 * i);
-        load_to_lds16(vh, v_src[i], to + K_BYTES + 1024 * i);
-      }
-    };
+    // `last`: the stage holds the row's last key (std::true_type) and may reach past it
     auto stage = [&](auto last, int kb, int buf) {
       if (kb <= tile_last) {
-        const unsigned char* at = &stage_lds[buf][0];
         f32x16_t sc;
 #pragma unroll
         for (int i = 0; i < 16; ++i) sc[i] = 0.f;
-        bf16x8_t kf[D / 16];
+        bf16x8_t kf[D / 16];                       // all of a stage's key fragments are asked for at once
 #pragma unroll
-        for (int ds = 0; ds < D / 16; ++ds) kf[ds] = *reinterpret_cast<const bf16x8_t*>(at + k_at[ds]);
+        for (int ds = 0; ds < D / 16; ++ds) kf[ds] = sc_.key(buf, ds);
 #pragma unroll
         for (int ds = 0; ds < D / 16; ++ds) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds], qf[ds], sc, 0, 0, 0);
-        bf16x8_t vf[D / 32][2];
+        bf16x8_t vf[D / 32][2];                    // and its value fragments before the softmax that they wait for
 #pragma unroll
         for (int db = 0; db < D / 32; ++db) {
-          vf[db][0] = *reinterpret_cast<const bf16x8_t*>(at + v_at[0] + db * 1024);
-          vf[db][1] = *reinterpret_cast<const bf16x8_t*>(at + v_at[1] + db * 1024);
+          vf[db][0] = sc_.value(buf, db, 0);
+          vf[db][1] = sc_.value(buf, db, 1);
           if constexpr (decltype(last)::value) {
             zero_after(vf[db][0], kb + 8 * h, key_hi);
             zero_after(vf[db][1], kb + 16 + 8 * h, key_hi);
           }
         }
+        // value idx = 4i + r of this lane is key kb + 16*(i/2) + 8h + 4*(i%2) + r against query column c
         const int first = a.window > 0 ? qpos - a.window + 1 : 0;
         const bool whole = kb + 31 <= tile_first && (a.window <= 0 || kb >= tile_last - a.window + 1);
-        // value idx = 4i + r of this lane is key kb + 16*(i/2) + 8h + 4*(i%2) + r against query column c
         float sv[16];
 #pragma unroll
         for (int idx = 0; idx < 16; ++idx) sv[idx] = sc[idx];
@@ -1032,17 +1061,17 @@ __global__ void __launch_bounds__(256, 2) attn_prefill_dma_kernel(AttnArgs a) {
     const int kb_first = (key_lo / 32) * 32;
     wait_loads_but<0>();         // (a stage past the end of the pass before may still be on its way into a buffer)
     lds_barrier();               // the previous pass has finished reading the buffers; the table is in LDS
-    copy_stage(kb_first, 0);
-    copy_stage(kb_first + 32, 1);
-    wait_loads_but<4>();
+    sc_.copy(kb_first, kb_last, 0);
+    sc_.copy(kb_first + 32, kb_last, 1);
+    wait_loads_but<SC::LOADS>();
     lds_barrier();
     int buf = 0;
     for (int kb = kb_first; kb < kb_last; kb += 32) {          // every stage before the last one
-      copy_stage(kb + 64, buf >= 1 ? buf - 1 : 2);             // (buf + 2) % 3: read last a stage ago
+      sc_.copy(kb + 64, kb_last, SC::before(buf));             // two stages on, into the buffer read a stage ago
       stage(std::false_type{}, kb, buf);
-      wait_loads_but<4>();                                     // the next stage has landed (this wave's share of it)
+      wait_loads_but<SC::LOADS>();                             // the next stage has landed (this wave's share of it)
       lds_barrier();
-      buf = buf == 2 ? 0 : buf + 1;
+      buf = SC::after(buf);
     }
     stage(std::true_type{}, kb_last, buf);
     float lt = l + __shfl_xor(l, 32, WAVE);
@@ -1649,10 +1678,11 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict
 #ifndef PAIR_UNPAIR_BELOW
 #define PAIR_UNPAIR_BELOW 512
 #endif
-// Long prompt portions of groups of up to 32 heads: two tiles of 32 rows a wave from PAIR_FROM_KEYS keys on (measured,
-// 32 heads over 8 kv heads of 128, portions of 4,096 tokens, us a layer, one tile against two: behind 4,096 tokens 616
-// and 636, behind 12,288 tokens 1,366 and 1,279, behind 28,672 tokens 2,625 and 2,441; whole prompts of 2,048 and
-// 4,096 tokens 78 and 101, 208 and 298: short rows have too few blocks of 256 rows to fill the GPU).
+// Long prompt portions of groups of up to 32 heads whose stages pass registers on their way into LDS (head_dim 64; 128
+// when the direct copies are switched off): two tiles of 32 rows a wave from PAIR_FROM_KEYS keys on (measured, 32 heads
+// over 8 kv heads of 128, portions of 4,096 tokens, us a layer, one tile against two: behind 4,096 tokens 616 and 636,
+// behind 12,288 tokens 1,366 and 1,279, behind 28,672 tokens 2,625 and 2,441; whole prompts of 2,048 and 4,096 tokens
+// 78 and 101, 208 and 298: short rows have too few blocks of 256 rows to fill the GPU).
 // holon_attention_prefill_form: 0 never, 1 by that rule, 2 always (tests run both forms at the same sizes); returns
 // what was set before; a negative argument only asks.
 constexpr int PAIR_FROM_KEYS = 12288;
@@ -1663,8 +1693,12 @@ extern "C" int holon_attention_prefill_form(int form) {
   return was;
 }
 
-// Whether tiles of 32 rows at head_dim 128 have their stages copied into LDS by the memory pipeline (1, the default) or
-// through registers (0; tests run both); returns what was set before; a negative argument only asks.
+// Whether long portions at head_dim 128 (groups of up to 32 heads) have their stages copied into LDS by the memory
+// pipeline, one tile of 32 rows a wave (1, the default), or through registers, one or two tiles a wave (0; tests run
+// both); returns what was set before; a negative argument only asks. Measured, 32 heads over 8 kv heads, portions of
+// 4,096 tokens, us a layer, direct against the better of the register forms: a whole prompt of 2,048 tokens 65 and 76,
+// of 4,096 tokens 204 and 204; behind 4,096 tokens 552 and 603, behind 12,288 tokens 1,108 and 1,221, behind 28,672
+// tokens 2,206 and 2,246 (0.93 PFLOP/s), behind 61,440 tokens 4,624 and 4,430; 64 heads over 8: 0.97 PFLOP/s behind 28,672.
 static int g_prefill_dma = 1;
 extern "C" int holon_attention_prefill_copies(int direct) {
   const int was = g_prefill_dma;
@@ -1708,7 +1742,9 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
     const TileMap32 tm32 = tile_map32(heads / kv_heads);
     const int ranges32 = ((max_query + tm32.pos_per_tile - 1) / tm32.pos_per_tile + 3) / 4;
     const int ranges_pair = ((max_query + tm32.pos_per_tile - 1) / tm32.pos_per_tile + 7) / 8;
-    if (heads / kv_heads <= 32 && (g_prefill_pair == 2 || (g_prefill_pair == 1 && max_len >= PAIR_FROM_KEYS))) {
+    const bool direct = g_prefill_dma && head_dim == 128 && heads / kv_heads <= 32;   // (then one tile a wave is the faster)
+    if (!direct && heads / kv_heads <= 32 &&
+        (g_prefill_pair == 2 || (g_prefill_pair == 1 && max_len >= PAIR_FROM_KEYS))) {
       // two tiles of 32 rows a wave
       a.unpaired = (int64_t)((ranges_pair + 1) / 2) * kv_heads * n_rows < PAIR_UNPAIR_BELOW ? 1 : 0;
       dim3 lgrid((ranges_pair + 1) / 2, kv_heads, a.unpaired ? 2 * n_rows : n_rows);
@@ -1721,7 +1757,7 @@ extern "C" int holon_attention_prefill_bf16(const void* q, void* out, const void
       a.unpaired = (int64_t)((ranges32 + 1) / 2) * kv_heads * n_rows < UNPAIR_BELOW ? 1 : 0;
       dim3 lgrid((ranges32 + 1) / 2, kv_heads, a.unpaired ? 2 * n_rows : n_rows);
       if (head_dim == 64) attn_prefill_wide_kernel<64><<<lgrid, 256, 0, ls>>>(a);
-      else if (g_prefill_dma) attn_prefill_dma_kernel<<<lgrid, 256, 0, ls>>>(a);
+      else if (direct) attn_prefill_dma_kernel<<<lgrid, 256, 0, ls>>>(a);
       else attn_prefill_wide_kernel<128><<<lgrid, 256, 0, ls>>>(a);
     } else if (blocks2 >= 512) {
       dim3 lgrid((ranges2 + 1) / 2, kv_heads * tm.head_blocks, n_rows);
