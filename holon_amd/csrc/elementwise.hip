@@ -453,6 +453,57 @@ __global__ void qk_norm_rope_write_kernel(const T* qkv, int64_t qkv_stride, T* q
   }
 }
 
+// Values of 16 consecutive tokens of one kv head into the cache. Inside a page values are stored transposed
+// ([D, P]), so a token alone writes D scattered elements; 16 tokens that fill consecutive places of one page are
+// transposed through LDS and written as 32 contiguous bytes per dim. A block of 256 threads; `tile` and `together`
+// are the block's.
+template <typename T, int PITCH>
+__device__ __forceinline__ void v_write_group(T (*tile)[PITCH], int* together, int t0, int hk,
+                                              const T* __restrict__ qkv, int64_t qkv_stride, int v_col0, int tokens,
+                                              int kv_heads, int head_dim, T* __restrict__ pages,
+                                              const int32_t* __restrict__ write_page,
+                                              const int32_t* __restrict__ write_off, int page_size) {
+  const int tid = threadIdx.x;
+  const int count = min(16, tokens - t0);
+  if (tid == 0) {
+    int ok = count == 16 && write_off[t0] % 8 == 0 && write_off[t0] + 16 <= page_size;
+    for (int j = 1; ok && j < 16; ++j)
+      ok = write_page[t0 + j] == write_page[t0] && write_off[t0 + j] == write_off[t0] + j;
+    *together = ok;
+  }
+  const int per_row = head_dim / 8;   // head_dim % 8 == 0 (checked by the host)
+  for (int q = tid; q < count * per_row; q += 256) {
+    const int tk = q / per_row, c8 = (q % per_row) * 8;
+    const T* src = qkv + (int64_t)(t0 + tk) * qkv_stride + v_col0 + (int64_t)hk * head_dim + c8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) tile[tk][c8 + j] = src[j];
+  }
+  __syncthreads();
+  const int64_t plane = (int64_t)page_size * head_dim;
+  if (*together) {
+    T* base = pages + (((int64_t)write_page[t0] * 2 + 1) * kv_heads + hk) * plane + write_off[t0];
+    for (int r = tid; r < head_dim * 2; r += 256) {
+      const int d = r / 2, half = r % 2;
+      T out8[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) out8[j] = tile[half * 8 + j][d];
+      T* dst = base + (int64_t)d * page_size + half * 8;
+      if (sizeof(T) == 2) {
+        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(out8);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst[j] = out8[j];
+      }
+    }
+  } else {
+    for (int q = tid; q < count * head_dim; q += 256) {
+      const int tk = q % count, d = q / count;
+      pages[(((int64_t)write_page[t0 + tk] * 2 + 1) * kv_heads + hk) * plane + (int64_t)d * page_size +
+            write_off[t0 + tk]] = tile[tk][d];
+    }
+  }
+}
+
 // The same for head_dim 64, 128 or 256 with the whole head rotated (or not at all): each lane holds 8 consecutive
 // values (one 16-byte load), LPH = head_dim / 8 lanes make a head, a wave holds 64 / LPH heads. The rotation partner
 // of a value sits LPH / 2 lanes away; norm sums run over the LPH lanes of a head. No LDS.
@@ -461,9 +512,19 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
     const T* qkv, int64_t qkv_stride, T* q_out, int heads, int kv_heads, const T* __restrict__ q_weight,
     const T* __restrict__ k_weight, float eps, const float* __restrict__ table, const int32_t* __restrict__ positions,
     T* __restrict__ pages, const int32_t* __restrict__ write_page, const int32_t* __restrict__ write_off,
-    int page_size, int total_heads) {
+    int page_size, int total_heads, int tokens, int value_groups) {
   constexpr int D = LPH * 8;
   constexpr int HPB = 256 / LPH;                     // heads a block covers at a time
+  // With many tokens the values do not go through the heads' loop (a token alone would write them an element at a
+  // time): blocks behind the tokens' own take 16 tokens of one kv head each (`value_groups` groups of 16 tokens).
+  __shared__ T tile[16][D + 8];
+  __shared__ int together;
+  if ((int)blockIdx.x >= tokens) {
+    const int v = blockIdx.x - tokens;
+    v_write_group<T, D + 8>(tile, &together, (v % value_groups) * 16, v / value_groups, qkv, qkv_stride, (heads + kv_heads) * D,
+                     tokens, kv_heads, D, pages, write_page, write_off, page_size);
+    return;
+  }
   const int t = blockIdx.x;
   const int li = threadIdx.x % LPH;                  // lane within the head
   // Everything the block reads is asked for before anything is waited for, the longest chain first: the token's
@@ -547,58 +608,6 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
   }
 }
 
-// Values of 16 consecutive tokens of one kv head into the cache. Inside a page values are stored transposed
-// ([D, P]), so a token alone writes D scattered elements; 16 tokens that fill consecutive places of one page are
-// transposed through LDS and written as 32 contiguous bytes per dim.
-template <typename T>
-__global__ void __launch_bounds__(256) v_write_group_kernel(const T* __restrict__ qkv, int64_t qkv_stride, int v_col0,
-                                                            int tokens, int kv_heads, int head_dim,
-                                                            T* __restrict__ pages,
-                                                            const int32_t* __restrict__ write_page,
-                                                            const int32_t* __restrict__ write_off, int page_size) {
-  __shared__ T tile[16][MAX_HEAD_DIM + 8];
-  __shared__ int together;
-  const int t0 = blockIdx.x * 16, hk = blockIdx.y, tid = threadIdx.x;
-  const int count = min(16, tokens - t0);
-  if (tid == 0) {
-    int ok = count == 16 && write_off[t0] % 8 == 0 && write_off[t0] + 16 <= page_size;
-    for (int j = 1; ok && j < 16; ++j)
-      ok = write_page[t0 + j] == write_page[t0] && write_off[t0 + j] == write_off[t0] + j;
-    together = ok;
-  }
-  const int per_row = head_dim / 8;   // head_dim % 8 == 0 (checked by the host)
-  for (int q = tid; q < count * per_row; q += 256) {
-    const int tk = q / per_row, c8 = (q % per_row) * 8;
-    const T* src = qkv + (int64_t)(t0 + tk) * qkv_stride + v_col0 + (int64_t)hk * head_dim + c8;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) tile[tk][c8 + j] = src[j];
-  }
-  __syncthreads();
-  const int64_t plane = (int64_t)page_size * head_dim;
-  if (together) {
-    T* base = pages + (((int64_t)write_page[t0] * 2 + 1) * kv_heads + hk) * plane + write_off[t0];
-    for (int r = tid; r < head_dim * 2; r += 256) {
-      const int d = r / 2, half = r % 2;
-      T out8[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) out8[j] = tile[half * 8 + j][d];
-      T* dst = base + (int64_t)d * page_size + half * 8;
-      if (sizeof(T) == 2) {
-        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(out8);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) dst[j] = out8[j];
-      }
-    }
-  } else {
-    for (int q = tid; q < count * head_dim; q += 256) {
-      const int tk = q % count, d = q / count;
-      pages[(((int64_t)write_page[t0 + tk] * 2 + 1) * kv_heads + hk) * plane + (int64_t)d * page_size +
-            write_off[t0 + tk]] = tile[tk][d];
-    }
-  }
-}
-
 extern "C" int holon_qk_norm_rope_write(const void* qkv, int64_t qkv_stride, void* q_out, int tokens, int heads,
                                         int kv_heads, int head_dim, const void* q_weight, const void* k_weight,
                                         float eps, const float* table, int rotary_dim, int max_positions,
@@ -619,17 +628,18 @@ extern "C" int holon_qk_norm_rope_write(const void* qkv, int64_t qkv_stride, voi
   hipStream_t s = (hipStream_t)stream;
   if ((head_dim == 64 || head_dim == 128 || head_dim == 256) && (table == nullptr || rotary_dim == head_dim) &&
       qkv != q_out) {
-    // many tokens: values go through their own kernel, 16 tokens at a time (contiguous writes); the heads kernel then
-    // covers queries and keys only
+    // many tokens: the values are written 16 tokens at a time (contiguous writes) by blocks of their own behind the
+    // tokens' blocks in the same launch; the heads' loop then covers queries and keys only
     const bool split_v = pages != nullptr && tokens >= 256;
     const int fast_heads = split_v ? heads + kv_heads : total_heads;
     const int lph = head_dim / 8;
+    const int value_groups = split_v ? (tokens + 15) / 16 : 0;
     // many tokens: one block a token walks all its heads, with the token's cosines and sines read once
-    grid = dim3(tokens, tokens >= 256 ? 1 : (fast_heads + 256 / lph - 1) / (256 / lph));
+    grid = dim3(tokens + value_groups * kv_heads, tokens >= 256 ? 1 : (fast_heads + 256 / lph - 1) / (256 / lph));
 #define QK_FAST(T, LPH)                                                                                            \
   qk_norm_rope_write_fast_kernel<T, LPH><<<grid, 256, 0, s>>>(                                                      \
       (const T*)qkv, qkv_stride, (T*)q_out, heads, kv_heads, (const T*)q_weight, (const T*)k_weight, eps, table,    \
-      positions, (T*)pages, write_page, write_off, page_size, fast_heads)
+      positions, (T*)pages, write_page, write_off, page_size, fast_heads, tokens, value_groups)
     if (dtype == HOLON_F32) {
       if (head_dim == 64) QK_FAST(float, 8); else if (head_dim == 128) QK_FAST(float, 16); else QK_FAST(float, 32);
     } else {
@@ -637,17 +647,6 @@ extern "C" int holon_qk_norm_rope_write(const void* qkv, int64_t qkv_stride, voi
     }
 #undef QK_FAST
     HOLON_LAUNCH_OK();
-    if (split_v) {
-      dim3 vgrid((tokens + 15) / 16, kv_heads);
-      const int v_col0 = (heads + kv_heads) * head_dim;
-      if (dtype == HOLON_F32)
-        v_write_group_kernel<float><<<vgrid, 256, 0, s>>>((const float*)qkv, qkv_stride, v_col0, tokens, kv_heads,
-                                                          head_dim, (float*)pages, write_page, write_off, page_size);
-      else
-        v_write_group_kernel<bf16_t><<<vgrid, 256, 0, s>>>((const bf16_t*)qkv, qkv_stride, v_col0, tokens, kv_heads,
-                                                           head_dim, (bf16_t*)pages, write_page, write_off, page_size);
-      HOLON_LAUNCH_OK();
-    }
     return 0;
   }
 #define QK_LAUNCH(T)                                                                                              \

@@ -388,6 +388,34 @@ def test_fused_norm_rope_write_is_the_three_ops(hip, dtype, geometry):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geometry", [(32, 8, 128, 16), (16, 4, 256, 32), (6, 2, 64, 16)])
+def test_values_of_many_tokens_are_written_16_tokens_a_block(hip, dtype, geometry):
+    """From 256 tokens on, the norm + rotation + write kernel's launch has blocks behind the tokens' own that write the
+    values, 16 tokens of one kv head each, transposed through LDS: whole groups inside one page, groups that straddle
+    pages or start off a multiple of 8, a ragged last group, scattered places. Values bit for bit, nothing else touched,
+    queries and keys within the budget."""
+    from holon_amd.parts.positions import rope_table
+    heads, kv_heads, head_dim, page = geometry
+    table = rope_table(4096, head_dim, 1e6).cuda()
+    rng = np.random.default_rng(1)
+    qw, kw = _randn(head_dim, dtype=dtype, seed=9), _randn(head_dim, dtype=dtype, seed=10)
+    for t, where in ((530, np.arange(530) + page + 5), (1040, np.arange(1040) + 2 * page),
+                     (257, rng.permutation(60 * page)[:257]), (300, np.arange(300) * 2)):
+        units = int(where.max()) // page + 2
+        qkv = _randn(t, (heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=t)
+        pos = torch.as_tensor(rng.integers(0, 4096, t).astype(np.int32)).cuda()
+        wp, wo = (torch.as_tensor((where // page).astype(np.int32)).cuda(), torch.as_tensor((where % page).astype(np.int32)).cuda())
+        pages_h = torch.zeros(units, 2, kv_heads, page * head_dim, dtype=dtype).cuda()
+        pages_p = pages_h.clone()
+        got = hip.qk_norm_rope_write(qkv, heads, kv_heads, head_dim, qw, kw, 1e-6, table, pos, pages_h, wp, wo, page)
+        want = PLAIN.qk_norm_rope_write(qkv, heads, kv_heads, head_dim, qw, kw, 1e-6, table, pos, pages_p, wp, wo, page)
+        assert torch.equal(pages_h[:, 1], pages_p[:, 1]), (geometry, t, "values are copied bit for bit")
+        assert torch.equal(pages_h == 0, pages_p == 0), "a cache entry outside the written ones changed"
+        assert H.op_budget_usage(got, want, dtype, head_dim) <= 1
+        assert H.op_budget_usage(pages_h[:, 0], pages_p[:, 0], dtype, head_dim) <= 1
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_linear(hip, dtype):
     # up to 16 rows the few-row kernel runs (bfloat16, K >= 256), above that the vendor library's product
     for t, k, n in ((1, 4096, 6144), (8, 4096, 1000), (17, 100, 333), (64, 12288, 4096), (300, 120, 1000), (2, 96, 384),
