@@ -943,6 +943,7 @@ __global__ void __launch_bounds__(256, 2) attn_prefill_dma_kernel(AttnArgs a) {
   constexpr int D = SC::D;
   __shared__ __attribute__((aligned(1024))) unsigned char stage_lds[SC::BUFFERS * SC::STAGE_BYTES];
   __shared__ int32_t pg_lds[SC::PG];
+  static_assert(sizeof(stage_lds) + sizeof(pg_lds) <= 64 * 1024, "a block's static LDS; two blocks share a compute unit");
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, tid = threadIdx.x;
   const int h = lane / 32, c = lane % 32;
   const int b = a.row_ids[a.unpaired ? blockIdx.z / 2 : blockIdx.z];
