@@ -76,6 +76,7 @@ class SamplingParams:
     seed: int | None = None
     logprobs: int | None = None          # with every generated token: its log-probability and the k most likely (k <= 32)
     prompt_logprobs: int | None = None   # the same for the prompt's own tokens, each given the tokens before it
+    ext: dict[str, Any] = dataclasses.field(default_factory=dict)   # a caller's own values; the engine reads none (core/holon/api/batch.py:61)
 
     def check(self) -> None:
         for name in ("logprobs", "prompt_logprobs"):
