@@ -32,7 +32,9 @@ def engine_flags(parser: argparse.ArgumentParser | argparse._ArgumentGroup) -> N
         flag, kind = "--" + f.name.replace("_", "-"), hints[f.name]
         help_ = f.metadata["help"] + (f" (default: {f.default})" if f.default is not None else "")
         if kind is bool:
-            parser.add_argument(flag, action=argparse.BooleanOptionalAction, default=f.default, help=help_)
+            # (`--cuda-graphs` is the reference's name for `--graphs`, core/holon/core/engine.py:83; both are taken)
+            also = ["--cuda-graphs", "--no-cuda-graphs"] if f.name == "graphs" else []
+            parser.add_argument(flag, *also[:1], action=argparse.BooleanOptionalAction, default=f.default, help=help_)
         elif f.name == "max_model_len":            # also `auto` (core/holon/core/cli.py:44-47, 76)
             parser.add_argument(flag, type=lambda s: s if s == "auto" else int(s), default=f.default,
                                 help=help_ + f"; auto: the model's trained context, at most {AUTO_CONTEXT}")

@@ -107,6 +107,7 @@ def test_command_line_has_a_flag_per_engine_setting():
     a = ap.parse_args(["--dtype", "float32", "--page-size", "8", "--max-seqs", "3", "--no-graphs", "--chunk-with-decode", "0"])
     cfg = engine_config("folder", a)
     assert (cfg.model, cfg.dtype, cfg.page_size, cfg.max_seqs, cfg.graphs) == ("folder", "float32", 8, 3, False)
+    assert not engine_config("folder", ap.parse_args(["--no-cuda-graphs"])).graphs     # the reference's name for the flag
     flags = {x.dest for x in ap._actions}
     assert {f.name for f in dataclasses.fields(EngineConfig)} - {"model"} <= flags
     out = subprocess.run([sys.executable, "-m", "holon_amd", "models"], capture_output=True, text=True, check=True)
