@@ -852,21 +852,6 @@ __device__ __forceinline__ void scores_to_probs(const f32x16_t& sc, int kb, int 
 // The compiler does not know these loads (it would wait for all of them before every read of LDS): they are issued
 // from inline assembly, and the one wait per stage that they need (all but the newest stage's four loads a lane) is
 // written by hand in front of the stage's barrier. Nothing else loads from memory inside the loop.
-// (the source: a base every lane shares, in scalar registers, plus a byte offset of the lane's own)
-// M0 holds the wave's place in LDS for the instruction behind it; nothing the compiler writes in these kernels uses M0.
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-__device__ __forceinline__ void load_to_lds16(const void* base, uint32_t lane_bytes, uint32_t lds_wave_base) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               : : "v"(lane_bytes), "s"(base), "s"(lds_wave_base) : "memory", "m0");
-}
-#pragma clang diagnostic pop
-template <int N>
-__device__ __forceinline__ void wait_loads_but() {          // until at most N of this wave's loads are under way
-  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
 // A block's staging of 32-key stages at head_dim 128 through three LDS buffers: what each lane copies, where it reads.
 struct StagedCopies {
   static constexpr int D = 128;

@@ -50,6 +50,27 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// A copy from memory straight into LDS (global_load_lds_dwordx4): 16 bytes a lane, the wave's 64 lanes into one
+// contiguous kilobyte of LDS at `lds_wave_base` (the same for every lane); the source is a base every lane shares, in
+// scalar registers, plus a byte offset of the lane's own. The compiler does not know these loads (known ones make it
+// wait for all of them before every read of LDS): a kernel that issues them writes its own waits (`wait_loads_but`)
+// in front of the barrier that publishes what they brought. They count among the wave's loads like any other, in
+// the order of issue.
+// M0 holds the wave's place in LDS for the instruction behind it; nothing the compiler writes in these kernels uses M0.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void load_to_lds16(const void* base, uint32_t lane_bytes, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               : : "v"(lane_bytes), "s"(base), "s"(lds_wave_base) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+template <int N>
+__device__ __forceinline__ void wait_loads_but() {          // until at most N of this wave's loads are under way
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+
 // Host side: every entry point returns 0 or a negative code and leaves a message for holon_last_error().
 void holon_set_error(const char* fmt, ...);
 #define HOLON_CHECK(cond, ...)        \

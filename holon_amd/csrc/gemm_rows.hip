@@ -3,10 +3,13 @@
 //
 // The few-row kernel streams the weights and lets every block read its rows of activations from L2; with 64 rows those
 // reads cost as much as the weights. Here a block's waves walk K together and share the rows through LDS: a chunk of
-// KC columns of all rows is copied in once per block (double buffered, the next chunk's copy under way while this one
-// is used), each wave streams the weights of its own tile (from the tiled copy: a contiguous kilobyte a product) for
-// the next chunk while it multiplies this one, and reads its activations as B operands from LDS. A wave sums its tile
-// over all of K in order, so a result depends on nothing but the operands.
+// KC columns of all rows is copied in once per block by the memory pipeline itself (global_load_lds, no register and
+// no LDS write instruction on the way; double buffered, the next chunk's copy under way while this one is used), each
+// wave streams the weights of its own tile (from the tiled copy: a contiguous kilobyte a product) for the next chunk
+// while it multiplies this one, and reads its activations as B operands from LDS. A copy's kilobyte is contiguous
+// in LDS, so rows are not padded apart but swizzled: a row's 16-byte piece j sits at place j ^ (row % 16) (rows of 128
+// bytes: j ^ (row / 2 % 8)), and 16 lanes that read the same piece of 16 consecutive rows touch every bank once. A
+// wave sums its tile over all of K in order, so a result depends on nothing but the operands.
 //
 // Weights with tiles enough to fill the GPU (a gated feed-forward's first product, the head) are served whole. Narrow
 // ones (a few hundred tiles: q/k/v, output and down projections) have K split over blocks as well (grid y): every
@@ -29,11 +32,14 @@ template <int MT, int WAVES, int KC, int OUT>
 __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(const bf16_t* __restrict__ x,
                                                                const bf16_t* __restrict__ w, void* __restrict__ y,
                                                                int M, int N, int K) {
-  constexpr int ROWS = MT * 16, PITCH = KC + 8, STEPS = KC / 32, THREADS = WAVES * 64;
-  constexpr int PIECES = ROWS * KC / 8;                     // 16-byte pieces of a chunk of activations
-  constexpr int XCH = (PIECES + THREADS - 1) / THREADS;     // of which a thread copies this many
-  __shared__ __attribute__((aligned(16))) bf16_t xs[2][ROWS * PITCH];
-  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, tid = threadIdx.x;
+  constexpr int ROWS = MT * 16, STEPS = KC / 32;
+  constexpr int PPR = KC / 8;                               // 16-byte pieces a row of a chunk has
+  constexpr int RPI = 64 / PPR;                             // rows one copy instruction (a kilobyte) brings
+  constexpr int COPIES = ROWS / RPI;                        // instructions a chunk takes
+  constexpr int XCH = (COPIES + WAVES - 1) / WAVES;         // of which a wave issues this many
+  static_assert(KC == 64 || KC == 128 || KC == 256, "rows of 128, 256 or 512 bytes");
+  __shared__ __attribute__((aligned(1024))) bf16_t xs[2][ROWS * KC];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
   constexpr bool GATED = OUT == 2;
   constexpr int COLS = GATED ? WAVES / 2 : WAVES;            // output tiles of 16 columns a block writes
@@ -44,58 +50,59 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(const bf16_t* __r
   f32x4_t acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  bf16x8_t wcur[STEPS], wnext[STEPS], xr[XCH];
+  bf16x8_t wcur[STEPS], wnext[STEPS];
   auto load_w = [&](int chunk, bf16x8_t (&to)[STEPS]) {
 #pragma unroll
     for (int s = 0; s < STEPS; ++s)
       to[s] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wp + ((int64_t)chunk * STEPS + s) * 512));
   };
-  auto load_x = [&](int chunk) {                            // rows beyond M are zeros
+  // what this lane copies: of instruction j = i * WAVES + wave, row j * RPI + lane / PPR, the piece that belongs at
+  // place lane % PPR (rows beyond M repeat the last row: what they give is never written)
+  uint32_t x_src[XCH];
+#pragma unroll
+  for (int i = 0; i < XCH; ++i) {
+    const int row = (i * WAVES + wave) * RPI + lane / PPR;
+    const int piece = (lane % PPR) ^ (KC == 64 ? (row / 2) % 8 : row % 16);
+    x_src[i] = (uint32_t)(((int64_t)min(row, M - 1) * K + piece * 8) * 2);
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&xs[0][0];
+  auto copy_x = [&](int chunk, int buf) {
+    const bf16_t* from = x + (int64_t)chunk * KC;
 #pragma unroll
     for (int i = 0; i < XCH; ++i) {
-      const int q = tid + i * THREADS;
-      const int row = q / (KC / 8), col = (q % (KC / 8)) * 8;
-      if (q < PIECES && row < M) {
-        xr[i] = *reinterpret_cast<const bf16x8_t*>(x + (int64_t)row * K + (int64_t)chunk * KC + col);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) xr[i][j] = (__bf16)0.f;
-      }
+      const int j = i * WAVES + wave;                       // (uniform over the wave)
+      if (j < COPIES) load_to_lds16(from, x_src[i], lds0 + (uint32_t)(buf * ROWS * KC * 2 + j * 1024));
     }
   };
-  auto store_x = [&](int buf) {
+  // where this lane reads the B operand of product s for the tile of tokens t: row 16 t + c, piece 4 s + g
+  uint32_t x_at[STEPS];
 #pragma unroll
-    for (int i = 0; i < XCH; ++i) {
-      const int q = tid + i * THREADS;
-      const int row = q / (KC / 8), col = (q % (KC / 8)) * 8;
-      if (q < PIECES) *reinterpret_cast<bf16x8_t*>(&xs[buf][row * PITCH + col]) = xr[i];
-    }
-  };
+  for (int s = 0; s < STEPS; ++s) x_at[s] = (uint32_t)(c * KC + 8 * ((4 * s + g) ^ (KC == 64 ? (c / 2) % 8 : c)));
   const int chunks = K / KC / (int)gridDim.y;              // this block's share of K (all of it unless OUT == 3)
   const int first = (int)blockIdx.y * chunks;
   load_w(first, wcur);
-  load_x(first);
-  store_x(0);
+  copy_x(first, 0);
+  wait_loads_but<0>();
   __syncthreads();
   for (int ch = 0; ch < chunks; ++ch) {
     const int buf = ch & 1;
     const bool more = ch + 1 < chunks;                      // (uniform)
     if (more) {
       load_w(first + ch + 1, wnext);
-      load_x(first + ch + 1);
+      copy_x(first + ch + 1, buf ^ 1);                      // the other buffer: last read before the barrier behind us
     }
 #pragma unroll
     for (int s = 0; s < STEPS; ++s)
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(&xs[buf][(t * 16 + c) * PITCH + s * 32 + 8 * g]);
+        const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(&xs[buf][t * 16 * KC + x_at[s]]);
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wcur[s], b, acc[t], 0, 0, 0);
       }
     if (more) {
-      store_x(buf ^ 1);                                     // the other buffer: last read before the barrier below
 #pragma unroll
       for (int s = 0; s < STEPS; ++s) wcur[s] = wnext[s];
     }
+    wait_loads_but<0>();                                    // the next chunk's rows have landed (this wave's share)
     __syncthreads();
   }
   if constexpr (GATED) {                                     // the gate waves hand their rounded sums to the up waves
