@@ -138,7 +138,10 @@ int holon_sum_parts(const void* parts, void* y, int splits, int64_t count, void*
 int holon_gemm_f32(const void* x, const void* w, void* y, int M, int N, int K, void* stream);
 // scale (nullable, [K] bfloat16): tiled holds round(w[n][k] * scale[k]).
 int holon_tile_weight_bf16(const void* w, void* tiled, int N, int K, const void* scale, void* stream);
-int holon_argmax(const float* logits, int32_t* out, int rows, int vocab, void* stream);
+// `pieces`: room for rows x holon_argmax_pieces(vocab) pairs (float32, int32) when that is not 0 (a wide row is then
+// searched by many blocks and a second kernel picks among them), or NULL (one block a row).
+int holon_argmax_pieces(int vocab);
+int holon_argmax(const float* logits, int32_t* out, int rows, int vocab, void* pieces, void* stream);
 // last_token[slots[r]] = tokens[r] for r < rows (slots are distinct; last_token has n_slots entries).
 int holon_store_tokens(int32_t* last_token, const int32_t* slots, const int32_t* tokens, int rows, int n_slots,
                        void* stream);

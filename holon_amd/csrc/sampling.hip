@@ -17,7 +17,8 @@ __device__ __forceinline__ ArgMax better(ArgMax a, ArgMax b) {   // larger value
   return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
 }
 
-__device__ ArgMax block_argmax(const float* __restrict__ row, int vocab, float temp) {
+// (nothing to choose from, a row of NaN: index 0, or 0x7fffffff with `none_is_zero` off)
+__device__ ArgMax block_argmax(const float* __restrict__ row, int vocab, float temp, bool none_is_zero = true) {
   __shared__ ArgMax part[SAMPLE_THREADS / WAVE];
   __shared__ ArgMax result;
   ArgMax best{-INFINITY, 0x7fffffff};
@@ -43,7 +44,7 @@ __device__ ArgMax block_argmax(const float* __restrict__ row, int vocab, float t
   if (threadIdx.x == 0) {
     ArgMax r = part[0];
     for (int w = 1; w < (int)blockDim.x / WAVE; ++w) r = better(r, part[w]);
-    if (r.i == 0x7fffffff) r.i = 0;   // a row of NaN or -inf: the first token
+    if (r.i == 0x7fffffff && none_is_zero) r.i = 0;   // a row of NaN: the first token
     result = r;
   }
   __syncthreads();
@@ -55,10 +56,47 @@ __global__ void argmax_kernel(const float* __restrict__ logits, int32_t* __restr
   if (threadIdx.x == 0) out[blockIdx.x] = r.i;
 }
 
-extern "C" int holon_argmax(const float* logits, int32_t* out, int rows, int vocab, void* stream) {
+// A wide row in two kernels: block (piece, row) finds the best of its ARGMAX_PIECE values, then one wave a row the best
+// of the pieces (ties go to the smaller index in both, so the answer is the one block's). One block walking 151,936
+// values alone takes 17.5 us; the two kernels together 7.
+constexpr int ARGMAX_PIECE = 4096;
+constexpr int ARGMAX_MAX_PIECES = 1024;
+__global__ void __launch_bounds__(SAMPLE_THREADS) argmax_pieces_kernel(const float* __restrict__ logits,
+                                                                        ArgMax* __restrict__ pieces, int vocab) {
+  const int lo = blockIdx.x * ARGMAX_PIECE;
+  const ArgMax r = block_argmax(logits + (int64_t)blockIdx.y * vocab + lo, min(ARGMAX_PIECE, vocab - lo), 1.0f, false);
+  if (threadIdx.x == 0)
+    pieces[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = ArgMax{r.v, r.i == 0x7fffffff ? r.i : r.i + lo};
+}
+__global__ void __launch_bounds__(WAVE) argmax_of_pieces_kernel(const ArgMax* __restrict__ pieces,
+                                                                int32_t* __restrict__ out, int n) {
+  ArgMax best{-INFINITY, 0x7fffffff};
+  for (int i = threadIdx.x; i < n; i += WAVE) best = better(best, pieces[(int64_t)blockIdx.x * n + i]);
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) {
+    ArgMax other{__shfl_xor(best.v, o, WAVE), __shfl_xor(best.i, o, WAVE)};
+    best = better(best, other);
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = best.i == 0x7fffffff ? 0 : best.i;
+}
+
+// `pieces`: room for holon_argmax_pieces(vocab) pairs of (float, int32) a row, or NULL (one block a row).
+extern "C" int holon_argmax_pieces(int vocab) {
+  const int n = (vocab + ARGMAX_PIECE - 1) / ARGMAX_PIECE;
+  return n >= 4 && n <= ARGMAX_MAX_PIECES ? n : 0;
+}
+
+extern "C" int holon_argmax(const float* logits, int32_t* out, int rows, int vocab, void* pieces, void* stream) {
   HOLON_CHECK(rows >= 0 && vocab > 0, "argmax: bad sizes");
   if (rows == 0) return 0;
-  argmax_kernel<<<rows, SAMPLE_THREADS, 0, (hipStream_t)stream>>>(logits, out, vocab);
+  const int n = holon_argmax_pieces(vocab);
+  if (pieces != nullptr && n > 0) {
+    argmax_pieces_kernel<<<dim3(n, rows), SAMPLE_THREADS, 0, (hipStream_t)stream>>>(logits, (ArgMax*)pieces, vocab);
+    HOLON_LAUNCH_OK();
+    argmax_of_pieces_kernel<<<rows, WAVE, 0, (hipStream_t)stream>>>((const ArgMax*)pieces, out, n);
+  } else {
+    argmax_kernel<<<rows, SAMPLE_THREADS, 0, (hipStream_t)stream>>>(logits, out, vocab);
+  }
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -91,7 +91,8 @@ class HipKernels:
             "holon_gemm_f32": [_P, _P, _P, _I, _I, _I, _P],
             "holon_gemm_skinny_add_bf16": [_P, _P, _P, _I, _I, _I, _P, _P],
             "holon_gemm_skinny_glu_bf16": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _F, _P],
-            "holon_argmax": [_P, _P, _I, _I, _P],
+            "holon_argmax": [_P, _P, _I, _I, _P, _P],
+            "holon_argmax_pieces": [_I],
             "holon_store_tokens": [_P, _P, _P, _I, _I, _P],
             "holon_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P],
             "holon_scatter_rows": [_P, _P, _P, _I, _I, _I, _P],
@@ -724,8 +725,10 @@ class HipKernels:
     def argmax(self, logits):
         self._check(logits, "argmax logits", torch.float32)
         out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+        n = self.lib.holon_argmax_pieces(logits.shape[1])
+        pieces = torch.empty((logits.shape[0] * n, 2), dtype=torch.float32, device=logits.device) if n else None
         self._call(self.lib.holon_argmax, logits.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1],
-                   self._stream())
+                   _ptr(pieces), self._stream())
         return out
 
     def store_tokens(self, last_token, slots, tokens):

@@ -20,7 +20,8 @@ SHORT = (("_Z18gemm_skinny_kernelILi", "gemm_skinny<"), ("_Z22gemm_skinny_glu_ke
          ("_Z18attn_decode_kernelILi", "attn_decode<"), ("_Z19attn_prefill_kernelILi", "attn_prefill<"),
          ("_Z24attn_prefill_wide_kernelILi", "attn_prefill_wide<"), ("_Z23attn_prefill_lds_kernelILi", "attn_prefill_lds<"),
          ("_Z23attn_prefill_dma_kernel8AttnArgs", "attn_prefill_dma"), ("_Z24attn_prefill_pair_kernelILi", "attn_prefill_pair<"),
-         ("_Z17attn_merge_kernel", "attn_merge"), ("_Z13argmax_kernel", "argmax"), ("_Z16embedding_kernel", "embedding"),
+         ("_Z17attn_merge_kernel", "attn_merge"), ("_Z13argmax_kernel", "argmax"), ("_Z20argmax_pieces_kernel", "argmax_pieces"),
+         ("_Z23argmax_of_pieces_kernel", "argmax_of_pieces"), ("_Z16embedding_kernel", "embedding"),
          ("_Z15gemm_f32_kernel", "gemm_f32"), ("_Z13sample_kernel", "sample"),
          ("_ZN12_GLOBAL__N_116gemm_rows_kernelILi", "gemm_rows<"),
          ("_Z19silu_mul_vec_kernel", "silu_mul_vec"), ("Cijk_Alik_Bljk_BBS_BH_Bias_HA_S_SAV_UserArgs_", "hipBLASLt "),

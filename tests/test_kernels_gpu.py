@@ -744,6 +744,27 @@ def test_argmax_and_sampling(hip):
     logits[3, 777] = logits[3, 90_000] = 50.0                     # a tie: the first index wins
     assert hip.argmax(logits).tolist() == logits.argmax(-1).tolist()
     assert int(hip.argmax(logits)[3]) == 777
+    # wide rows are searched in pieces of 4,096: ties across pieces, rows of -inf and of NaN, widths that are no
+    # multiple of 4 (or of the piece), a best value at a piece's first and last place
+    for rows, vocab in ((3, 16_385), (70, 20_001), (2, 16_384), (5, 9_001)):
+        x = torch.randn(rows, vocab, generator=g).cuda()
+        x[0, 4095] = x[0, 4096] = x[0, vocab - 1] = 9.0
+        x[1, :] = float("-inf")
+        x[1, 5000:5003] = float("nan")
+        if rows > 2:
+            x[2, :] = float("nan")
+        if rows > 3:
+            x[3, :4100] = float("nan")
+            x[3, 4100:] = float("-inf")
+            x[4, 8192] = 30.0
+        got = hip.argmax(x).tolist()
+        want = torch.where(x.isnan(), torch.full_like(x, float("-inf")), x).cpu().argmax(-1).tolist()
+        if rows > 2:
+            want[2] = 0                        # nothing to choose from: the first token
+        if rows > 3:
+            want[3] = 4100                     # the first value that is a number
+        assert got == want, (rows, vocab, got[:5], want[:5])
+        assert got[0] == 4095 and got[1] == 0
     # the law, by counting: one row of 40 logits drawn 100,000 times at consecutive positions
     v, n = 40, 100_000
     row = torch.randn(v, generator=torch.Generator().manual_seed(0)) * 2
