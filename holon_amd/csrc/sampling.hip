@@ -24,7 +24,22 @@ __device__ ArgMax block_argmax(const float* __restrict__ row, int vocab, float t
   ArgMax best{-INFINITY, 0x7fffffff};
   if ((vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {   // 16-byte loads where the row allows
     const float4* row4 = reinterpret_cast<const float4*>(row);
-    for (int i = threadIdx.x; i < vocab / 4; i += blockDim.x) {
+    const int n4 = vocab / 4, step = blockDim.x;
+    int i = threadIdx.x;
+    for (; i + 3 * step < n4; i += 4 * step) {           // four loads under way at a time
+      float4 v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = row4[i + e * step];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int at = 4 * (i + e * step);
+        best = better(best, ArgMax{v[e].x / temp, at});
+        best = better(best, ArgMax{v[e].y / temp, at + 1});
+        best = better(best, ArgMax{v[e].z / temp, at + 2});
+        best = better(best, ArgMax{v[e].w / temp, at + 3});
+      }
+    }
+    for (; i < n4; i += step) {
       const float4 v = row4[i];
       best = better(best, ArgMax{v.x / temp, 4 * i});
       best = better(best, ArgMax{v.y / temp, 4 * i + 1});
@@ -478,8 +493,21 @@ __device__ u64 block_scan_u64(u64 v, u64& total) {
 template <typename F>
 __device__ __forceinline__ void for_each_token(const float* __restrict__ row, int vocab, float temp, F f) {
   if ((vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    // four loads under way at a time: a block walks its row alone, and what it waits for is the loads
     const float4* row4 = reinterpret_cast<const float4*>(row);
-    for (int i = threadIdx.x; i < vocab / 4; i += blockDim.x) {
+    const int n4 = vocab / 4, step = blockDim.x;
+    int i = threadIdx.x;
+    for (; i + 3 * step < n4; i += 4 * step) {
+      float4 v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = row4[i + e * step];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int at = 4 * (i + e * step);
+        f(v[e].x / temp, at); f(v[e].y / temp, at + 1); f(v[e].z / temp, at + 2); f(v[e].w / temp, at + 3);
+      }
+    }
+    for (; i < n4; i += step) {
       const float4 v = row4[i];
       f(v.x / temp, 4 * i); f(v.y / temp, 4 * i + 1); f(v.z / temp, 4 * i + 2); f(v.w / temp, 4 * i + 3);
     }
@@ -682,6 +710,137 @@ __device__ bool top_k_cut_wide(const float* __restrict__ row, int vocab, float t
   return true;
 }
 
+// ---- a row's mass by distance below its largest value -----------------------------------------------------------
+// Bins of 1/64 down to 32 below the largest value (what lies further weighs nothing): the mass and the number of the
+// tokens in each. With it "the last token, in sorted order, that has at most a given mass before it" (top-p's last
+// kept token; the drawn token, with the target as the bound) lies in a known bin, and only that bin's tokens have to be
+// collected and sorted, however many tokens precede them. The masses are integers, so the sums are exact.
+#define HIST_BINS 2048
+__device__ __forceinline__ int hist_bin(float d) { return d < 32.f ? (int)(d * 64.f) : HIST_BINS; }   // (a NaN: none)
+
+// Fills the bins; returns the row's mass.
+__device__ u64 mass_histogram(const float* __restrict__ row, int vocab, float temp, float xmax, u64* h_mass, int* h_cnt) {
+  for (int i = threadIdx.x; i < HIST_BINS; i += blockDim.x) { h_mass[i] = 0; h_cnt[i] = 0; }
+  __syncthreads();
+  for_each_token(row, vocab, temp, [&](float x, int) {
+    const int b = hist_bin(xmax - x);
+    if (b < HIST_BINS) {
+      atomicAdd(&h_mass[b], (u64)fixed_mass(__expf(x - xmax)));
+      atomicAdd(&h_cnt[b], 1);
+    }
+  });
+  __syncthreads();
+  u64 mine = 0;
+  for (int i = threadIdx.x; i < HIST_BINS; i += blockDim.x) mine += h_mass[i];
+  return block_sum_u64(mine);
+}
+
+struct BinAt {
+  int bin;        // the first bin at whose end more than the bound has gone by; HIST_BINS: the whole row is within it
+  u64 before;     // the mass of the bins before it
+  int n_before;   // their tokens
+};
+__device__ BinAt bin_past(const u64* h_mass, const int* h_cnt, u64 bound) {
+  __shared__ BinAt found;
+  constexpr int PER = HIST_BINS / SAMPLE_THREADS;
+  const int tid = threadIdx.x;
+  u64 mine = 0, n_mine = 0;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) { mine += h_mass[tid * PER + e]; n_mine += (u64)h_cnt[tid * PER + e]; }
+  u64 total, n_total;
+  const u64 before = block_scan_u64(mine, total);
+  const u64 n_before = block_scan_u64(n_mine, n_total);
+  if (tid == 0) found = BinAt{HIST_BINS, total, (int)n_total};
+  __syncthreads();
+  if (before <= bound && bound < before + mine) {      // (one thread)
+    u64 run = before;
+    int n = (int)n_before;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const u64 m = h_mass[tid * PER + e];
+      if (run + m > bound) { found = BinAt{tid * PER + e, run, n}; break; }
+      run += m;
+      n += h_cnt[tid * PER + e];
+    }
+  }
+  __syncthreads();
+  const BinAt at = found;
+  __syncthreads();
+  return at;
+}
+
+// The tokens of bins lo .. hi into cand[] as order keys, sorted (taken earlier first) and padded with zeros to a power
+// of two, which `n_pad` receives; returns how many there are. The caller knows from the bins' counts that they fit.
+__device__ int collect_bins_sorted(const float* __restrict__ row, int vocab, float temp, float xmax, int lo, int hi,
+                                   u64* cand, int* n_cand, int& n_pad) {
+  if (threadIdx.x == 0) *n_cand = 0;
+  __syncthreads();
+  for_each_token(row, vocab, temp, [&](float x, int i) {
+    const int b = hist_bin(xmax - x);
+    if (b >= lo && b <= hi) {
+      const int at = atomicAdd(n_cand, 1);
+      if (at < SAMPLE_CANDIDATES) cand[at] = order_key(x, i);
+    }
+  });
+  __syncthreads();
+  const int count = min(*n_cand, SAMPLE_CANDIDATES);
+  n_pad = WAVE;
+  while (n_pad < count) n_pad <<= 1;
+  for (int i = count + threadIdx.x; i < n_pad; i += blockDim.x) cand[i] = 0;
+  __syncthreads();
+  bitonic_sort(cand, n_pad, true);
+  return count;
+}
+
+// cand[0 .. count) sorted, `above` the mass of what precedes them all: how many of them have at most `bound` before
+// them (a prefix, as the sums only grow), and in `through` the mass up to and including the last of those.
+__device__ int within_bound(const u64* cand, int count, int n_pad, float xmax, u64 above, u64 bound, u64& through) {
+  __shared__ u64 through_s;
+  const int tid = threadIdx.x;
+  const int per = max(1, n_pad / SAMPLE_THREADS);     // 1, 2 or 4
+  u64 incl[SAMPLE_PER];
+  u64 run = 0;
+#pragma unroll
+  for (int e = 0; e < SAMPLE_PER; ++e) {
+    const int i = tid * per + e;
+    if (e < per && i < count) run += fixed_mass(__expf(key_float((uint32_t)(cand[i] >> 32)) - xmax));
+    incl[e] = run;
+  }
+  u64 all;
+  const u64 before = above + block_scan_u64(run, all);
+  int mine = 0;
+#pragma unroll
+  for (int e = 0; e < SAMPLE_PER; ++e) {
+    const int i = tid * per + e;
+    if (e < per && i < count) mine += (before + (e ? incl[e - 1] : 0)) <= bound;
+  }
+  const int kept = block_sum_int(mine);
+  if (tid == 0) through_s = above;
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < SAMPLE_PER; ++e)
+    if (e < per && tid * per + e == kept - 1) through_s = before + incl[e];
+  __syncthreads();
+  through = through_s;
+  __syncthreads();
+  return kept;
+}
+
+// The order key of the last token, in sorted order, with at most `bound` before it, from the bins: 0 when the bin
+// that holds it has more tokens than there is room for, or when the whole row lies within the bound (the caller then
+// halves ranges instead). `through`: the mass up to and including that token.
+__device__ u64 last_within(const float* __restrict__ row, int vocab, float temp, float xmax, u64 bound,
+                           const u64* h_mass, const int* h_cnt, u64* cand, int* n_cand, u64& through) {
+  const BinAt at = bin_past(h_mass, h_cnt, bound);
+  if (at.bin == HIST_BINS || h_cnt[at.bin] > SAMPLE_CANDIDATES) return 0;
+  int n_pad;
+  const int count = collect_bins_sorted(row, vocab, temp, xmax, at.bin, at.bin, cand, n_cand, n_pad);
+  const int kept = within_bound(cand, count, n_pad, xmax, at.before, bound, through);   // >= 1: the bin's first token
+  const u64 key = cand[max(kept, 1) - 1];
+  __syncthreads();
+  return key;
+}
+
 __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     const float* __restrict__ logits, int32_t* __restrict__ out, int vocab, const float* __restrict__ temperature,
     const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
@@ -692,6 +851,8 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
   __shared__ int band_counts[SAMPLE_WAVES][SAMPLE_BANDS];
   __shared__ int n_cand, n_keep_s, pick_s;
   __shared__ u64 z_k_s;
+  __shared__ u64 h_mass[HIST_BINS];
+  __shared__ int h_cnt[HIST_BINS];
   const int r = blockIdx.x, tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const float* row = logits + (int64_t)r * vocab;
   const int pr = slots != nullptr ? slots[r] : r;     // where this row's parameters lie: by its slot, or by its place
@@ -722,7 +883,36 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
   if (filtered) {
     u64 cut = 0;
     bool wide = !(k_on || p_on || m_on);         // k >= vocab and nothing else: everything is kept, in sorted order
-    if (k_on || p_on) {
+    bool binned = false;                         // h_mass / h_cnt hold this row
+    u64 kept_mass = 0;                           // (wide, top-p alone, no min-p) the mass of the kept tokens, else 0
+    if (p_on && !k_on) {
+      // top-p alone: the row's mass by bins says which bin holds the last kept token and how many tokens precede it.
+      // A kept set that fits the room is collected whole, sorted, and drawn from there; of a larger one only that bin.
+      const u64 z_all = mass_histogram(row, vocab, temp, xmax, h_mass, h_cnt);
+      binned = true;
+      const u64 bound = (u64)((double)p_keep * (double)z_all);
+      const BinAt at = bin_past(h_mass, h_cnt, bound);
+      if (at.bin == HIST_BINS) {
+        wide = true;                             // (a row whose mass rounds to the bound: everything is kept)
+      } else if (at.n_before + h_cnt[at.bin] <= SAMPLE_CANDIDATES) {
+        int n_pad;
+        const int count = collect_bins_sorted(row, vocab, temp, xmax, 0, at.bin, cand, &n_cand, n_pad);
+        u64 through;
+        const int kept = within_bound(cand, count, n_pad, xmax, 0, bound, through);
+        if (tid == 0) n_keep_s = kept;
+        __syncthreads();
+      } else {
+        wide = true;
+        u64 through = 0;
+        cut = last_within(row, vocab, temp, xmax, bound, h_mass, h_cnt, cand, &n_cand, through);
+        if (cut != 0 && !m_on) kept_mass = through;
+        if (cut == 0) cut = top_p_cut_wide(row, vocab, temp, xmax, bound, cand, &n_cand);
+        if (cut == 0) {                          // thousands of equal values where the cut falls
+          sample_row_general(row, out + r, vocab, temp, top, k, p_keep, p_min, u);
+          return;
+        }
+      }
+    } else if (k_on || p_on) {
       u64 z_all = 0;
       if (!k_on) {                               // top-p without top-k: the mass of the whole row
         u64 mass = 0;
@@ -884,14 +1074,23 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     // target: the search for "the last token whose preceding mass is within a bound" that top-p uses, with the target as
     // the bound (what precedes a kept token is kept, so the search need not know the filters).
     __syncthreads();                            // `cand` is free from here on
-    u64 mass = 0;
-    for_each_token(row, vocab, temp, [&](float x, int i) {
-      const float q = __expf(x - xmax);
-      if (order_key(x, i) >= cut && q >= p_min) mass += fixed_mass(q);
-    });
-    const u64 total = block_sum_u64(mass);
+    u64 total = kept_mass;
+    if (total == 0) {
+      u64 mass = 0;
+      for_each_token(row, vocab, temp, [&](float x, int i) {
+        const float q = __expf(x - xmax);
+        if (order_key(x, i) >= cut && q >= p_min) mass += fixed_mass(q);
+      });
+      total = block_sum_u64(mass);
+    }
     const u64 target = (u64)((double)u * (double)total);
-    const u64 hit = total > 0 ? top_p_cut_wide(row, vocab, temp, xmax, target, cand, &n_cand) : 0;
+    u64 hit = 0;
+    if (total > 0) {
+      if (!binned) mass_histogram(row, vocab, temp, xmax, h_mass, h_cnt);
+      u64 through;
+      hit = last_within(row, vocab, temp, xmax, target, h_mass, h_cnt, cand, &n_cand, through);
+      if (hit == 0) hit = top_p_cut_wide(row, vocab, temp, xmax, target, cand, &n_cand);
+    }
     if (total > 0 && hit == 0) {                 // thousands of equal values around the target
       sample_row_general(row, out + r, vocab, temp, top, k, p_keep, p_min, u);
       return;
