@@ -403,10 +403,13 @@ __device__ void sample_row_general(const float* __restrict__ row, int32_t* __res
 // The fast form. Masses are integers, Q = trunc(exp(x - max) * (2^32 - 256)): sums of them are exact in any order, so
 // every decision below is the same whatever the threads' order, and a sum over a part of the row is exact too.
 //   1. the largest value;
-//   2. (a filter is set) how many tokens lie in each of 16 bands below the largest value (within 1, 2, ... 8, 12, 16,
-//      ... 128), and for top-p without top-k the row's mass; the fewest bands that are sure to hold the kept set are
-//      collected into LDS (at most SAMPLE_CANDIDATES tokens) and sorted by (value descending, index ascending): the
-//      order in which top-k and top-p take tokens. If no such set fits, the row takes the general form;
+//   2. (top-k is set) how many tokens lie in each of 16 bands below the largest value (within 1, 2, ... 8, 12, 16,
+//      ... 128); the fewest bands that are sure to hold the kept set are collected into LDS (at most SAMPLE_CANDIDATES
+//      tokens) and sorted by (value descending, index ascending): the order in which top-k and top-p take tokens.
+//      (top-p alone) the row's mass and token counts in 2,048 bins below the largest value say which bin holds the last
+//      kept token and how many tokens precede it: a kept set that fits is collected whole and sorted, of a longer one
+//      only that bin, which gives the cut. A cut that cannot be found this way is found by halving ranges, and where
+//      thousands of equal values lie at the cut the row takes the general form;
 //   3. top-k keeps the first k of the sorted set; top-p those whose preceding mass is <= top_p * (mass of what top-k
 //      kept); both keep a prefix, so the kept set is "(value, index) at or before the last kept one": one compare;
 //   4. min-p drops q < min_p (the largest q is 1): a prefix again; the draw is the inverse CDF over the integer masses
