@@ -465,18 +465,26 @@ __device__ __forceinline__ void v_write_group(T (*tile)[PITCH], int* together, i
                                               const int32_t* __restrict__ write_off, int page_size) {
   const int tid = threadIdx.x;
   const int count = min(16, tokens - t0);
-  if (tid == 0) {
-    int ok = count == 16 && write_off[t0] % 8 == 0 && write_off[t0] + 16 <= page_size;
-    for (int j = 1; ok && j < 16; ++j)
-      ok = write_page[t0 + j] == write_page[t0] && write_off[t0 + j] == write_off[t0] + j;
-    *together = ok;
+  if (tid < WAVE) {                    // lane j looks at token j's place: one round of loads, not sixteen
+    int pg = 0, off = 0;
+    if (tid < count) { pg = write_page[t0 + tid]; off = write_off[t0 + tid]; }
+    const int pg0 = __shfl(pg, 0, WAVE), off0 = __shfl(off, 0, WAVE);
+    const bool ok = count == 16 && off0 % 8 == 0 && off0 + 16 <= page_size &&
+                    (tid >= 16 || (pg == pg0 && off == off0 + tid));
+    const bool all_ok = __all(ok);
+    if (tid == 0) *together = all_ok;
   }
   const int per_row = head_dim / 8;   // head_dim % 8 == 0 (checked by the host)
   for (int q = tid; q < count * per_row; q += 256) {
     const int tk = q / per_row, c8 = (q % per_row) * 8;
     const T* src = qkv + (int64_t)(t0 + tk) * qkv_stride + v_col0 + (int64_t)hk * head_dim + c8;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) tile[tk][c8 + j] = src[j];
+    // (16-byte pieces: the caller's sizes put every piece of eight values on a 16-byte edge, here and in `tile`)
+    if (sizeof(T) == 2) {
+      *reinterpret_cast<uint4*>(&tile[tk][c8]) = *reinterpret_cast<const uint4*>(src);
+    } else {
+      *reinterpret_cast<float4*>(&tile[tk][c8]) = *reinterpret_cast<const float4*>(src);
+      *reinterpret_cast<float4*>(&tile[tk][c8 + 4]) = *reinterpret_cast<const float4*>(src + 4);
+    }
   }
   __syncthreads();
   const int64_t plane = (int64_t)page_size * head_dim;
@@ -517,7 +525,7 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
   constexpr int HPB = 256 / LPH;                     // heads a block covers at a time
   // With many tokens the values do not go through the heads' loop (a token alone would write them an element at a
   // time): blocks behind the tokens' own take 16 tokens of one kv head each (`value_groups` groups of 16 tokens).
-  __shared__ T tile[16][D + 8];
+  __shared__ __attribute__((aligned(16))) T tile[16][D + 8];
   __shared__ int together;
   if ((int)blockIdx.x >= tokens) {
     const int v = blockIdx.x - tokens;
