@@ -9,13 +9,9 @@ typedef uint16_t bf16_t;   // bfloat16 kept as its bit pattern; all arithmetic i
 
 __device__ __forceinline__ float bf16_to_float(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
-// Round to nearest, ties to even (what torch's .bfloat16() does); NaN stays NaN.
-__device__ __forceinline__ bf16_t float_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
-}
+// Round to nearest, ties to even (what torch's .bfloat16() does); NaN stays NaN. The hardware's conversion
+// (v_cvt_pk_bf16_f32): one instruction where the same in integer arithmetic takes seven.
+__device__ __forceinline__ bf16_t float_to_bf16(float f) { return __builtin_bit_cast(bf16_t, (__bf16)f); }
 
 template <typename T> struct Elem;
 template <> struct Elem<float> {
