@@ -512,6 +512,33 @@ __device__ __forceinline__ void v_write_group(T (*tile)[PITCH], int* together, i
   }
 }
 
+// Among the LPH lanes of a head: the sum over them, and the value LPH / 2 lanes away. With 16 lanes a head (a DPP row)
+// both are register moves (rotations of the row, swaps inside a quad) that hand every lane the very values the
+// shuffles by xor 8, 4, 2, 1 would: after the step by 8, lanes l and l ^ 8 hold the same, so the lane 4 before holds
+// what lane l ^ 4 does. Other head sizes go through the shuffles.
+template <int CTRL>
+__device__ __forceinline__ float row_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int LPH>
+__device__ __forceinline__ float head_sum(float ss) {
+  if constexpr (LPH == 16) {
+    ss += row_move<0x128>(ss);     // row_ror:8
+    ss += row_move<0x124>(ss);     // row_ror:4
+    ss += row_move<0x4e>(ss);      // quad_perm:[2,3,0,1]
+    ss += row_move<0xb1>(ss);      // quad_perm:[1,0,3,2]
+  } else {
+#pragma unroll
+    for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
+  }
+  return ss;
+}
+template <int LPH>
+__device__ __forceinline__ float half_away(float v) {
+  if constexpr (LPH == 16) return row_move<0x128>(v);
+  else return __shfl_xor(v, LPH / 2, WAVE);
+}
+
 // The same for head_dim 64, 128 or 256 with the whole head rotated (or not at all): each lane holds 8 consecutive
 // values (one 16-byte load), LPH = head_dim / 8 lanes make a head, a wave holds 64 / LPH heads. The rotation partner
 // of a value sits LPH / 2 lanes away; norm sums run over the LPH lanes of a head. No LDS.
@@ -586,8 +613,7 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
       float ss = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
-#pragma unroll
-      for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
+      ss = head_sum<LPH>(ss);
       const float inv = 1.0f / sqrtf(ss / (float)D + eps);
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = Elem<T>::round((v[j] * inv) * Elem<T>::load(w[j]));
@@ -595,7 +621,7 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
     if (table != nullptr) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float other = __shfl_xor(v[j], LPH / 2, WAVE);
+        const float other = half_away<LPH>(v[j]);
         v[j] = li < LPH / 2 ? v[j] * co[j] - other * si[j] : v[j] * co[j] + other * si[j];
       }
     }
