@@ -59,6 +59,16 @@ __device__ __forceinline__ void load_to_lds16(const void* base, uint32_t lane_by
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                : : "v"(lane_bytes), "s"(base), "s"(lds_wave_base) : "memory", "m0");
 }
+// A 16-byte load into registers that the compiler does not track either, for kernels whose other loads are the copies
+// above: the compiler counts only the loads it knows, so where both kinds are under way the waits it inserts before a
+// known load's first use come out wrong for the mix (far too early a wait, measured). The caller waits
+// (`wait_loads_but`) before the first use, and keeps the result where it is until then (no copy of it may be made
+// before the wait: the register still holds what it held before). OFFSET: a constant added to the address, 0 to 4095.
+template <typename V, int OFFSET>
+__device__ __forceinline__ void load16_untracked(V& to, const void* base, uint32_t lane_bytes) {
+  static_assert(sizeof(V) == 16 && OFFSET >= 0 && OFFSET < 4096, "one 16-byte vector, an offset the instruction holds");
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=&v"(to) : "v"(lane_bytes), "s"(base), "n"(OFFSET) : "memory");
+}
 #pragma clang diagnostic pop
 template <int N>
 __device__ __forceinline__ void wait_loads_but() {          // until at most N of this wave's loads are under way

@@ -132,6 +132,13 @@ int holon_gemm_rows_splits(int M, int N, int K);
 int holon_gemm_rows_parts_supported(int M, int N, int K, int splits);
 int holon_gemm_rows_parts_bf16(const void* x, const void* w_tiled, void* parts, int M, int N, int K, int splits,
                                void* stream);
+// The same for 129 to 1,024 rows over a weight whose K is at least twice its N (a feed-forward's second product):
+// blocks of 128 rows against 256 columns. holon_gemm_tiles_splits: the shares to take, 0 where the shape is not served
+// or not this kernel's to take.
+int holon_gemm_tiles_splits(int M, int N, int K);
+int holon_gemm_tiles_parts_supported(int M, int N, int K, int splits);
+int holon_gemm_tiles_parts_bf16(const void* x, const void* w_tiled, void* parts, int M, int N, int K, int splits,
+                                void* stream);
 int holon_sum_parts(const void* parts, void* y, int splits, int64_t count, void* stream);
 // y[M, N] = x[M, K] w[N, K]^T, all float32, true 32-bit products and sums in an order that depends on K alone: a row's
 // result is bit for bit the same whatever other rows are in the call.

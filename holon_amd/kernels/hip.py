@@ -85,6 +85,9 @@ class HipKernels:
             "holon_gemm_rows_splits": [_I, _I, _I],
             "holon_gemm_rows_parts_supported": [_I, _I, _I, _I],
             "holon_gemm_rows_parts_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
+            "holon_gemm_tiles_splits": [_I, _I, _I],
+            "holon_gemm_tiles_parts_supported": [_I, _I, _I, _I],
+            "holon_gemm_tiles_parts_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
             "holon_sum_parts": [_P, _P, _I, _L, _P],
             "holon_rmsnorm_parts": [_P, _I, _P, _P, _P, _L, _I, _F, _P],
             "holon_gemm_skinny_scaled_bf16": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _F, _P],
@@ -449,17 +452,19 @@ class HipKernels:
                        self._stream())
         return y
 
-    parts_rows = 128          # the product in shares of K serves steps of 17 to this many rows
+    parts_rows = 1024         # the products in shares of K serve steps of 17 to this many rows
+    parts_rows_short = 128    # of which the kernel for weights of any K serves up to this many
 
     def linear_parts(self, x, weight, tiled):
-        """-> float32 [splits, M, N], the product over each share of K, when that kernel serves this step (17 to 128
-        bfloat16 rows over a narrow tiled weight) and, timed once per weight shape and row bucket against the vendor
-        library's product (each with the add + norm that reads it), is the faster; None otherwise (nothing was done)."""
+        """-> float32 [splits, M, N], the product over each share of K, when a kernel of that kind serves this step
+        (17 to 128 bfloat16 rows over a narrow tiled weight; 129 to 1,024 rows where K is at least twice N) and,
+        timed once per weight shape and row bucket against the vendor library's product (each with the add + norm
+        that reads it), is the faster; None otherwise (nothing was done)."""
         (m, k), n = x.shape, weight.shape[0]
         if not (tiled is not None and 16 < m <= self.parts_rows and x.dtype == torch.bfloat16
                 and weight.dtype == torch.bfloat16 and weight.shape[1] == k and x.is_contiguous()):
             return None
-        splits = self.lib.holon_gemm_rows_splits(m, n, k)
+        splits = (self.lib.holon_gemm_rows_splits if m <= self.parts_rows_short else self.lib.holon_gemm_tiles_splits)(m, n, k)
         if not splits:
             return None
         use = self.product_choice("parts", weight, m, lambda: self._time_parts(x, weight, tiled, splits))
@@ -472,8 +477,8 @@ class HipKernels:
             raise KernelError(f"linear in parts: bfloat16 rows {tuple(x.shape)} over a tiled bfloat16 weight "
                               f"{tuple(weight.shape)} expected")
         parts = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
-        self._call(self.lib.holon_gemm_rows_parts_bf16, x.data_ptr(), tiled.data_ptr(), parts.data_ptr(), m, n, k,
-                   splits, self._stream())
+        entry = self.lib.holon_gemm_rows_parts_bf16 if m <= self.parts_rows_short else self.lib.holon_gemm_tiles_parts_bf16
+        self._call(entry, x.data_ptr(), tiled.data_ptr(), parts.data_ptr(), m, n, k, splits, self._stream())
         return parts
 
     def _time_parts(self, x, weight, tiled, splits) -> str:

@@ -543,7 +543,7 @@ def test_product_in_shares_of_k_for_narrow_weights(hip):
     assert hip.configured("vendor", {"parts:4096x4096:32": "parts"}).linear_parts(x, w, tiled).shape == (8, 32, 4096)
     assert hip.linear_parts(x, w, tiled).shape == (8, 32, 4096)
     assert hip.linear_parts(x[:16].contiguous(), w, tiled) is None and hip.linear_parts(x, w, None) is None
-    assert hip.linear_parts(_randn(129, 4096, dtype=bf, seed=99), w, tiled) is None            # beyond 128 rows
+    assert hip.linear_parts(_randn(129, 4096, dtype=bf, seed=99), w, tiled) is None            # beyond 128 rows, K < 2 N
     assert hip.linear_parts(_randn(32, 4096, dtype=torch.float32, seed=96), w.float(), tiled) is None          # float32 rows: not this path
     w = _randn(4096, 4224, dtype=bf, seed=97)                                             # K = 33 x 128: no equal shares
     assert hip.linear_parts(_randn(32, 4224, dtype=bf, seed=98), w, hip.tile_weight(w)) is None
@@ -918,6 +918,56 @@ def test_sampling_under_random_settings(hip):
             assert law[got[r]] > 0, case
             order = S.drawing_order(logits[r], temp[r], top_k[r], top_p[r], min_p[r])
             assert _at_uniform(law, order, got[r], S.uniform(11, r)), case
+
+
+def test_product_in_shares_of_k_for_prompt_portions(hip):
+    """129 to 1,024 rows over a weight whose K is at least twice its N (a feed-forward's second product): blocks of
+    128 rows against 256 columns, K in shares. Every share against float64 over its columns, for every number of
+    shares the kernel takes; the sum against the whole product and the vendor library's; rows whatever rows lie beside
+    them (another number of row blocks); the norm that reads the parts; what the kernel does not take."""
+    from holon_amd.kernels.hip import KernelError
+    bf = torch.bfloat16
+    for m, k, n in ((129, 512, 256), (200, 1024, 512), (512, 12288, 4096), (1000, 2048, 512), (1024, 1536, 768),
+                    (300, 25600, 5120), (640, 9728, 2560)):
+        x, w = _randn(m, k, dtype=bf, seed=190), _randn(n, k, dtype=bf, seed=191, scale=0.05)
+        tiled = hip.tile_weight(w)
+        auto = hip.lib.holon_gemm_tiles_splits(m, n, k)
+        assert auto in (0, 1, 2, 4, 8) and (auto > 0 or n <= 512), (m, k, n, auto)    # (0: too few blocks to be worth taking)
+        whole = x.double() @ w.double().T
+        for splits in (1, 2, 4, 8):
+            if not hip.lib.holon_gemm_tiles_parts_supported(m, n, k, splits):
+                assert splits != auto
+                continue
+            parts = hip._rows_parts(x, w, tiled, splits)
+            assert parts.shape == (splits, m, n) and parts.dtype == torch.float32
+            share = k // splits
+            for s in range(splits):
+                want = x[:, s * share:(s + 1) * share].double() @ w[:, s * share:(s + 1) * share].double().T
+                assert H.op_budget_usage(parts[s], want, torch.float32, share) <= 1, (m, k, n, splits, s)
+            total = hip.sum_parts(parts)
+            assert H.op_budget_usage(total, whole, bf, k) <= 1
+            if splits == (auto or 2):
+                assert H.op_budget_usage(total, hip.linear(x, w).double(), bf, k) <= 1       # the vendor library's product
+                some = hip._rows_parts(x[5:200].contiguous(), w, tiled, splits) if m >= 200 else None
+                assert some is None or torch.equal(some, parts[:, 5:200])
+                weight, eps = _randn(n, dtype=bf, seed=192) + 1, 1e-5
+                res_a, res_b = _randn(m, n, dtype=bf, seed=193), _randn(m, n, dtype=bf, seed=193)
+                normed_a = hip.add_rmsnorm(parts, res_a, weight, eps)
+                normed_b = hip.add_rmsnorm(total, res_b, weight, eps)
+                assert torch.equal(res_a, res_b), (m, k, n)
+                assert H.op_budget_usage(normed_a, normed_b.double(), bf, 1) <= 1, (m, k, n)
+    x, w = _randn(512, 12288, dtype=bf, seed=194), _randn(4096, 12288, dtype=bf, seed=195, scale=0.05)
+    tiled = hip.tile_weight(w)
+    assert hip.linear_parts(x, w, tiled).shape == (8, 512, 4096)                            # mode `own`
+    assert hip.configured("vendor").linear_parts(x, w, tiled) is None
+    assert hip.configured("vendor", {"parts:4096x12288:512": "parts"}).linear_parts(x, w, tiled).shape == (8, 512, 4096)
+    assert hip.linear_parts(_randn(1025, 12288, dtype=bf, seed=196), w, tiled) is None     # beyond 1,024 rows
+    wide = _randn(8192, 4096, dtype=bf, seed=197)
+    assert hip.linear_parts(_randn(512, 4096, dtype=bf, seed=198), wide, hip.tile_weight(wide)) is None   # K < 2 N
+    with pytest.raises(KernelError):
+        hip._rows_parts(x, w, tiled, 5)
+    with pytest.raises(KernelError):
+        hip._rows_parts(x, w[:4000].contiguous(), hip.tile_weight(w[:4000].contiguous()), 4)   # 4,000 columns: no whole blocks
 
 
 def test_kernels_refuse_what_they_do_not_serve(hip):
