@@ -40,9 +40,12 @@ def key_of(kind: str, shape: tuple[int, int], bucket: int) -> str:
 
 
 def row_bucket(rows: int) -> int:
-    """The row bucket a step of `rows` rows falls in: up to 32, up to 64, then powers of two."""
+    """The row bucket a step of `rows` rows falls in: up to 32, up to 64, then powers of two, and 768 between 512 and
+    1,024 (a portion of 512 tokens beside decode rows is served as it would be alone, not as 1,024 rows are)."""
     if rows <= 32:
         return 32
+    if 512 < rows <= 768:
+        return 768
     return 1 << (rows - 1).bit_length()
 
 

@@ -110,7 +110,7 @@ def assemble(cfg: EngineConfig, kernels=None, *, random_config: dict | None = No
     return out
 
 
-TIMED_ROWS = (32, 64, 128, 256, 512, 1024)       # one step in each row bucket a product choice is kept for
+TIMED_ROWS = (32, 64, 128, 256, 512, 768, 1024)       # one step in each row bucket a product choice is kept for
 
 
 def time_products(a: Assembled, cfg: EngineConfig) -> None:

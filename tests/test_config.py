@@ -138,7 +138,8 @@ def test_product_choices_resolve_pinned_then_by_mode_then_timed_at_start_only():
 
     from holon_amd import cli
     from holon_amd.config.products import ProductError, ProductPlan, key_of, row_bucket
-    assert [row_bucket(r) for r in (17, 32, 33, 64, 65, 128, 129, 1000)] == [32, 32, 64, 64, 128, 128, 256, 1024]
+    assert [row_bucket(r) for r in (17, 32, 33, 64, 65, 128, 129, 512, 513, 768, 769, 1000)] == \
+        [32, 32, 64, 64, 128, 128, 256, 512, 768, 768, 1024, 1024]
     assert key_of("parts", (4096, 12288), 64) == "parts:4096x12288:64"
     calls = []
 
