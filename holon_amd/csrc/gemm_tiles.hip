@@ -163,13 +163,16 @@ extern "C" int holon_gemm_tiles_parts_supported(int M, int N, int K, int splits)
 }
 
 // How many shares of K to take, 0 where the kernel does not serve the shape or is not the one to take: it is for
-// weights whose K is at least twice their N (few output tiles, long sums), with as few shares (a power of two, at most
+// weights whose K is well above their N (few output tiles, long sums), with as few shares (a power of two, at most
 // eight) as give 384 blocks. Measured on MI355X with the add + norm that reads the parts, against the vendor library's
 // product with its add + norm, us: 4096 x 12288 at 256 / 512 / 768 / 1,024 rows 46 / 73 / 103 / 114 against 61 / 93 /
 // 111 / 135; 5120 x 25600: 120 / 171 / 210 / 291 against 268 / 278 / 303 / 362; 2560 x 9728: 37 / 57 / 63 / 87 against
-// 43 / 57 / 71 / 90. Blocks of eight waves (the rows read half as often) were no faster.
+// 43 / 57 / 71 / 90. With K between 1.5 and 2 times N it still wins up to 768 rows (5120 x 8192: 54 / 76 / 87 against
+// 78 / 81 / 90; at 1,024 rows 119 against 111); with K = N it loses everywhere (4096 x 4096: 26 / 36 / 52 / 58 against
+// 24 / 33 / 37 / 47). Blocks of eight waves (the rows read half as often) were no faster.
 extern "C" int holon_gemm_tiles_splits(int M, int N, int K) {
-  if (M <= 128 || M > 1024 || N <= 0 || K < 2 * N || N % (16 * TILES_WAVES * TILES_NT)) return 0;
+  if (M <= 128 || M > 1024 || N <= 0 || N % (16 * TILES_WAVES * TILES_NT)) return 0;
+  if (!(K >= 2 * N || (2 * (int64_t)K >= 3 * (int64_t)N && M <= 768))) return 0;
   const int blocks = N / (16 * TILES_WAVES * TILES_NT) * ((M + 127) / 128);
   int splits = 1;
   while (splits < TILES_MAX_SPLITS && blocks * splits < 384) splits *= 2;

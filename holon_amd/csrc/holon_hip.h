@@ -132,7 +132,8 @@ int holon_gemm_rows_splits(int M, int N, int K);
 int holon_gemm_rows_parts_supported(int M, int N, int K, int splits);
 int holon_gemm_rows_parts_bf16(const void* x, const void* w_tiled, void* parts, int M, int N, int K, int splits,
                                void* stream);
-// The same for 129 to 1,024 rows over a weight whose K is at least twice its N (a feed-forward's second product):
+// The same for 129 to 1,024 rows over a weight whose K is at least twice its N (a feed-forward's second product;
+// up to 768 rows: one and a half times):
 // blocks of 128 rows against 256 columns. holon_gemm_tiles_splits: the shares to take, 0 where the shape is not served
 // or not this kernel's to take.
 int holon_gemm_tiles_splits(int M, int N, int K);

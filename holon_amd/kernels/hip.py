@@ -457,7 +457,7 @@ class HipKernels:
 
     def linear_parts(self, x, weight, tiled):
         """-> float32 [splits, M, N], the product over each share of K, when a kernel of that kind serves this step
-        (17 to 128 bfloat16 rows over a narrow tiled weight; 129 to 1,024 rows where K is at least twice N) and,
+        (17 to 128 bfloat16 rows over a narrow tiled weight; 129 to 1,024 rows where K is well above N) and,
         timed once per weight shape and row bucket against the vendor library's product (each with the add + norm
         that reads it), is the faster; None otherwise (nothing was done)."""
         (m, k), n = x.shape, weight.shape[0]
