@@ -73,7 +73,7 @@ __global__ void argmax_kernel(const float* __restrict__ logits, int32_t* __restr
 
 // A wide row in two kernels: block (piece, row) finds the best of its ARGMAX_PIECE values, then one wave a row the best
 // of the pieces (ties go to the smaller index in both, so the answer is the one block's). One block walking 151,936
-// values alone takes 17.5 us; the two kernels together 7.
+// values alone takes 17.5 us; the two kernels together 9.4.
 constexpr int ARGMAX_PIECE = 4096;
 constexpr int ARGMAX_MAX_PIECES = 1024;
 __global__ void __launch_bounds__(SAMPLE_THREADS) argmax_pieces_kernel(const float* __restrict__ logits,
