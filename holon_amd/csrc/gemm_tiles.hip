@@ -159,7 +159,8 @@ constexpr int TILES_MAX_SPLITS = 8;
 // Whether holon_gemm_tiles_parts_bf16 serves this product with K cut into `splits` shares.
 extern "C" int holon_gemm_tiles_parts_supported(int M, int N, int K, int splits) {
   return M > 128 && M <= 1024 && N % (16 * TILES_WAVES * TILES_NT) == 0 && splits >= 1 && splits <= TILES_MAX_SPLITS &&
-         K > 0 && K % (TILES_KC * splits) == 0 && K % 32 == 0;
+         K > 0 && K % (TILES_KC * splits) == 0 && K % 32 == 0 &&
+         (int64_t)M * K * 2 < (int64_t)1 << 32;             // (a lane's place among the rows is a 32-bit byte offset)
 }
 
 // How many shares of K to take, 0 where the kernel does not serve the shape or is not the one to take: it is for
