@@ -135,6 +135,11 @@ def test_every_way_of_cutting_at_the_measured_shapes(shape, dtype):
     rep = Replayer(loaded)
     got = H.run_trace(rep, H.trace_whole(requests))
     _check(shape, dtype, requests, got, "whole")
+    if dtype == "bfloat16":        # the prompts of 300 and 130 tokens took this package's product for the down projection
+        taken, cfg = loaded.kernels.plan.report(), SHAPES[shape]
+        for bucket in (256, 512):
+            key = f"parts:{cfg['hidden_size']}x{cfg['intermediate_size']}:{bucket}"
+            assert taken.get(key) == "parts", (key, taken)
     got = H.run_trace(rep, H.trace_decode_tail("r0", requests["r0"], 32))          # the tail replays from graphs
     _check(shape, dtype, requests, got, "decode tail")
     assert loaded.runner.graph_replays >= 30
