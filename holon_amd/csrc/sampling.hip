@@ -196,9 +196,10 @@ __device__ int block_sum_int(int v) {
   return result;
 }
 
-// Order-preserving map of a float onto unsigned integers (larger float, larger key).
+// Order-preserving map of a float onto unsigned integers (larger float, larger key; equal floats, equal keys: -0 is
+// made +0 first, the two being the same value with different bits).
 __device__ __forceinline__ uint32_t float_key(float f) {
-  const uint32_t u = __float_as_uint(f);
+  const uint32_t u = __float_as_uint(f + 0.0f);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 __device__ __forceinline__ float key_float(uint32_t k) {

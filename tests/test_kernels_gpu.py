@@ -855,6 +855,8 @@ def test_sampling_filters_at_the_full_vocabulary(hip):
     tied[order[2:5]] = peaked[order[3]]
     plateau = peaked.clone()
     plateau[order[:6000]] = peaked[order[0]]
+    coarse = (torch.randn(v, generator=g) * 0.4).round() / 4     # five values, tens of thousands of each; +0 and -0 are one
+    assert (coarse == 0).sum() > 50_000 and ((coarse == 0) & coarse.signbit()).sum() > 10_000
     cases = [(peaked, 0.8, 50, 1.0, 0.0), (peaked, 0.8, 0, 0.9, 0.0), (peaked, 1.0, 50, 0.9, 0.02), (peaked, 0.7, 0, 1.0, 0.05),
              (peaked, 1.0, 1, 1.0, 0.0), (peaked, 1.0, 0, 1e-6, 0.0), (peaked, 1.2, 2048, 0.99, 0.0), (peaked, 1.0, 5000, 1.0, 0.0),
              (flat, 1.0, 0, 0.9, 0.0), (flat, 1.0, 300, 0.5, 0.0), (tied, 1.0, 50, 1.0, 0.0), (tied, 1.0, 48, 0.95, 0.0),
@@ -864,7 +866,8 @@ def test_sampling_filters_at_the_full_vocabulary(hip):
              (flat, 1.0, 0, 1.0, 0.2), (peaked, 1.0, 200_000, 1.0, 0.0),   # kept sets too long to collect: min-p alone, all
              (plateau, 1.0, 0, 0.5, 0.0), (plateau, 1.0, 0, 1.0, 0.5), (plateau, 1.0, 7000, 1.0, 0.0),   # 6,000 equal values
              (flat, 0.8, 50, 0.9, 0.0), (flat, 0.8, 20, 0.95, 0.05), (peaked, 1.0, 5000, 0.9, 0.01),    # cuts found by halving
-             (plateau, 1.0, 3000, 1.0, 0.0), (peaked * 40, 1.0, 5000, 1.0, 0.0)]   # a cut inside equal values; k beyond what weighs
+             (plateau, 1.0, 3000, 1.0, 0.0), (peaked * 40, 1.0, 5000, 1.0, 0.0),   # a cut inside equal values; k beyond what weighs
+             (coarse, 0.3, 0, 0.9, 0.0), (coarse, 1.0, 0, 0.5, 0.0), (coarse, 1.0, 70_000, 1.0, 0.0), (coarse, 0.3, 0, 1.0, 0.15)]
     n = 48
     for at, (row, temp, top_k, top_p, min_p) in enumerate(cases):
         f = lambda x, dt: torch.full((n,), x, dtype=dt).cuda()
@@ -878,7 +881,7 @@ def test_sampling_filters_at_the_full_vocabulary(hip):
         assert all(law[t] > 0 for t in tokens), (at, "a filtered token was drawn")
         for pos, t in enumerate(tokens):                   # the inverse CDF at the hashed uniform, to float32 rounding
             assert _at_uniform(law, order, t, S.uniform(seed, pos)), (at, pos, t)
-        if row is not flat and top_k < v:   # few tokens carry the mass: a draw then sits well inside its token's share
+        if row is not flat and row is not coarse and top_k < v:   # few tokens carry the mass: a draw then sits well inside its token's share
             want = [S.draw(law, S.uniform(seed, pos), order) for pos in range(n)]
             assert sum(a != b for a, b in zip(tokens, want)) <= 1, (at, temp, top_k, top_p, min_p)
     # rows of one batch with different settings do not disturb each other
