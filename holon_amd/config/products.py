@@ -25,7 +25,7 @@ MODES = ("own", "vendor", "timed")
 KINDS: dict[str, tuple[str, tuple[str, ...]]] = {
     "rows": ("rows", ("rows", "vendor")),         # 17 to 64 rows over many tiles, rows shared through LDS
     "glu": ("rows", ("rows", "vendor")),          # the same with SiLU-mul inside
-    "parts": ("parts", ("parts", "vendor")),      # 17 to 128 rows over a narrow weight, K in shares
+    "parts": ("parts", ("parts", "vendor")),      # a narrow weight, K in shares: 17 to 128 rows; to 1,024 where K is well above N
     "vendor": ("bf16", ("bf16", "f32", "f32x2")),  # the vendor product's own forms (result type, K in halves)
 }
 

@@ -61,7 +61,8 @@ class Linear(Part):
         """x W^T. With `residual`, the product is added into the stream's rows in place when one kernel can do both
         (steps of few rows), which also leaves the rows' statistics there, and None is returned; otherwise the
         product is returned and the add is the caller's. It may then come as `PartialSums` (a narrow weight at 17 to
-        128 rows, K split over blocks), which the norm that adds it reads as they are."""
+        128 rows, or up to 1,024 where its K is well above its N: K split over blocks), which the norm that adds it
+        reads as they are."""
         if isinstance(x, Normed):
             if self.folds(x):
                 return self.kernels.linear(x.h, self.weight, out_dtype, self.tiled, row_scale=self.row_scale(x))
